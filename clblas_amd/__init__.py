@@ -1,0 +1,161 @@
+"""clblas_amd -- Python access to libclblas_amd.so, the MI355X (gfx950) xGEMM / xTRSM core
+behind clBLAS's call surface.
+
+The product is the shared library (C ABI declared in include/clblas_amd.h).  This module
+only loads it with ctypes and mirrors the four entry points with the reference's argument
+order (src/clBLAS.h:7382-7405, 7463-7486, 7988-8008, 8063-8083); matrices are passed as
+torch CUDA tensors (used purely as device allocations) or as integer device addresses.
+
+There is no CPU fallback: if the library has not been built, loading raises.
+"""
+import ctypes
+import enum
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libclblas_amd.so")
+
+
+class Order(enum.IntEnum):
+    RowMajor = 0
+    ColumnMajor = 1
+
+
+class Transpose(enum.IntEnum):
+    NoTrans = 0
+    Trans = 1
+    ConjTrans = 2
+
+
+class Uplo(enum.IntEnum):
+    Upper = 0
+    Lower = 1
+
+
+class Diag(enum.IntEnum):
+    Unit = 0
+    NonUnit = 1
+
+
+class Side(enum.IntEnum):
+    Left = 0
+    Right = 1
+
+
+class Status(enum.IntEnum):
+    Success = 0
+    InvalidValue = -30
+    InvalidDevice = -33
+    OutOfResources = -5
+    OutOfHostMemory = -6
+    NotImplemented = -1024
+    NotInitialized = -1023
+    InvalidMatA = -1022
+    InvalidMatB = -1021
+    InvalidMatC = -1020
+    InvalidDim = -1017
+    InvalidLeadDimA = -1016
+    InvalidLeadDimB = -1015
+    InvalidLeadDimC = -1014
+    InsufficientMemMatA = -1011
+    InsufficientMemMatB = -1010
+    InsufficientMemMatC = -1009
+
+
+EXPORTED_SYMBOLS = (
+    "clblasGetVersion",
+    "clblasSetup",
+    "clblasTeardown",
+    "clblasSgemm",
+    "clblasDgemm",
+    "clblasStrsm",
+    "clblasDtrsm",
+)
+
+_lib = None
+
+
+def _declare(lib):
+    sz, vp, i = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int
+    for name, real in (("clblasSgemm", ctypes.c_float), ("clblasDgemm", ctypes.c_double)):
+        fn = getattr(lib, name)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, sz, real, vp, sz, sz, vp, sz, sz, real, vp, sz, sz, vp]
+    for name, real in (("clblasStrsm", ctypes.c_float), ("clblasDtrsm", ctypes.c_double)):
+        fn = getattr(lib, name)
+        fn.restype = i
+        fn.argtypes = [i, i, i, i, i, sz, sz, real, vp, sz, sz, vp, sz, sz, vp]
+    lib.clblasSetup.restype = i
+    lib.clblasSetup.argtypes = []
+    lib.clblasTeardown.restype = None
+    lib.clblasTeardown.argtypes = []
+    lib.clblasGetVersion.restype = i
+    lib.clblasGetVersion.argtypes = [ctypes.POINTER(ctypes.c_uint)] * 3
+
+
+def load_library(path=None):
+    """Loads libclblas_amd.so (once) and returns the ctypes handle. Raises if it is missing."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    p = path or LIB_PATH
+    if not os.path.exists(p):
+        raise RuntimeError(
+            "%s not found: build it with `python -m clblas_amd.build` (there is no fallback path)" % p)
+    lib = ctypes.CDLL(p)
+    _declare(lib)
+    if path is None:
+        _lib = lib
+    return lib
+
+
+def _ptr(x):
+    """Device address of a torch tensor, or the integer itself."""
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return ctypes.c_void_p(x)
+    return ctypes.c_void_p(x.data_ptr())
+
+
+def _stream(stream):
+    if stream is None:
+        import torch
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    if isinstance(stream, int):
+        return ctypes.c_void_p(stream)
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def setup():
+    return load_library().clblasSetup()
+
+
+def teardown():
+    load_library().clblasTeardown()
+
+
+def get_version():
+    a, b, c = ctypes.c_uint(), ctypes.c_uint(), ctypes.c_uint()
+    load_library().clblasGetVersion(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))
+    return a.value, b.value, c.value
+
+
+def sgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    return load_library().clblasSgemm(int(order), int(transA), int(transB), M, N, K, alpha, _ptr(A), offA, lda,
+                                      _ptr(B), offB, ldb, beta, _ptr(C), offC, ldc, _stream(stream))
+
+
+def dgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    return load_library().clblasDgemm(int(order), int(transA), int(transB), M, N, K, alpha, _ptr(A), offA, lda,
+                                      _ptr(B), offB, ldb, beta, _ptr(C), offC, ldc, _stream(stream))
+
+
+def strsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):
+    return load_library().clblasStrsm(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha,
+                                      _ptr(A), offA, lda, _ptr(B), offB, ldb, _stream(stream))
+
+
+def dtrsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):
+    return load_library().clblasDtrsm(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha,
+                                      _ptr(A), offA, lda, _ptr(B), offB, ldb, _stream(stream))

@@ -1,0 +1,57 @@
+"""Builds libclblas_amd.so (HIP kernels + C ABI) for gfx950, in-tree.
+
+Usage:  python -m clblas_amd.build        (or  clblas_amd.build.build_library())
+hipcc cross-compiles without a GPU present.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ_DIR = os.path.join(HERE, "build")
+LIB_PATH = os.path.join(HERE, "libclblas_amd.so")
+
+SOURCES = ["api.cpp", "gemm_f32.hip", "gemm_f64.hip", "trsm.hip"]
+
+# -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+COMMON_FLAGS = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option"]
+
+
+def _hipcc():
+    return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+
+def _compile(src):
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    cmd = [_hipcc()] + COMMON_FLAGS
+    if src.endswith(".hip"):
+        cmd += DEVICE_FLAGS
+    cmd += ["-c", os.path.join(CSRC, src), "-o", obj]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # The host pass warns that it does not know the packed-fp32 feature; that is harmless.
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError("compile failed: %s\n%s" % (" ".join(cmd), err))
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build_library(verbose=True):
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    with ThreadPoolExecutor(max_workers=4) as ex:
+        objs = list(ex.map(_compile, SOURCES))
+    cmd = [_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950"] + objs + ["-o", LIB_PATH]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("link failed: %s\n%s" % (" ".join(cmd), res.stderr))
+    if verbose:
+        print("built", LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build_library()

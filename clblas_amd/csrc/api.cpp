@@ -1,0 +1,257 @@
+// C ABI of libclblas_amd.so: argument validation, row-major folding and dispatch.
+//
+// This is the host front end that stands where the reference has
+//   src/library/blas/xgemm.cc:667-783  (clblasSgemm / clblasDgemm),
+//   src/library/blas/xgemm.cc:341-383  (clblasGemm<T>: ConjTrans and row-major folding),
+//   src/library/blas/xtrsm.cc:1600-1785 (clblasStrsm / clblasDtrsm),
+//   src/library/blas/functor/functor_xtrsm.cc:57-75 (doTrsm validation),
+//   src/library/blas/generic/common.c:585-688 (checkMatrixSizes),
+//   src/library/blas/init.c:33-263 (GetVersion / Setup / Teardown).
+#include "../../include/clblas_amd.h"
+#include "internal.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdlib>
+#include <map>
+#include <mutex>
+#include <utility>
+#include <vector>
+
+namespace cba {
+
+int forced_gemm_tile() {
+    const char *s = std::getenv("CLBLAS_AMD_GEMM_TILE");
+    if (!s || !*s) return -1;
+    return std::atoi(s);
+}
+
+int forced_trsm_nb() {
+    const char *s = std::getenv("CLBLAS_AMD_TRSM_NB");
+    if (!s || !*s) return 0;
+    return std::atoi(s);
+}
+
+namespace {
+struct WsSlot {
+    void *ptr = nullptr;
+    size_t bytes = 0;
+};
+std::mutex g_ws_mutex;
+std::map<std::pair<int, hipStream_t>, WsSlot> g_ws;  // (device, stream) -> current buffer
+std::vector<std::pair<int, void *>> g_ws_retired;    // outgrown buffers, freed at teardown
+std::mutex g_lds_mutex;
+std::map<std::pair<int, const void *>, size_t> g_lds_limit;
+}  // namespace
+
+void *workspace_get(hipStream_t stream, size_t bytes) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    WsSlot &slot = g_ws[std::make_pair(dev, stream)];
+    if (slot.bytes >= bytes && slot.ptr) return slot.ptr;
+    size_t want = bytes < (size_t)(1 << 20) ? (size_t)(1 << 20) : bytes;
+    void *p = nullptr;
+    if (hipMalloc(&p, want) != hipSuccess) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    if (slot.ptr) g_ws_retired.push_back(std::make_pair(dev, slot.ptr));
+    slot.ptr = p;
+    slot.bytes = want;
+    return p;
+}
+
+void workspace_release_all() {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    int cur = 0;
+    (void)hipGetDevice(&cur);
+    for (auto &kv : g_ws) {
+        if (kv.second.ptr) {
+            (void)hipSetDevice(kv.first.first);
+            (void)hipFree(kv.second.ptr);
+        }
+    }
+    for (auto &r : g_ws_retired) {
+        (void)hipSetDevice(r.first);
+        (void)hipFree(r.second);
+    }
+    g_ws.clear();
+    g_ws_retired.clear();
+    (void)hipSetDevice(cur);
+}
+
+hipError_t ensure_dynamic_lds(const void *fn, size_t bytes) {
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    std::lock_guard<std::mutex> lock(g_lds_mutex);
+    size_t &cur = g_lds_limit[std::make_pair(dev, fn)];
+    if (cur >= bytes) return hipSuccess;
+    err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (err == hipSuccess) cur = bytes;
+    return err;
+}
+
+}  // namespace cba
+
+namespace {
+
+enum MatId { MAT_A = 0, MAT_B = 1, MAT_C = 2 };
+
+clblasStatus lead_dim_error(MatId m) {
+    return m == MAT_A ? clblasInvalidLeadDimA : (m == MAT_B ? clblasInvalidLeadDimB : clblasInvalidLeadDimC);
+}
+
+// Restates checkMatrixSizes (generic/common.c:585-688) for a rows x cols logical matrix:
+// zero dimension -> InvalidDim; ld below the number of elements that are contiguous in
+// memory -> InvalidLeadDim{A,B,C}.  The reference's third outcome, InsufficientMemMat*,
+// compares against CL_MEM_SIZE of the cl_mem; a raw device pointer carries no size, so
+// that code cannot arise here.
+clblasStatus check_matrix_sizes(clblasOrder order, clblasTranspose trans, size_t rows, size_t cols, size_t ld,
+                                MatId which) {
+    if (rows == 0 || cols == 0) return clblasInvalidDim;
+    const bool rows_contiguous = (order == clblasRowMajor && trans != clblasNoTrans) ||
+                                 (order == clblasColumnMajor && trans == clblasNoTrans);
+    if (rows_contiguous ? (ld < rows) : (ld < cols)) return lead_dim_error(which);
+    return clblasSuccess;
+}
+
+bool valid_order(clblasOrder o) { return o == clblasRowMajor || o == clblasColumnMajor; }
+bool valid_trans(clblasTranspose t) { return t == clblasNoTrans || t == clblasTrans || t == clblasConjTrans; }
+
+clblasStatus map_hip_error(hipError_t e) {
+    if (e == hipSuccess) return clblasSuccess;
+    (void)hipGetLastError();
+    if (e == hipErrorOutOfMemory) return clblasOutOfResources;
+    if (e == hipErrorInvalidValue) return clblasInvalidValue;
+    return clblasOutOfResources;
+}
+
+const size_t kMaxDim = 0x7fffffff;  // kernels index tiles with 32-bit ints (reference: cl_uint, xgemm.cc:362-372)
+
+template <typename T, typename Fn>
+clblasStatus gemm_front(Fn launch, clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M,
+                        size_t N, size_t K, T alpha, const T *A, size_t offA, size_t lda, const T *B, size_t offB,
+                        size_t ldb, T beta, T *C, size_t offC, size_t ldc, hipStream_t stream) {
+    // Order of checks follows xgemm.cc:685-706: objects A, B, C; then (K != 0) sizes of A,
+    // sizes of B; then sizes of C.
+    if (!A) return clblasInvalidMatA;
+    if (!B) return clblasInvalidMatB;
+    if (!C) return clblasInvalidMatC;
+    if (!valid_order(order) || !valid_trans(transA) || !valid_trans(transB)) return clblasInvalidValue;
+    clblasStatus st;
+    if (K != 0) {
+        if ((st = check_matrix_sizes(order, transA, M, K, lda, MAT_A)) != clblasSuccess) return st;
+        if ((st = check_matrix_sizes(order, transB, K, N, ldb, MAT_B)) != clblasSuccess) return st;
+    }
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if (M > kMaxDim || N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
+
+    // Real types: ConjTrans is Trans (xgemm.cc:330-335).
+    bool tA = transA != clblasNoTrans, tB = transB != clblasNoTrans;
+    const T *pa = A + offA, *pb = B + offB;
+    // Row major is the column-major product C^T = op(B)^T op(A)^T (xgemm.cc:40-61):
+    // swap the operands, their transposes, leading dimensions, and M with N.
+    if (order == clblasRowMajor) {
+        std::swap(tA, tB);
+        std::swap(M, N);
+        std::swap(lda, ldb);
+        std::swap(pa, pb);
+    }
+    return map_hip_error(launch(tA, tB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb, (int64_t)ldb, beta,
+                                C + offC, (int64_t)ldc, stream));
+}
+
+template <typename T, typename Fn>
+clblasStatus trsm_front(Fn launch, clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                        clblasDiag diag, size_t M, size_t N, T alpha, const T *A, size_t offA, size_t lda, T *B,
+                        size_t offB, size_t ldb, hipStream_t stream) {
+    // Order of checks follows doTrsm (functor_xtrsm.cc:57-75): objects, A (msize^2), B (M x N).
+    if (!A) return clblasInvalidMatA;
+    if (!B) return clblasInvalidMatB;
+    if (!valid_order(order) || !valid_trans(transA) || (side != clblasLeft && side != clblasRight) ||
+        (uplo != clblasUpper && uplo != clblasLower) || (diag != clblasUnit && diag != clblasNonUnit))
+        return clblasInvalidValue;
+    const size_t msize = side == clblasLeft ? M : N;
+    clblasStatus st;
+    if ((st = check_matrix_sizes(order, transA, msize, msize, lda, MAT_A)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B)) != clblasSuccess) return st;
+    if (M > kMaxDim || N > kMaxDim) return clblasNotImplemented;
+
+    bool right = side == clblasRight, lower = uplo == clblasLower;
+    // Row major: the same memory read column-major holds A^T and B^T, so solve the
+    // transposed system: swap M and N, flip side and uplo; trans and diag stay
+    // (xtrsm.cc:54-64).
+    if (order == clblasRowMajor) {
+        std::swap(M, N);
+        right = !right;
+        lower = !lower;
+    }
+    return map_hip_error(launch(right, lower, transA != clblasNoTrans, diag == clblasUnit, (int)M, (int)N, alpha,
+                                A + offA, (int64_t)lda, B + offB, (int64_t)ldb, stream));
+}
+
+}  // namespace
+
+extern "C" {
+
+clblasStatus clblasGetVersion(unsigned int *major, unsigned int *minor, unsigned int *patch) {
+    if (major) *major = 0;
+    if (minor) *minor = 1;
+    if (patch) *patch = 0;
+    return clblasSuccess;
+}
+
+clblasStatus clblasSetup(void) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return clblasInvalidDevice;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return clblasInvalidDevice;
+    }
+    // The code object holds gfx950 ISA only.
+    const char *arch = prop.gcnArchName;
+    const char want[] = "gfx950";
+    for (int i = 0; i < 6; ++i)
+        if (arch[i] != want[i]) return clblasInvalidDevice;
+    return clblasSuccess;
+}
+
+void clblasTeardown(void) { cba::workspace_release_all(); }
+
+clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
+                         size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B,
+                         size_t offB, size_t ldb, float beta, float *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return gemm_front<float>(cba::sgemm_colmajor, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb,
+                             beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
+                         size_t K, double alpha, const double *A, size_t offA, size_t lda, const double *B,
+                         size_t offB, size_t ldb, double beta, double *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return gemm_front<double>(cba::dgemm_colmajor, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB,
+                              ldb, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasStrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, float alpha, const float *A, size_t offA, size_t lda,
+                         float *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<float>(cba::strsm_colmajor, order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
+                             offB, ldb, stream);
+}
+
+clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, double alpha, const double *A, size_t offA,
+                         size_t lda, double *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<double>(cba::dtrsm_colmajor, order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
+                              offB, ldb, stream);
+}
+
+}  // extern "C"

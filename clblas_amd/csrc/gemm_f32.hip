@@ -1,0 +1,27 @@
+// FP32 GEMM: tile table and entry point.
+#include "gemm_launch.hpp"
+
+namespace cba {
+
+// Ordered from the largest tile to the smallest.
+//   0: 256x128x16, wave 128x64 (2 workgroups of 4 waves per CU)
+//   1: 128x128x16, wave 64x64
+//   2:  64x64x16,  wave 32x32, split-K capable (small / deep-K problems)
+static const TileEntry<float> *f32_tiles(int *n) {
+    static const TileEntry<float> tab[] = {
+        make_tile_entry<float, 256, 128, 16, 128, 64, 2, false>(),
+        make_tile_entry<float, 128, 128, 16, 64, 64, 2, false>(),
+        make_tile_entry<float, 64, 64, 16, 32, 32, 2, true>(),
+    };
+    *n = (int)(sizeof(tab) / sizeof(tab[0]));
+    return tab;
+}
+
+hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float alpha, const float *A, int64_t lda,
+                          const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream) {
+    int n;
+    const TileEntry<float> *tab = f32_tiles(&n);
+    return run_gemm_colmajor<float>(tab, n, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+
+}  // namespace cba

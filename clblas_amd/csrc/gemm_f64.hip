@@ -1,0 +1,26 @@
+// FP64 GEMM: tile table and entry point.
+#include "gemm_launch.hpp"
+
+namespace cba {
+
+// Ordered from the largest tile to the smallest.
+//   0: 128x128x16, wave 64x64 (2 workgroups of 4 waves per CU)
+//   1:  64x64x16,  wave 32x32, split-K capable
+static const TileEntry<double> *f64_tiles(int *n) {
+    static const TileEntry<double> tab[] = {
+        make_tile_entry<double, 128, 128, 16, 64, 64, 2, false>(),
+        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true>(),
+    };
+    *n = (int)(sizeof(tab) / sizeof(tab[0]));
+    return tab;
+}
+
+hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double alpha, const double *A,
+                          int64_t lda, const double *B, int64_t ldb, double beta, double *C, int64_t ldc,
+                          hipStream_t stream) {
+    int n;
+    const TileEntry<double> *tab = f64_tiles(&n);
+    return run_gemm_colmajor<double>(tab, n, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+
+}  // namespace cba

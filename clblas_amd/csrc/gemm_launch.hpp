@@ -1,0 +1,152 @@
+// Host-side launch plumbing shared by the FP32 and FP64 GEMM translation units:
+// one table entry per (tile shape), each holding the 4 transpose x {plain, split-K}
+// kernel instantiations.  Takes the place of the reference's generated
+// gemmSelectKernel<T>() / makeGemmKernel / enqueueGemmKernel
+// (src/library/blas/xgemm.cc:160-313, AutoGemm/KernelSelection.py:101-305): kernels are
+// compiled ahead of time, so "selection" is only a table lookup.
+#pragma once
+
+#include "gemm_kernel.hpp"
+#include "internal.h"
+
+namespace cba {
+
+template <typename T> struct TileEntry {
+    int bm, bn, bk, threads;
+    size_t smem;
+    bool has_splitk;
+    // index: (transA ? 2 : 0) | (transB ? 1 : 0)
+    void (*plain[4])(const GemmParams<T>);
+    void (*splitk[4])(const GemmParams<T>);
+};
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK>
+TileEntry<T> make_tile_entry() {
+    typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;  // smem / threads do not depend on transposes
+    TileEntry<T> e;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.smem = Cfg::SMEM; e.has_splitk = WITH_SPLITK;
+    // A is k-contiguous when transposed; B is k-contiguous when NOT transposed.
+    e.plain[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, false, MINW>;   // NN
+    e.plain[1] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, false, false, MINW>;  // NT
+    e.plain[2] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, true, false, MINW>;    // TN
+    e.plain[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, false, MINW>;   // TT
+    if constexpr (WITH_SPLITK) {
+        e.splitk[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, true, MINW>;
+        e.splitk[1] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, false, true, MINW>;
+        e.splitk[2] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, true, true, MINW>;
+        e.splitk[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, true, MINW>;
+    } else {
+        for (int i = 0; i < 4; ++i) e.splitk[i] = nullptr;
+    }
+    return e;
+}
+
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Chooses tile and split count.  The reference keys its choice on M*N brackets and
+// divisibility (AutoGemmParameters.py:8-55); here remainders are handled in-kernel, so
+// the only question is how to fill 256 CUs: the largest tile that still yields enough
+// workgroups, and a K split when even the smallest tile cannot.
+template <typename T>
+static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, int *tile_out,
+                        int *splits_out) {
+    const int64_t kCUs = 256;
+    int pick = ntab - 1;  // table is ordered large -> small
+    if (force >= 0 && force < ntab) {
+        pick = force;
+    } else {
+        for (int i = 0; i < ntab; ++i) {
+            int64_t t = ceil_div64(M, tab[i].bm) * ceil_div64(N, tab[i].bn);
+            // Work actually computed vs. useful work: avoid tiles that are mostly padding.
+            double useful = ((double)M * N) / ((double)t * tab[i].bm * tab[i].bn);
+            int64_t resident = (tab[i].smem * 2 <= 160 * 1024 && tab[i].threads <= 256) ? 2 : 1;
+            if (t >= kCUs * resident && useful >= 0.80) { pick = i; break; }
+        }
+    }
+    int splits = 1;
+    if (tab[pick].has_splitk) {
+        int64_t t = ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn);
+        if (t < kCUs && K >= 8 * tab[pick].bk) {
+            int64_t want = (2 * kCUs) / t;              // aim for ~2 workgroups per CU
+            int64_t max_by_k = K / (4 * tab[pick].bk);  // at least 4 panels per split
+            splits = (int)(want < max_by_k ? want : max_by_k);
+            if (splits < 1) splits = 1;
+            if (splits > 64) splits = 64;
+        }
+    }
+    *tile_out = pick;
+    *splits_out = splits;
+}
+
+template <typename T>
+static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, bool tB, int M, int N, int K,
+                                    T alpha, const T *A, int64_t lda, const T *B, int64_t ldb, T beta, T *C,
+                                    int64_t ldc, hipStream_t stream) {
+    if (K == 0) {
+        int mb = (int)ceil_div64(M, 256);
+        hipLaunchKernelGGL(scale_c_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
+                           beta, C, ldc);
+        return hipGetLastError();
+    }
+    // 32-bit panel offsets: (tile edge or panel depth) * ld * sizeof(T) must stay < 2^31.
+    const int64_t max_edge = 256;
+    const int64_t ld_limit = (int64_t)0x7fffffff / (max_edge * (int64_t)sizeof(T)) - 8;
+    if (lda > ld_limit || ldb > ld_limit) {
+        int mb = (int)ceil_div64(M, 256);
+        hipLaunchKernelGGL(gemm_wide_ld_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream,
+                           tA ? 1 : 0, tB ? 1 : 0, M, N, K, mb, alpha, A, lda, B, ldb, beta, C, ldc);
+        return hipGetLastError();
+    }
+
+    int tile, splits;
+    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), &tile, &splits);
+    const TileEntry<T> &e = tab[tile];
+
+    GemmParams<T> p;
+    p.A = A; p.B = B; p.C = C;
+    p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    // op(A) is M x K: stored M x K (ld rows = M) when not transposed, K x M when transposed.
+    p.a_bytes = (tA ? ((int64_t)(M - 1) * lda + K) : ((int64_t)(K - 1) * lda + M)) * (int64_t)sizeof(T);
+    p.b_bytes = (tB ? ((int64_t)(K - 1) * ldb + N) : ((int64_t)(N - 1) * ldb + K)) * (int64_t)sizeof(T);
+    p.M = M; p.N = N; p.K = K;
+    p.alpha = alpha; p.beta = beta;
+    p.tiles_m = (int)ceil_div64(M, e.bm);
+    p.tiles_n = (int)ceil_div64(N, e.bn);
+    p.group_m = p.tiles_m < 8 ? p.tiles_m : 8;
+    p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
+    p.k_per_split = K;
+    const int idx = (tA ? 2 : 0) | (tB ? 1 : 0);
+    const int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n;
+    if (ntiles > 0x7fffffffLL) return hipErrorInvalidValue;
+
+    auto fn = e.plain[idx];
+    if (splits > 1) {
+        int64_t kps = ceil_div64(ceil_div64(K, splits), e.bk) * e.bk;
+        splits = (int)ceil_div64(K, kps);
+        if (splits > 1) {
+            p.k_per_split = (int)kps;
+            p.ws_ld = ((int64_t)M + 63) / 64 * 64;
+            p.ws_slice = p.ws_ld * N;
+            void *w = workspace_get(stream, (size_t)(p.ws_slice * splits) * sizeof(T));
+            if (!w) return hipErrorOutOfMemory;
+            p.ws = (T *)w;
+            fn = e.splitk[idx];
+        }
+    }
+    if (e.smem > 64 * 1024) {
+        hipError_t err = ensure_dynamic_lds((const void *)fn, e.smem);
+        if (err != hipSuccess) return err;
+    }
+    hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)splits), dim3(e.threads), e.smem, stream, p);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    if (splits > 1) {
+        int mb = (int)ceil_div64(M, 256);
+        hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, p.ws,
+                           p.ws_ld, p.ws_slice, splits, M, N, mb, alpha, beta, C, ldc);
+        err = hipGetLastError();
+    }
+    return err;
+}
+
+}  // namespace cba

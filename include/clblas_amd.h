@@ -1,0 +1,144 @@
+/*
+ * clblas_amd.h -- C ABI of the MI355X (gfx950) BLAS-3 core that stands in for the
+ * xGEMM / xTRSM path of clBLAS.
+ *
+ * The entry points keep clBLAS's names, argument order and status codes.  The only
+ * differences to the reference prototypes are the ones a HIP back end forces:
+ *   - `cl_mem` matrices become device pointers (`const float *`, `double *`, ...);
+ *     element offsets (offA/offB/offC) are kept and are added to those pointers,
+ *   - the five trailing queue/event arguments
+ *       (numCommandQueues, commandQueues, numEventsInWaitList, eventWaitList, events)
+ *     collapse into one `hipStream_t stream`; stream order supplies both the wait and
+ *     the completion semantics.
+ * Every call returns after enqueueing its work on `stream`.
+ *
+ * The library is plain C ABI: no C++ or torch types cross it.
+ */
+#ifndef CLBLAS_AMD_H_
+#define CLBLAS_AMD_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Same opaque stream type as <hip/hip_runtime_api.h>; repeating the typedef is legal. */
+typedef struct ihipStream_t *hipStream_t;
+
+/* Enumerations: numeric values identical to reference src/clBLAS.h:78-113. */
+typedef enum clblasOrder_ {
+    clblasRowMajor = 0,
+    clblasColumnMajor = 1
+} clblasOrder;
+
+typedef enum clblasTranspose_ {
+    clblasNoTrans = 0,
+    clblasTrans = 1,
+    clblasConjTrans = 2 /* same as clblasTrans for real types (xgemm.cc:330-335) */
+} clblasTranspose;
+
+typedef enum clblasUplo_ {
+    clblasUpper = 0,
+    clblasLower = 1
+} clblasUplo;
+
+typedef enum clblasDiag_ {
+    clblasUnit = 0,
+    clblasNonUnit = 1
+} clblasDiag;
+
+typedef enum clblasSide_ {
+    clblasLeft = 0,
+    clblasRight = 1
+} clblasSide;
+
+/* Status codes: numeric values identical to reference src/clBLAS.h:123-155
+ * (the OpenCL aliases keep the OpenCL numbers they had there). */
+typedef enum clblasStatus_ {
+    clblasSuccess = 0,
+    clblasInvalidValue = -30,         /* CL_INVALID_VALUE: bad enum argument */
+    clblasInvalidCommandQueue = -36,  /* CL_INVALID_COMMAND_QUEUE */
+    clblasInvalidContext = -34,
+    clblasInvalidMemObject = -38,
+    clblasInvalidDevice = -33,
+    clblasInvalidEventWaitList = -57,
+    clblasOutOfResources = -5,        /* a HIP launch or allocation failed */
+    clblasOutOfHostMemory = -6,
+    clblasInvalidOperation = -59,
+    clblasCompilerNotAvailable = -3,
+    clblasBuildProgramFailure = -11,
+    clblasNotImplemented = -1024,
+    clblasNotInitialized = -1023,
+    clblasInvalidMatA = -1022,
+    clblasInvalidMatB = -1021,
+    clblasInvalidMatC = -1020,
+    clblasInvalidVecX = -1019,
+    clblasInvalidVecY = -1018,
+    clblasInvalidDim = -1017,
+    clblasInvalidLeadDimA = -1016,
+    clblasInvalidLeadDimB = -1015,
+    clblasInvalidLeadDimC = -1014,
+    clblasInvalidIncX = -1013,
+    clblasInvalidIncY = -1012,
+    clblasInsufficientMemMatA = -1011,
+    clblasInsufficientMemMatB = -1010,
+    clblasInsufficientMemMatC = -1009,
+    clblasInsufficientMemVecX = -1008,
+    clblasInsufficientMemVecY = -1007
+} clblasStatus;
+
+/* Replaces clblasGetVersion (src/clBLAS.h:176-177, src/library/blas/init.c:33-41).
+ * Reports this library's own version. Always clblasSuccess. */
+clblasStatus clblasGetVersion(unsigned int *major, unsigned int *minor, unsigned int *patch);
+
+/* Replaces clblasSetup (src/clBLAS.h:196-197, src/library/blas/init.c:43-223).
+ * Checks that a gfx950 device is current and its code object loads.  GEMM and TRSM
+ * do not require it (the reference's GEMM path does not check it either). */
+clblasStatus clblasSetup(void);
+
+/* Replaces clblasTeardown (src/clBLAS.h:208-209, src/library/blas/init.c:232-263).
+ * Releases the library-owned device workspace. */
+void clblasTeardown(void);
+
+/* Replaces clblasSgemm (src/clBLAS.h:7382-7405, src/library/blas/xgemm.cc:667-723).
+ *   C <- alpha * op(A) * op(B) + beta * C, fp32.  beta == 0 means C is not read.
+ * Validation order and codes follow xgemm.cc:685-706 and generic/common.c:585-688:
+ *   null A/B/C -> clblasInvalidMat{A,B,C}; if K != 0 sizes of A then B; sizes of C.
+ * K == 0 computes C <- beta*C (the reference kernel loop is undefined there). */
+clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB,
+                         size_t M, size_t N, size_t K, float alpha,
+                         const float *A, size_t offA, size_t lda,
+                         const float *B, size_t offB, size_t ldb, float beta,
+                         float *C, size_t offC, size_t ldc, hipStream_t stream);
+
+/* Replaces clblasDgemm (src/clBLAS.h:7463-7486, src/library/blas/xgemm.cc:728-783). */
+clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB,
+                         size_t M, size_t N, size_t K, double alpha,
+                         const double *A, size_t offA, size_t lda,
+                         const double *B, size_t offB, size_t ldb, double beta,
+                         double *C, size_t offC, size_t ldc, hipStream_t stream);
+
+/* Replaces clblasStrsm (src/clBLAS.h:7988-8008, src/library/blas/xtrsm.cc:1600-1661).
+ *   side == Left : solve op(A) * X = alpha * B,  A is M x M
+ *   side == Right: solve X * op(A) = alpha * B,  A is N x N
+ * X overwrites B (M x N).  Only the `uplo` triangle of A is read and, with
+ * diag == Unit, not its diagonal.  Validation follows doTrsm
+ * (src/library/blas/functor/functor_xtrsm.cc:57-75): null A/B -> clblasInvalidMat{A,B},
+ * then A (msize x msize), then B (M x N). */
+clblasStatus clblasStrsm(clblasOrder order, clblasSide side, clblasUplo uplo,
+                         clblasTranspose transA, clblasDiag diag, size_t M, size_t N,
+                         float alpha, const float *A, size_t offA, size_t lda,
+                         float *B, size_t offB, size_t ldb, hipStream_t stream);
+
+/* Replaces clblasDtrsm (src/clBLAS.h:8063-8083, src/library/blas/xtrsm.cc:1663-1785). */
+clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo,
+                         clblasTranspose transA, clblasDiag diag, size_t M, size_t N,
+                         double alpha, const double *A, size_t offA, size_t lda,
+                         double *B, size_t offB, size_t ldb, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CLBLAS_AMD_H_ */

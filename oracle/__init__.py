@@ -1,0 +1,192 @@
+"""numpy-facing loader for the CPU oracle (oracle/liboracle.so, oracle/_ref/libnaive_ref.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by __graft_entry__.smoke() and by the
+cpu_baseline leg of bench.py -- never by the product package (clblas_amd).
+
+All matrices are 1-D numpy buffers addressed exactly as the C API addresses them
+(element offsets and leading dimensions), so the tests read like the reference's own.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "liboracle.so")
+REF_LIB_PATH = os.path.join(_HERE, "_ref", "libnaive_ref.so")
+
+_lib = None
+_ref = None
+
+_sz = ctypes.c_size_t
+_i = ctypes.c_int
+_vp = ctypes.c_void_p
+_u64 = ctypes.c_uint64
+
+
+def build(verbose=False):
+    """Compiles liboracle.so and, if the reference tree is present, _ref/libnaive_ref.so."""
+    res = subprocess.run(["make", "-C", _HERE, "-B", "all"], capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("oracle build failed:\n" + res.stdout + res.stderr)
+    if verbose:
+        print(res.stdout.strip())
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        L = ctypes.CDLL(LIB_PATH)
+        for name, real in (("oracle_sgemm", ctypes.c_float), ("oracle_dgemm", ctypes.c_double)):
+            f = getattr(L, name)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, _sz, real, _vp, _sz, _sz, _vp, _sz, _sz, real, _vp, _sz, _sz]
+        for name, real in (("oracle_sgemm_exact", ctypes.c_float), ("oracle_dgemm_exact", ctypes.c_double)):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_i, _i, _sz, real, _vp, _sz, _vp, _sz, real, _vp, _sz, _sz, _vp, _vp, _vp, _vp]
+        for name, real in (("oracle_strsm_naive", ctypes.c_float), ("oracle_dtrsm_naive", ctypes.c_double),
+                           ("oracle_strsm_blocked", ctypes.c_float), ("oracle_dtrsm_blocked", ctypes.c_double)):
+            f = getattr(L, name)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _i, _i, _sz, _sz, real, _vp, _sz, _sz, _vp, _sz, _sz]
+        L.oracle_check_gemm.restype = _i
+        L.oracle_check_gemm.argtypes = [_i, _i, _i, _sz, _sz, _sz, _i, _sz, _sz, _sz, _i, _sz, _sz, _sz, _i, _sz,
+                                        _sz, _sz]
+        L.oracle_check_trsm.restype = _i
+        L.oracle_check_trsm.argtypes = [_i, _i, _i, _sz, _sz, _i, _sz, _sz, _sz, _i, _sz, _sz, _sz]
+        L.oracle_num_threads.restype = _i
+        for name in ("oracle_fill_uniform_f32", "oracle_fill_uniform_f64", "oracle_fill_normal_f32",
+                     "oracle_fill_normal_f64"):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_vp, _sz, _u64]
+        for name in ("oracle_fill_int_f32", "oracle_fill_int_f64"):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_vp, _sz, _u64, ctypes.c_uint32]
+        for name in ("oracle_fill_tri_f32", "oracle_fill_tri_f64"):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_vp, _sz, _sz, _i, _i, _u64]
+        _lib = L
+    return _lib
+
+
+def ref_lib():
+    """The reference's own naive BLAS (compiled from the reference tree), or None if absent."""
+    global _ref
+    if _ref is None:
+        if not os.path.exists(REF_LIB_PATH):
+            return None
+        L = ctypes.CDLL(REF_LIB_PATH)
+        for name, real in (("ref_naive_sgemm", ctypes.c_float), ("ref_naive_dgemm", ctypes.c_double)):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_i, _i, _i, _sz, _sz, _sz, real, _vp, _sz, _vp, _sz, real, _vp, _sz]
+        for name, real in (("ref_naive_strsm", ctypes.c_float), ("ref_naive_dtrsm", ctypes.c_double)):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_i, _i, _i, _i, _i, _sz, _sz, real, _vp, _sz, _vp, _sz]
+        _ref = L
+    return _ref
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(_vp)
+
+
+def _real(a):
+    return "s" if a.dtype == np.float32 else "d"
+
+
+def num_threads():
+    return lib().oracle_num_threads()
+
+
+def gemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    """In-place on C (1-D buffer). Returns the clblasStatus the reference would return."""
+    ref = C if C is not None else (A if A is not None else B)
+    f = lib().oracle_sgemm if ref.dtype == np.float32 else lib().oracle_dgemm
+    return f(int(order), int(transA), int(transB), M, N, K, alpha, _p(A), offA, lda, _p(B), offB, ldb, beta, _p(C),
+             offC, ldc)
+
+
+def gemm_exact(transA, transB, K, alpha, A, lda, B, ldb, beta, C, ldc, rows, cols):
+    """Column-major; A/B/C buffers start at element (0,0).  Returns (exact, magnitude) in
+    float64 for the listed elements: magnitude = |alpha| sum|a b| + |beta c|."""
+    rows = np.ascontiguousarray(rows, dtype=np.int64)
+    cols = np.ascontiguousarray(cols, dtype=np.int64)
+    exact = np.empty(rows.size, dtype=np.float64)
+    mag = np.empty(rows.size, dtype=np.float64)
+    f = lib().oracle_sgemm_exact if A.dtype == np.float32 else lib().oracle_dgemm_exact
+    f(int(bool(transA)), int(bool(transB)), K, alpha, _p(A), lda, _p(B), ldb, beta, _p(C), ldc, rows.size, _p(rows),
+      _p(cols), _p(exact), _p(mag))
+    return exact, mag
+
+
+def trsm_naive(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
+    ref = B if B is not None else A
+    f = lib().oracle_strsm_naive if ref.dtype == np.float32 else lib().oracle_dtrsm_naive
+    return f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha, _p(A), offA, lda, _p(B), offB,
+             ldb)
+
+
+def trsm_blocked(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
+    ref = B if B is not None else A
+    f = lib().oracle_strsm_blocked if ref.dtype == np.float32 else lib().oracle_dtrsm_blocked
+    return f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha, _p(A), offA, lda, _p(B), offB,
+             ldb)
+
+
+def check_gemm(order, transA, transB, M, N, K, haveA, offA, lda, memA, haveB, offB, ldb, memB, haveC, offC, ldc,
+               memC):
+    return lib().oracle_check_gemm(int(order), int(transA), int(transB), M, N, K, int(haveA), offA, lda, memA,
+                                   int(haveB), offB, ldb, memB, int(haveC), offC, ldc, memC)
+
+
+def check_trsm(order, side, transA, M, N, haveA, offA, lda, memA, haveB, offB, ldb, memB):
+    return lib().oracle_check_trsm(int(order), int(side), int(transA), M, N, int(haveA), offA, lda, memA,
+                                   int(haveB), offB, ldb, memB)
+
+
+def ref_gemm(order, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc):
+    """Reference naive gemm (no offsets: pass views that start at the first element)."""
+    f = ref_lib().ref_naive_sgemm if C.dtype == np.float32 else ref_lib().ref_naive_dgemm
+    f(int(order), int(transA), int(transB), M, N, K, alpha, _p(A), lda, _p(B), ldb, beta, _p(C), ldc)
+
+
+def ref_trsm(order, side, uplo, transA, diag, M, N, alpha, A, lda, B, ldb):
+    f = ref_lib().ref_naive_strsm if B.dtype == np.float32 else ref_lib().ref_naive_dtrsm
+    f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha, _p(A), lda, _p(B), ldb)
+
+
+# ---- seeded generators -------------------------------------------------------------------
+
+def uniform(n, seed, dtype=np.float32):
+    x = np.empty(n, dtype=dtype)
+    (lib().oracle_fill_uniform_f32 if dtype == np.float32 else lib().oracle_fill_uniform_f64)(_p(x), n, seed)
+    return x
+
+
+def normal(n, seed, dtype=np.float64):
+    x = np.empty(n, dtype=dtype)
+    (lib().oracle_fill_normal_f32 if dtype == np.float32 else lib().oracle_fill_normal_f64)(_p(x), n, seed)
+    return x
+
+
+def integers(n, seed, limit, dtype=np.float32):
+    x = np.empty(n, dtype=dtype)
+    (lib().oracle_fill_int_f32 if dtype == np.float32 else lib().oracle_fill_int_f64)(_p(x), n, seed, limit)
+    return x
+
+
+def triangular(n, ld, lower, seed, dtype=np.float64, poison_diag=False, tail=0):
+    """ld*n (+tail) element buffer holding a conditioned triangular matrix, NaN elsewhere in the square."""
+    a = np.full(ld * n + tail, np.nan, dtype=dtype)
+    (lib().oracle_fill_tri_f32 if dtype == np.float32 else lib().oracle_fill_tri_f64)(_p(a), n, ld, int(lower),
+                                                                                    int(poison_diag), seed)
+    return a

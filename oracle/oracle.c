@@ -1,0 +1,412 @@
+/*
+ * oracle.c -- CPU restatement of the clBLAS xGEMM / xTRSM hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing in the shipped library links or calls this file; it is
+ * used by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of bench.py as the
+ * checker / the timed CPU reference.
+ *
+ * Every function names the reference lines (relative to the clBLAS source tree) it follows.
+ *
+ * How each function is pinned (see tests/test_oracle.py):
+ *   oracle_{s,d}gemm        - README.md:77-156 and src/samples/example_sgemm.c:31-73 fixed
+ *                             inputs with hand-computed expected outputs; integer-exact inputs
+ *                             (src/tests/include/blas-random.h:60-93) against exact integer
+ *                             products; closed forms (identity, rank-1, alpha=0, NaN in C with
+ *                             beta=0); transposition and row/column-major identities; the
+ *                             reference's own naive gemm compiled from
+ *                             src/library/tools/ktest/naive/naive_blas.cpp (oracle/_ref).
+ *   oracle_{s,d}gemm_exact  - same integer-exact inputs (must reproduce them exactly).
+ *   oracle_{s,d}trsm_naive  - TRSM_extratest closed form (src/tests/correctness/corr-trsm.cpp:
+ *                             240-452, X_r = r+1); src/samples/example_strsm.c:30-63 fixed
+ *                             input; oracle/_ref naive trsm; residual identities.
+ *   oracle_{s,d}trsm_blocked- the same, plus agreement with the naive solver within the
+ *                             reference's own per-element bound (trsm-delta.h:44-240 style),
+ *                             NaN-poisoned unused triangle, zero-diagonal -> 1 behaviour.
+ *   oracle_check_*          - expectations of src/tests/functional/func-error.cpp:58-104 and
+ *                             the branch table of generic/common.c:585-688.
+ *   Bit-for-bit output of the OpenCL kernels (implementation-defined `mad` contraction,
+ *   AutoGemm/KernelOpenCL.py:100) is NOT pinned: no OpenCL device exists to run them.
+ *   Parity is judged with the K*eps bound, as the task states.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* enum values of src/clBLAS.h:78-155 */
+enum { ROW_MAJOR = 0, COL_MAJOR = 1 };
+enum { NO_TRANS = 0, TRANS = 1, CONJ_TRANS = 2 };
+enum { UPPER = 0, LOWER = 1 };
+enum { UNIT = 0, NON_UNIT = 1 };
+enum { LEFT = 0, RIGHT = 1 };
+enum {
+    ST_SUCCESS = 0,
+    ST_NOT_IMPLEMENTED = -1024,
+    ST_INVALID_MAT_A = -1022,
+    ST_INVALID_MAT_B = -1021,
+    ST_INVALID_MAT_C = -1020,
+    ST_INVALID_DIM = -1017,
+    ST_INVALID_LD_A = -1016,
+    ST_INVALID_LD_B = -1015,
+    ST_INVALID_LD_C = -1014,
+    ST_INSUFF_A = -1011,
+    ST_INSUFF_B = -1010,
+    ST_INSUFF_C = -1009
+};
+
+int oracle_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* Argument checks                                                                       */
+/* ------------------------------------------------------------------------------------ */
+
+/* checkMatrixSizes, src/library/blas/generic/common.c:585-688.  which: 0=A 1=B 2=C.
+ * mem_elems: size of the buffer in elements, or 0 for "unknown / large enough". */
+static int check_matrix_sizes(int order, int trans, size_t M, size_t N, size_t off, size_t ld, size_t mem_elems,
+                              int which) {
+    size_t matr;
+    int tra;
+    if (M == 0 || N == 0) return ST_INVALID_DIM; /* :601-603 */
+    tra = (order == ROW_MAJOR && trans != NO_TRANS) || (order == COL_MAJOR && trans == NO_TRANS); /* :606-607 */
+    if (tra) {
+        if (ld < M) return ST_INVALID_LD_A + which; /* :610-624 */
+        matr = (N - 1) * ld + M;                    /* :625 */
+    } else {
+        if (ld < N) return ST_INVALID_LD_A + which; /* :628-641 */
+        matr = (M - 1) * ld + N;                    /* :642 */
+    }
+    if (mem_elems != 0 && off + matr > mem_elems) return ST_INSUFF_A + which; /* :670-684 */
+    return ST_SUCCESS;
+}
+
+/* clblasSgemm / clblasDgemm front-end checks, src/library/blas/xgemm.cc:685-706.
+ * haveX: nonzero if the X object is valid (checkMemObjects, generic/common.c:837-900). */
+int oracle_check_gemm(int order, int transA, int transB, size_t M, size_t N, size_t K, int haveA, size_t offA,
+                      size_t lda, size_t memA, int haveB, size_t offB, size_t ldb, size_t memB, int haveC,
+                      size_t offC, size_t ldc, size_t memC) {
+    int st;
+    if (!haveA) return ST_INVALID_MAT_A;
+    if (!haveB) return ST_INVALID_MAT_B;
+    if (!haveC) return ST_INVALID_MAT_C;
+    if (K != 0) {
+        if ((st = check_matrix_sizes(order, transA, M, K, offA, lda, memA, 0))) return st;
+        if ((st = check_matrix_sizes(order, transB, K, N, offB, ldb, memB, 1))) return st;
+    }
+    return check_matrix_sizes(order, NO_TRANS, M, N, offC, ldc, memC, 2);
+}
+
+/* doTrsm checks, src/library/blas/functor/functor_xtrsm.cc:57-75. */
+int oracle_check_trsm(int order, int side, int transA, size_t M, size_t N, int haveA, size_t offA, size_t lda,
+                      size_t memA, int haveB, size_t offB, size_t ldb, size_t memB) {
+    int st;
+    size_t msize = side == LEFT ? M : N;
+    if (!haveA) return ST_INVALID_MAT_A;
+    if (!haveB) return ST_INVALID_MAT_B;
+    if ((st = check_matrix_sizes(order, transA, msize, msize, offA, lda, memA, 0))) return st;
+    return check_matrix_sizes(order, NO_TRANS, M, N, offB, ldb, memB, 1);
+}
+
+/* ------------------------------------------------------------------------------------ */
+/* GEMM                                                                                  */
+/* ------------------------------------------------------------------------------------ */
+
+/* Column-major kernel arithmetic, src/library/blas/AutoGemm/KernelOpenCL.py:
+ *   :311-422  one accumulator per C element, k strictly ascending, TYPE_MAD = mad(a,b,acc)
+ *             (restated as a fused multiply-add)
+ *   :100-104  epilogue  C = alpha*acc + beta*C  (beta != 0)   or   C = alpha*acc (beta == 0,
+ *             C never read)
+ * Element addressing: :68-81.  The loops are arranged so that rows of C vectorise; every
+ * element still sees k = 0,1,2,... in order. */
+#define GEMM_COLMAJOR(NAME, T, FMA)                                                                         \
+    static void NAME(int tA, int tB, size_t M, size_t N, size_t K, T alpha, const T *A, size_t lda,         \
+                     const T *B, size_t ldb, T beta, T *C, size_t ldc) {                                    \
+        const size_t MBLK = 64;                                                                              \
+        ptrdiff_t nb;                                                                                        \
+        const ptrdiff_t n_mblk = (ptrdiff_t)((M + MBLK - 1) / MBLK);                                         \
+        _Pragma("omp parallel for schedule(dynamic, 1)")                                                     \
+        for (nb = 0; nb < n_mblk; ++nb) {                                                                    \
+            const size_t m0 = (size_t)nb * MBLK;                                                             \
+            const size_t mlen = (M - m0) < MBLK ? (M - m0) : MBLK;                                           \
+            T acc[64];                                                                                       \
+            T apan[64];                                                                                      \
+            size_t n, k, i;                                                                                  \
+            for (n = 0; n < N; ++n) {                                                                        \
+                for (i = 0; i < mlen; ++i) acc[i] = (T)0;                                                    \
+                for (k = 0; k < K; ++k) {                                                                    \
+                    const T b = tB ? B[n + k * ldb] : B[k + n * ldb];                                        \
+                    if (tA) {                                                                                \
+                        for (i = 0; i < mlen; ++i) apan[i] = A[k + (m0 + i) * lda];                          \
+                    } else {                                                                                 \
+                        const T *ap = A + m0 + k * lda;                                                      \
+                        for (i = 0; i < mlen; ++i) apan[i] = ap[i];                                          \
+                    }                                                                                        \
+                    _Pragma("omp simd")                                                                      \
+                    for (i = 0; i < mlen; ++i) acc[i] = FMA(apan[i], b, acc[i]);                             \
+                }                                                                                            \
+                {                                                                                            \
+                    T *cp = C + m0 + n * ldc;                                                                \
+                    if (beta == (T)0) {                                                                      \
+                        for (i = 0; i < mlen; ++i) cp[i] = alpha * acc[i];                                   \
+                    } else {                                                                                 \
+                        for (i = 0; i < mlen; ++i) cp[i] = alpha * acc[i] + beta * cp[i];                    \
+                    }                                                                                        \
+                }                                                                                            \
+            }                                                                                                \
+        }                                                                                                    \
+    }
+
+GEMM_COLMAJOR(sgemm_colmajor, float, fmaf)
+GEMM_COLMAJOR(dgemm_colmajor, double, fma)
+
+/* Front end: checks (xgemm.cc:685-706), ConjTrans -> Trans for real types (xgemm.cc:330-335),
+ * row-major folded to column-major by swapping the operands (xgemm.cc:40-61). */
+#define GEMM_FRONT(NAME, T, CORE)                                                                            \
+    int NAME(int order, int transA, int transB, size_t M, size_t N, size_t K, T alpha, const T *A,          \
+             size_t offA, size_t lda, const T *B, size_t offB, size_t ldb, T beta, T *C, size_t offC,       \
+             size_t ldc) {                                                                                   \
+        int st = oracle_check_gemm(order, transA, transB, M, N, K, A != NULL, offA, lda, 0, B != NULL, offB, \
+                                   ldb, 0, C != NULL, offC, ldc, 0);                                         \
+        int tA, tB;                                                                                          \
+        if (st) return st;                                                                                   \
+        tA = transA != NO_TRANS;                                                                             \
+        tB = transB != NO_TRANS;                                                                             \
+        if (order == ROW_MAJOR)                                                                              \
+            CORE(tB, tA, N, M, K, alpha, B + offB, ldb, A + offA, lda, beta, C + offC, ldc);                 \
+        else                                                                                                 \
+            CORE(tA, tB, M, N, K, alpha, A + offA, lda, B + offB, ldb, beta, C + offC, ldc);                 \
+        return ST_SUCCESS;                                                                                   \
+    }
+
+GEMM_FRONT(oracle_sgemm, float, sgemm_colmajor)
+GEMM_FRONT(oracle_dgemm, double, dgemm_colmajor)
+
+/* High-precision evaluation of selected elements of a column-major GEMM, plus the magnitude
+ * term of the parity bound   |C - C_ref| <= c * K * eps * (|alpha| |A||B| + |beta| |C|).
+ * Products and sums are carried in a wider type (double for fp32 data, long double for fp64
+ * data).  rows/cols list `count` element positions; exact[i] and mag[i] are written.
+ * Not a restatement of reference code: this is the yardstick both the reference result and
+ * ours are measured against. */
+#define GEMM_EXACT(NAME, T, W, ABSW)                                                                         \
+    void NAME(int tA, int tB, size_t K, T alpha, const T *A, size_t lda, const T *B, size_t ldb, T beta,    \
+              const T *C, size_t ldc, size_t count, const int64_t *rows, const int64_t *cols, double *exact, \
+              double *mag) {                                                                                 \
+        ptrdiff_t i;                                                                                         \
+        _Pragma("omp parallel for schedule(static)")                                                         \
+        for (i = 0; i < (ptrdiff_t)count; ++i) {                                                             \
+            const size_t m = (size_t)rows[i], n = (size_t)cols[i];                                           \
+            W s = 0, sa = 0;                                                                                 \
+            size_t k;                                                                                        \
+            for (k = 0; k < K; ++k) {                                                                        \
+                const W a = tA ? A[k + m * lda] : A[m + k * lda];                                            \
+                const W b = tB ? B[n + k * ldb] : B[k + n * ldb];                                            \
+                s += a * b;                                                                                  \
+                sa += ABSW(a * b);                                                                           \
+            }                                                                                                \
+            {                                                                                                \
+                W r = (W)alpha * s, g = ABSW((W)alpha) * sa;                                                 \
+                if (!(beta == (T)0)) {                                                                       \
+                    r += (W)beta * (W)C[m + n * ldc];                                                        \
+                    g += ABSW((W)beta * (W)C[m + n * ldc]);                                                  \
+                }                                                                                            \
+                exact[i] = (double)r;                                                                        \
+                mag[i] = (double)g;                                                                          \
+            }                                                                                                \
+        }                                                                                                    \
+    }
+
+GEMM_EXACT(oracle_sgemm_exact, float, double, fabs)
+GEMM_EXACT(oracle_dgemm_exact, double, long double, fabsl)
+
+/* ------------------------------------------------------------------------------------ */
+/* TRSM                                                                                  */
+/* ------------------------------------------------------------------------------------ */
+
+/* Row-by-row substitution followed by a scaling with alpha: the reference's own CPU
+ * statement of TRSM, src/library/tools/ktest/naive/naive_blas.cpp:632-684.
+ * MatrixAccessor semantics (naive_blas.cpp:480-528): element (r,c) of op(A). */
+#define ACC_A(T, r, c) (a_rowstride * (r) + a_colstride * (c))
+#define TRSM_NAIVE(NAME, T)                                                                                  \
+    int NAME(int order, int side, int uplo, int transA, int diag, size_t M, size_t N, T alpha, const T *A,  \
+             size_t offA, size_t lda, T *B, size_t offB, size_t ldb) {                                       \
+        int st = oracle_check_trsm(order, side, transA, M, N, A != NULL, offA, lda, 0, B != NULL, offB, ldb, \
+                                   0);                                                                       \
+        size_t rowsA, colsB, i, j, k, a_rowstride, a_colstride, b_rowstride, b_colstride;                    \
+        int rev, tra;                                                                                        \
+        if (st) return st;                                                                                   \
+        A += offA;                                                                                           \
+        B += offB;                                                                                           \
+        rowsA = side == LEFT ? M : N;                                                                        \
+        colsB = side == LEFT ? N : M;                                                                        \
+        /* element (r,c) of op(A) and of B (viewed as rowsA x colsB) */                                      \
+        tra = transA != NO_TRANS;                                                                            \
+        rev = (uplo == UPPER) ^ tra;              /* :650 */                                                 \
+        if (side == RIGHT) {                      /* :651-655: solve the transposed system */                \
+            tra = !tra;                                                                                      \
+            rev = !rev;                                                                                      \
+        }                                                                                                    \
+        if ((order == COL_MAJOR) != tra) { a_rowstride = 1; a_colstride = lda; }                             \
+        else { a_rowstride = lda; a_colstride = 1; }                                                         \
+        if ((order == COL_MAJOR) != (side == RIGHT)) { b_rowstride = 1; b_colstride = ldb; }                 \
+        else { b_rowstride = ldb; b_colstride = 1; }                                                         \
+        for (i = 0; i < rowsA; ++i) {                                                                        \
+            const size_t row = rev ? rowsA - i - 1 : i;                                                      \
+            for (j = 0; j < colsB; ++j) {                                                                    \
+                const size_t boundK = rev ? rowsA - row - 1 : row;                                           \
+                T tmp = (T)0;                                                                                \
+                for (k = 0; k <= boundK; ++k) {                                                              \
+                    const size_t col = rev ? rowsA - k - 1 : k;                                              \
+                    if (col == row) {                                                                        \
+                        const T a = diag == UNIT ? (T)1 : A[ACC_A(T, row, col)];                             \
+                        tmp = (B[b_rowstride * row + b_colstride * j] - tmp) / a;                            \
+                    } else {                                                                                 \
+                        tmp = tmp + A[ACC_A(T, row, col)] * B[b_rowstride * col + b_colstride * j];          \
+                    }                                                                                        \
+                }                                                                                            \
+                B[b_rowstride * row + b_colstride * j] = tmp;                                                \
+            }                                                                                                \
+        }                                                                                                    \
+        for (i = 0; i < rowsA; ++i)                                                                          \
+            for (j = 0; j < colsB; ++j)                                                                      \
+                B[b_rowstride * i + b_colstride * j] = B[b_rowstride * i + b_colstride * j] * alpha;         \
+        return ST_SUCCESS;                                                                                   \
+    }
+
+TRSM_NAIVE(oracle_strsm_naive, float)
+TRSM_NAIVE(oracle_dtrsm_naive, double)
+
+/* The reference's device algorithm for DTRSM: gpu_dtrsm128, src/library/blas/xtrsm.cc:1136-1507.
+ *   1. InvA <- explicit inverses of the NB x NB (NB = 128) diagonal blocks of A
+ *      (diag_dtrtri128, xtrsm.cc:790-1134): every 16x16 diagonal block is inverted
+ *      column by column (trtri/diag_dtrtri_lower_128_16.cpp:85-165,
+ *      trtri/diag_dtrtri_upper_128_16.cpp), unit diagonal forced to 1, a zero diagonal
+ *      entry replaced by 1 (:87-96), rows/columns past the matrix read as zero (:67-74);
+ *      then blocks are doubled 16->32->64->128 with
+ *        lower: inv21 = -inv22 * (A21 * inv11)   (triple_dgemm_update_128_*_PART{1,2}_L.cpp)
+ *        upper: inv12 = -inv11 * (A12 * inv22)   (triple_dgemm_update_128_*_R.cpp)
+ *   2. block sweep X_i = op(InvA_ii) * B_i, B_rest = -op(A_rest,i) X_i + (alpha|1) B_rest with
+ *      the public DGEMM, writing X to a zeroed M x N temporary that is copied back at the
+ *      end (xtrsm.cc:1186-1192, 1229-1497).
+ * The same algorithm is used here for fp32 (the reference routes STRSM through its legacy
+ * solver instead, gens/trsm.c:1213-1456; its bit pattern is not restated). */
+#define REAL float
+#define FN(name) name##_s
+#define ORACLE_TRSM_BLOCKED oracle_strsm_blocked
+#define GEMM_CORE sgemm_colmajor
+#include "trsm_blocked.inc"
+#undef REAL
+#undef FN
+#undef ORACLE_TRSM_BLOCKED
+#undef GEMM_CORE
+
+#define REAL double
+#define FN(name) name##_d
+#define ORACLE_TRSM_BLOCKED oracle_dtrsm_blocked
+#define GEMM_CORE dgemm_colmajor
+#include "trsm_blocked.inc"
+#undef REAL
+#undef FN
+#undef ORACLE_TRSM_BLOCKED
+#undef GEMM_CORE
+
+/* ------------------------------------------------------------------------------------ */
+/* Seeded input generators (portable: splitmix64, identical on every host)               */
+/* ------------------------------------------------------------------------------------ */
+
+static inline uint64_t mix64(uint64_t z) {
+    z += 0x9e3779b97f4a7c15ULL;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+    return z ^ (z >> 31);
+}
+/* counter-based: value i of stream `seed` */
+static inline uint64_t rnd_u64(uint64_t seed, uint64_t i) { return mix64(mix64(seed) + i * 0x9e3779b97f4a7c15ULL); }
+static inline double rnd_unit(uint64_t seed, uint64_t i) { /* [0,1) with 53 bits */
+    return (double)(rnd_u64(seed, i) >> 11) * (1.0 / 9007199254740992.0);
+}
+
+/* uniform [-1,1) */
+void oracle_fill_uniform_f32(float *x, size_t n, uint64_t seed) {
+    ptrdiff_t i;
+    _Pragma("omp parallel for schedule(static)")
+    for (i = 0; i < (ptrdiff_t)n; ++i) {
+        /* 24 random bits so that the value is exactly representable in fp32 */
+        x[i] = (float)((double)(rnd_u64(seed, (uint64_t)i) >> 40) * (1.0 / 8388608.0) - 1.0);
+    }
+}
+void oracle_fill_uniform_f64(double *x, size_t n, uint64_t seed) {
+    ptrdiff_t i;
+    _Pragma("omp parallel for schedule(static)")
+    for (i = 0; i < (ptrdiff_t)n; ++i) x[i] = 2.0 * rnd_unit(seed, (uint64_t)i) - 1.0;
+}
+/* normal(0,1), Box-Muller on two counter-based uniforms */
+void oracle_fill_normal_f64(double *x, size_t n, uint64_t seed) {
+    ptrdiff_t i;
+    _Pragma("omp parallel for schedule(static)")
+    for (i = 0; i < (ptrdiff_t)n; ++i) {
+        double u1 = 1.0 - rnd_unit(seed, 2 * (uint64_t)i); /* (0,1] */
+        double u2 = rnd_unit(seed, 2 * (uint64_t)i + 1);
+        x[i] = sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2);
+    }
+}
+void oracle_fill_normal_f32(float *x, size_t n, uint64_t seed) {
+    ptrdiff_t i;
+    _Pragma("omp parallel for schedule(static)")
+    for (i = 0; i < (ptrdiff_t)n; ++i) {
+        double u1 = 1.0 - rnd_unit(seed, 2 * (uint64_t)i);
+        double u2 = rnd_unit(seed, 2 * (uint64_t)i + 1);
+        x[i] = (float)(sqrt(-2.0 * log(u1)) * cos(6.283185307179586476925 * u2));
+    }
+}
+/* signed integers in (-limit, limit): the reference tests' exact-arithmetic inputs,
+ * random<T>(limit) = +-(rand() % limit), src/tests/include/blas-math.h:232-246 */
+void oracle_fill_int_f32(float *x, size_t n, uint64_t seed, uint32_t limit) {
+    size_t i;
+    for (i = 0; i < n; ++i) {
+        uint64_t r = rnd_u64(seed, i);
+        float v = (float)((r >> 8) % limit);
+        x[i] = (r & 1) ? -v : v;
+    }
+}
+void oracle_fill_int_f64(double *x, size_t n, uint64_t seed, uint32_t limit) {
+    size_t i;
+    for (i = 0; i < n; ++i) {
+        uint64_t r = rnd_u64(seed, i);
+        double v = (double)((r >> 8) % limit);
+        x[i] = (r & 1) ? -v : v;
+    }
+}
+
+/* Well-conditioned triangular matrix of order n, column-major with leading dimension ld:
+ * strict triangle uniform[-1,1)/n, diagonal uniform[1,2); the other triangle (and, if
+ * poison_diag, the diagonal) is NaN so that any illegal read shows in the result, as in the
+ * reference tests (src/tests/include/blas-random.h:258-263, 311-317). */
+#define FILL_TRI(NAME, T)                                                                                    \
+    void NAME(T *a, size_t n, size_t ld, int lower, int poison_diag, uint64_t seed) {                        \
+        ptrdiff_t c;                                                                                         \
+        _Pragma("omp parallel for schedule(static)")                                                         \
+        for (c = 0; c < (ptrdiff_t)n; ++c) {                                                                 \
+            size_t r;                                                                                        \
+            for (r = 0; r < n; ++r) {                                                                        \
+                uint64_t idx = (uint64_t)r + (uint64_t)c * n;                                                \
+                T v;                                                                                         \
+                if (r == (size_t)c) v = poison_diag ? (T)NAN : (T)(1.0 + rnd_unit(seed, idx));               \
+                else if ((lower && r > (size_t)c) || (!lower && r < (size_t)c))                              \
+                    v = (T)((2.0 * rnd_unit(seed, idx) - 1.0) / (double)n);                                  \
+                else v = (T)NAN;                                                                             \
+                a[r + (size_t)c * ld] = v;                                                                   \
+            }                                                                                                \
+        }                                                                                                    \
+    }
+FILL_TRI(oracle_fill_tri_f32, float)
+FILL_TRI(oracle_fill_tri_f64, double)

@@ -1,0 +1,48 @@
+// Builds the reference's own CPU statement of GEMM / TRSM -- the "naive BLAS" its kernel
+// test tool checks against -- straight from the reference tree, for use as a second
+// opinion on oracle.c.  TEST INFRASTRUCTURE ONLY.
+//
+// The reference file is included by path from where it lies
+// (REF_ROOT/src/library/tools/ktest/naive/naive_blas.cpp); no reference text is copied into
+// this repository.  That file has no includes of its own, so the headers it relies on
+// (all present in this image) are pulled in first.
+#include <CL/cl.h>
+
+#include <cmath>
+#include <cstddef>
+#include <cstdlib>
+#include <string>
+using std::isnan;
+
+#include REF_NAIVE_BLAS_CPP
+
+extern "C" {
+
+void ref_naive_sgemm(int order, int transA, int transB, size_t M, size_t N, size_t K, float alpha, const float *A,
+                     size_t lda, const float *B, size_t ldb, float beta, float *C, size_t ldc) {
+    NaiveBlas::gemm<float>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasTranspose)transA,
+                           (NaiveBlas::clblasTranspose)transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
+}
+
+void ref_naive_dgemm(int order, int transA, int transB, size_t M, size_t N, size_t K, double alpha,
+                     const double *A, size_t lda, const double *B, size_t ldb, double beta, double *C,
+                     size_t ldc) {
+    NaiveBlas::gemm<double>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasTranspose)transA,
+                            (NaiveBlas::clblasTranspose)transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
+}
+
+void ref_naive_strsm(int order, int side, int uplo, int transA, int diag, size_t M, size_t N, float alpha,
+                     const float *A, size_t lda, float *B, size_t ldb) {
+    NaiveBlas::trsm<float>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasSide)side, (NaiveBlas::clblasUplo)uplo,
+                           (NaiveBlas::clblasTranspose)transA, (NaiveBlas::clblasDiag)diag, M, N, alpha, A, lda, B,
+                           ldb);
+}
+
+void ref_naive_dtrsm(int order, int side, int uplo, int transA, int diag, size_t M, size_t N, double alpha,
+                     const double *A, size_t lda, double *B, size_t ldb) {
+    NaiveBlas::trsm<double>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasSide)side,
+                            (NaiveBlas::clblasUplo)uplo, (NaiveBlas::clblasTranspose)transA,
+                            (NaiveBlas::clblasDiag)diag, M, N, alpha, A, lda, B, ldb);
+}
+
+}  // extern "C"

@@ -1,0 +1,140 @@
+"""Writes tests/golden/fixed_cases.json: the fixed-input cases the reference's own files hold
+for the xGEMM / xTRSM path, with expected outputs computed here in exact rational arithmetic
+(python Fractions) -- independent of both the oracle and the HIP library.
+
+Sources of the INPUT DATA (data only; no reference code is run or copied):
+  * README.md:77-156            row-major SGEMM 4x5 * 5x3, alpha=10, beta=20, zero offsets
+  * src/samples/example_sgemm.c:31-73,156-160  same matrices, sub-problem (M-1,N-1,K-1) at
+                                offA=K+1, offB=N+1, offC=N+1
+  * src/samples/example_strsm.c:30-63,140-142  row-major STRSM left/upper/notrans/nonunit,
+                                sub-problem (M-1,N-1) at offA=M+1, offB=N+1, alpha=10
+  * src/tests/correctness/corr-trsm.cpp:240-291,313-452  TRSM_extratest: column-major,
+                                left/upper/notrans/nonunit, M=5, N=2, lda=ldb=32,
+                                a_rr=r+1, a_rc=1 (c>r), b_r = sum(1..M)-sum(1..r+1)+(r+1)^2
+                                => x_r = r+1 (closed form)
+
+Run:  python tests/golden/make_golden.py
+"""
+import json
+import os
+from fractions import Fraction as F
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+ROW, COL = 0, 1
+N_, T_ = 0, 1
+UPPER, LOWER = 0, 1
+UNIT, NONUNIT = 0, 1
+LEFT, RIGHT = 0, 1
+
+
+def a_index(order, trans, r, c, ld):
+    """Buffer index of element (r,c) of op(X) (src/library/blas/AutoGemm/KernelOpenCL.py:68-81)."""
+    if (order == COL) == (trans == N_):
+        return r + c * ld
+    return r * ld + c
+
+
+def gemm_exact(order, tA, tB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    out = [F(x) for x in C]
+    for m in range(M):
+        for n in range(N):
+            s = F(0)
+            for k in range(K):
+                s += F(A[offA + a_index(order, tA, m, k, lda)]) * F(B[offB + a_index(order, tB, k, n, ldb)])
+            ci = offC + a_index(order, N_, m, n, ldc)
+            out[ci] = F(alpha) * s + F(beta) * F(C[ci])
+    return out
+
+
+def trsm_exact(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
+    """Solves op(A) X = alpha B (left) or X op(A) = alpha B (right) exactly."""
+    n = M if side == LEFT else N
+    # dense op(A) restricted to its triangle
+    opA = [[F(0)] * n for _ in range(n)]
+    for r in range(n):
+        for c in range(n):
+            # (r,c) of op(A) is (c,r) of A when transposed
+            rr, cc = (c, r) if tA != N_ else (r, c)
+            in_tri = (rr <= cc) if uplo == UPPER else (rr >= cc)
+            if not in_tri:
+                continue
+            if rr == cc and diag == UNIT:
+                opA[r][c] = F(1)
+            else:
+                opA[r][c] = F(A[offA + a_index(order, N_, rr, cc, lda)])
+    out = [F(x) for x in B]
+    nrhs = N if side == LEFT else M
+    for j in range(nrhs):
+        # right: x^T solves op(A)^T x^T = alpha b^T
+        Tm = opA if side == LEFT else [[opA[c][r] for c in range(n)] for r in range(n)]
+        def bidx(i):
+            return offB + (a_index(order, N_, i, j, ldb) if side == LEFT else a_index(order, N_, j, i, ldb))
+        rhs = [F(alpha) * F(B[bidx(i)]) for i in range(n)]
+        # generic exact elimination on a triangular system (forward or backward)
+        x = [None] * n
+        lower = all(Tm[r][c] == 0 for r in range(n) for c in range(r + 1, n))
+        order_rows = range(n) if lower else range(n - 1, -1, -1)
+        for r in order_rows:
+            s = rhs[r]
+            for c in range(n):
+                if c != r and x[c] is not None:
+                    s -= Tm[r][c] * x[c]
+            x[r] = s / Tm[r][r]
+        for i in range(n):
+            out[bidx(i)] = x[i]
+    return out
+
+
+def as_floats(v):
+    return [float(x) for x in v]
+
+
+def main():
+    cases = {}
+    A = [11, 12, 13, 14, 15, 21, 22, 23, 24, 25, 31, 32, 33, 34, 35, 41, 42, 43, 44, 45]
+    B = [11, 12, 13, 21, 22, 23, 31, 32, 33, 41, 42, 43, 51, 52, 53]
+    C = [11, 12, 13, 21, 22, 23, 31, 32, 33, 41, 42, 43]
+    M, N, K = 4, 3, 5
+    cases["readme_sgemm"] = dict(
+        kind="gemm", dtype="f32", order=ROW, transA=N_, transB=N_, M=M, N=N, K=K, alpha=10, beta=20, A=A, offA=0,
+        lda=K, B=B, offB=0, ldb=N, C=C, offC=0, ldc=N,
+        expected=as_floats(gemm_exact(ROW, N_, N_, M, N, K, 10, A, 0, K, B, 0, N, 20, C, 0, N)))
+    cases["sample_sgemm_offsets"] = dict(
+        kind="gemm", dtype="f32", order=ROW, transA=N_, transB=N_, M=M - 1, N=N - 1, K=K - 1, alpha=10, beta=20,
+        A=A, offA=K + 1, lda=K, B=B, offB=N + 1, ldb=N, C=C, offC=N + 1, ldc=N,
+        expected=as_floats(gemm_exact(ROW, N_, N_, M - 1, N - 1, K - 1, 10, A, K + 1, K, B, N + 1, N, 20, C, N + 1,
+                                      N)))
+    At = [11, 12, 13, 14, 0, 22, 23, 24, 0, 0, 33, 34, 0, 0, 0, 44]
+    Bt = [11, 12, 13, 14, 15, 21, 22, 23, 24, 25, 31, 32, 33, 34, 35, 41, 42, 43, 44, 45]
+    cases["sample_strsm_offsets"] = dict(
+        kind="trsm", dtype="f32", order=ROW, side=LEFT, uplo=UPPER, transA=N_, diag=NONUNIT, M=3, N=4, alpha=10,
+        A=At, offA=5, lda=4, B=Bt, offB=6, ldb=5,
+        expected=as_floats(trsm_exact(ROW, LEFT, UPPER, N_, NONUNIT, 3, 4, 10, At, 5, 4, Bt, 6, 5)))
+    # TRSM_extratest
+    Me, Ne, ld = 5, 2, 32
+    Ae = [0.0] * (Me * ld)
+    Be = [0.0] * (Ne * ld)
+    tri = lambda n: n * (n + 1) // 2
+    for i in range(Me):          # column i
+        for j in range(Me):      # row j
+            Ae[i * ld + j] = float(j + 1) if j == i else (0.0 if j > i else 1.0)
+    for i in range(Ne):
+        for j in range(Me):
+            Be[i * ld + j] = float(tri(Me) - tri(j + 1) + (j + 1) * (j + 1))
+    exp = trsm_exact(COL, LEFT, UPPER, N_, NONUNIT, Me, Ne, 1, Ae, 0, ld, Be, 0, ld)
+    # closed form from the reference test: X_r = r + 1
+    for i in range(Ne):
+        for j in range(Me):
+            assert exp[i * ld + j] == j + 1
+    for dt in ("f32", "f64"):
+        cases["extratest_" + dt] = dict(
+            kind="trsm", dtype=dt, order=COL, side=LEFT, uplo=UPPER, transA=N_, diag=NONUNIT, M=Me, N=Ne, alpha=1,
+            A=Ae, offA=0, lda=ld, B=Be, offB=0, ldb=ld, expected=as_floats(exp), tol=1e-5)
+    with open(os.path.join(HERE, "fixed_cases.json"), "w") as f:
+        json.dump(cases, f, indent=1)
+    print("wrote", len(cases), "cases")
+
+
+if __name__ == "__main__":
+    main()
