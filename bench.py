@@ -1,0 +1,188 @@
+#!/usr/bin/env python3
+"""Benchmark of the xGEMM / xTRSM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm]
+
+A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
+column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
+HBM).  Prints ONE JSON line.  `value` is SGEMM TFLOP/s using the reference's own flop
+count 2*M*N*K (src/client/clfunc_xgemm.hpp:95-107); DGEMM (config 4) and DTRSM (config 5,
+M*(M+1)*N flops, src/client/clfunc_xtrsm.hpp:70-92) are reported in `extra`.
+`cpu_baseline` times the CPU oracle (a port of the reference arithmetic, OpenMP over the
+host cores) on a bounded sample of the same workload; it is a reported baseline only.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MATRIX = 157.3  # TFLOP/s, MI355X dense MFMA
+PEAK_FP64_MATRIX = 78.6
+
+COL, NOTRANS, TRANS = 1, 0, 1
+LEFT, LOWER, NONUNIT = 0, 1, 1
+
+
+def timed_calls(torch, call, steps, warmup, before_each=None):
+    """Runs `call` warmup+steps times on torch's current stream; returns (wall seconds for the
+    timed steps, mean per-launch milliseconds from HIP events recorded on that stream)."""
+    for _ in range(warmup):
+        if before_each:
+            before_each()
+        call()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        if before_each:
+            before_each()
+        starts[i].record()
+        call()
+        stops[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = sum(s.elapsed_time(e) for s, e in zip(starts, stops)) / steps
+    return wall, ev_ms
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm or dtrsm (profiling)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (one MI355X per box); use --gpus 1")
+
+    import torch
+    import clblas_amd
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    torch.cuda.set_device(0)
+    if clblas_amd.setup() != 0:
+        sys.exit("bench.py: clblasSetup failed (library needs a gfx950 device)")
+
+    n = args.size
+    steps, warmup = args.steps, args.warmup
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1234)
+    extra = {}
+    result = None
+
+    # ---- SGEMM, BASELINE config 2 -------------------------------------------------------
+    if args.only in ("", "sgemm"):
+        A = torch.rand(n * n, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+        B = torch.rand(n * n, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+        C = torch.rand(n * n, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+
+        def sgemm():
+            st = clblas_amd.sgemm(COL, NOTRANS, NOTRANS, n, n, n, 1.0, A, 0, n, B, 0, n, 1.0, C, 0, n)
+            if st != 0:
+                raise RuntimeError("clblasSgemm returned %d" % st)
+
+        wall, ev_ms = timed_calls(torch, sgemm, steps, warmup)
+        flops = 2.0 * n * n * n
+        ms_per_step = wall * 1e3 / steps
+        tflops = flops / (wall / steps) / 1e12
+        kernel_tflops = flops / (ev_ms * 1e-3) / 1e12
+        result = {
+            "metric": "SGEMM TFLOP/s at %d^3 (col-major NN, alpha=1, beta=1) on 1 MI355X" % n,
+            "value": round(tflops, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+            "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "BASELINE config 2: SGEMM column-major NN M=N=K=%d, tight ld, alpha=1, beta=1, "
+                                   "uniform[-1,1)" % n},
+            "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MATRIX,
+                         "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MATRIX, 4), "traffic": None,
+                         "kernel": "gemm_mfma_kernel<float,256,128,16,...> (one launch per call)",
+                         "launch_ms": round(ev_ms, 4)},
+        }
+        extra["sgemm_pct_of_fp32_matrix_peak"] = round(100 * tflops / PEAK_FP32_MATRIX, 2)
+        del A, B, C
+
+    # ---- DGEMM, BASELINE config 4 -------------------------------------------------------
+    if args.only in ("", "dgemm"):
+        A = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
+        B = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
+        C = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
+
+        def dgemm():
+            st = clblas_amd.dgemm(COL, NOTRANS, TRANS, n, n, n, 1.0, A, 0, n, B, 0, n, 0.5, C, 0, n)
+            if st != 0:
+                raise RuntimeError("clblasDgemm returned %d" % st)
+
+        wall, ev_ms = timed_calls(torch, dgemm, steps, warmup)
+        d_tflops = 2.0 * n * n * n / (wall / steps) / 1e12
+        extra["dgemm"] = {"workload": "BASELINE config 4: DGEMM column-major NT %d^3, alpha=1, beta=0.5, normal(0,1)" % n,
+                          "tflops": round(d_tflops, 3), "ms_per_call": round(wall * 1e3 / steps, 4),
+                          "launch_ms": round(ev_ms, 4),
+                          "pct_of_fp64_matrix_peak": round(100 * d_tflops / PEAK_FP64_MATRIX, 2)}
+        del A, B, C
+    else:
+        d_tflops = None
+
+    # ---- DTRSM, BASELINE config 5 -------------------------------------------------------
+    if args.only in ("", "dtrsm"):
+        A = torch.rand(n * n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1
+        A /= n
+        Av = A.view(n, n)  # Av[c, r] is element (r, c) of the column-major matrix
+        Av.diagonal().copy_(torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) + 1)
+        Av.copy_(torch.where(torch.ones(n, n, device="cuda", dtype=torch.bool).tril(-1), torch.full_like(Av, float("nan")), Av))
+        B0 = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
+        B = B0.clone()
+
+        def restore():
+            B.copy_(B0)
+
+        def dtrsm():
+            st = clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, A, 0, n, B, 0, n)
+            if st != 0:
+                raise RuntimeError("clblasDtrsm returned %d" % st)
+
+        tsteps = max(3, steps // 2)
+        wall, ev_ms = timed_calls(torch, dtrsm, tsteps, 2, before_each=restore)
+        t_tflops = float(n) * (n + 1) * n / (ev_ms * 1e-3) / 1e12
+        extra["dtrsm"] = {"workload": "BASELINE config 5: DTRSM Left/Lower/NoTrans/NonUnit M=N=%d, alpha=1" % n,
+                          "tflops": round(t_tflops, 3), "ms_per_call": round(ev_ms, 4),
+                          "finite": bool(torch.isfinite(B).all().item())}
+        if d_tflops:
+            extra["dtrsm"]["pct_of_dgemm_rate"] = round(100 * t_tflops / d_tflops, 2)
+        del A, B, B0
+
+    # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
+    cpu = None
+    if not args.no_cpu and args.only == "":
+        import numpy as np
+        import oracle
+        m_s, n_s, k_s = 2048, 1024, n     # same K (same per-element work) on a block of C
+        a = oracle.uniform(m_s * k_s, 1, np.float32)
+        b = oracle.uniform(k_s * n_s, 2, np.float32)
+        c = oracle.uniform(m_s * n_s, 3, np.float32)
+        oracle.gemm(COL, NOTRANS, NOTRANS, 256, 64, 256, 1.0, a, 0, m_s, b, 0, k_s, 1.0, c, 0, m_s)  # warm-up
+        t0 = time.perf_counter()
+        oracle.gemm(COL, NOTRANS, NOTRANS, m_s, n_s, k_s, 1.0, a, 0, m_s, b, 0, k_s, 1.0, c, 0, m_s)
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(2.0 * m_s * n_s * k_s / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(),
+               "kind": "port",
+               "sample": "oracle SGEMM NN on a %dx%d block of C with the full K=%d (%.1f s); the reference clBLAS "
+                         "itself needs an OpenCL device (PoCL), which this image does not have" % (m_s, n_s, k_s, dt)}
+
+    if result is None:
+        result = {"metric": "partial run (--only %s)" % args.only, "value": None, "unit": "TFLOP/s", "n_gpus": 1,
+                  "steps": steps, "warmup": warmup}
+    result["cpu_baseline"] = cpu
+    result["extra"] = extra
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,33 @@
+"""Runs the C-ABI entry points on numpy buffers: upload, call, synchronise, download.
+torch is used only to hold device memory."""
+import os
+
+import numpy as np
+import torch
+
+import clblas_amd
+
+
+def _dev(x):
+    return torch.from_numpy(x).cuda()
+
+
+def gemm(order, tA, tB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, tile=None):
+    fn = clblas_amd.sgemm if C.dtype == np.float32 else clblas_amd.dgemm
+    dA, dB, dC = _dev(A), _dev(B), _dev(C)
+    if tile is not None:
+        os.environ["CLBLAS_AMD_GEMM_TILE"] = str(tile)
+    try:
+        st = fn(order, tA, tB, M, N, K, alpha, dA, offA, lda, dB, offB, ldb, beta, dC, offC, ldc)
+        torch.cuda.synchronize()
+    finally:
+        os.environ.pop("CLBLAS_AMD_GEMM_TILE", None)
+    return st, dC.cpu().numpy()
+
+
+def trsm(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
+    fn = clblas_amd.strsm if B.dtype == np.float32 else clblas_amd.dtrsm
+    dA, dB = _dev(A), _dev(B)
+    st = fn(order, side, uplo, tA, diag, M, N, alpha, dA, offA, lda, dB, offB, ldb)
+    torch.cuda.synchronize()
+    return st, dB.cpu().numpy()

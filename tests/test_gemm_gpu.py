@@ -1,0 +1,211 @@
+"""GPU parity tests for clblasSgemm / clblasDgemm through the C ABI, against the CPU oracle.
+
+Bars: exact equality on the reference tests' exact-integer inputs (any summation order gives
+the same bits there); for real-valued inputs
+    |C - C_exact| <= 2 (K+2) u (|alpha| |A||B| + |beta||C|),   u = unit roundoff,
+i.e. the task's c*K*eps bound with c = 2, which both our result and the reference's
+one-accumulator result satisfy."""
+import itertools
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import (COL, ROW, NOTRANS, TRANS, CONJ, buf_len, exact_int_limits, gemm_bound, golden_cases,
+                     logical_view, mem_dims)
+
+pytestmark = pytest.mark.gpu
+
+DT = {"f32": np.float32, "f64": np.float64}
+N_TILES = {np.float32: 3, np.float64: 2}
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import gpu_util
+    import torch
+    assert torch.cuda.is_available()
+    import clblas_amd
+    assert clblas_amd.setup() == 0
+    return gpu_util
+
+
+@pytest.mark.parametrize("name", ["readme_sgemm", "sample_sgemm_offsets"])
+def test_golden(gpu, name):
+    c = golden_cases()[name]
+    dt = DT[c["dtype"]]
+    A, B, C = (np.array(c[k], dtype=dt) for k in "ABC")
+    st, out = gpu.gemm(c["order"], c["transA"], c["transB"], c["M"], c["N"], c["K"], c["alpha"], A, c["offA"],
+                       c["lda"], B, c["offB"], c["ldb"], c["beta"], C, c["offC"], c["ldc"])
+    assert st == 0
+    np.testing.assert_array_equal(out, np.array(c["expected"], dtype=dt))
+
+
+def _layout(order, tA, tB, M, N, K, pad, offs):
+    ia, oa = mem_dims(order, tA, M, K)
+    ib, ob = mem_dims(order, tB, K, N)
+    ic, oc = mem_dims(order, NOTRANS, M, N)
+    lda, ldb, ldc = ia + pad, ib + pad, ic + pad
+    offA, offB, offC = offs
+    return (lda, ldb, ldc, offA + oa * lda, offB + ob * ldb, offC + oc * ldc)
+
+
+INT_SHAPES = [(1, 1, 1), (2, 1, 3), (8, 16, 17), (17, 32, 62), (64, 64, 64), (62, 144, 128), (256, 128, 16),
+              (257, 129, 33), (300, 520, 200), (130, 70, 1031)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("order", [ROW, COL])
+@pytest.mark.parametrize("tA,tB", list(itertools.product([NOTRANS, TRANS], [NOTRANS, TRANS, CONJ])))
+def test_integer_exact_all_tiles(gpu, dtype, order, tA, tB):
+    """The reference's own correctness method (corr-gemm.cpp:192, matrix.h:322-327): integer
+    data small enough that the result is exact, compared with assert-equal.  Every tile of
+    the table is forced in turn, plus the default choice."""
+    for si, (M, N, K) in enumerate(INT_SHAPES):
+        alpha, beta = 3.0, -2.0
+        la, lc = exact_int_limits(K, alpha, beta, dtype)
+        offs = (5, 7, 11)
+        lda, ldb, ldc, na, nb, nc = _layout(order, tA, tB, M, N, K, 3, offs)
+        A = oracle.integers(na, 100 + si, la, dtype)
+        B = oracle.integers(nb, 200 + si, la, dtype)
+        C = oracle.integers(nc, 300 + si, lc, dtype)
+        want = C.copy()
+        assert oracle.gemm(order, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, want, offs[2],
+                           ldc) == 0
+        for tile in [None] + list(range(N_TILES[dtype])):
+            st, got = gpu.gemm(order, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc,
+                               tile=tile)
+            assert st == 0
+            np.testing.assert_array_equal(got, want, err_msg="shape %s tile %s" % ((M, N, K), tile))
+
+
+def _check_sampled(dtype, tA, tB, M, N, K, alpha, beta, A, lda, B, ldb, C0, got, ldc, nsamp=3000, seed=0):
+    """Column-major buffers starting at element (0,0).  Checks sampled elements (all four
+    borders plus random interior points) against the high-precision oracle."""
+    rng = np.random.default_rng(seed)
+    rows = [rng.integers(0, M, nsamp), np.full(200, M - 1), np.zeros(200, dtype=np.int64), rng.integers(0, M, 400)]
+    cols = [rng.integers(0, N, nsamp), rng.integers(0, N, 200), rng.integers(0, N, 200),
+            np.concatenate([np.full(200, N - 1), np.zeros(200, dtype=np.int64)])]
+    rows, cols = np.concatenate(rows), np.concatenate(cols)
+    exact, mag = oracle.gemm_exact(tA, tB, K, alpha, A, lda, B, ldb, beta, C0, ldc, rows, cols)
+    vals = got[rows + cols * ldc].astype(np.float64)
+    err = np.abs(vals - exact)
+    bound = gemm_bound(K, mag, dtype)
+    worst = np.argmax(err / bound)
+    assert np.all(err <= bound), "element (%d,%d): err %.3e bound %.3e" % (rows[worst], cols[worst], err[worst],
+                                                                          bound[worst])
+    return float((err / bound).max())
+
+
+def test_config1_sgemm_1024_full_matrix(gpu):
+    """BASELINE config 1: SGEMM NN 1024^3, alpha=1, beta=0, uniform[-1,1): every element,
+    against the oracle's result and the exact product."""
+    n = 1024
+    A, B, C = oracle.uniform(n * n, 1, np.float32), oracle.uniform(n * n, 2, np.float32), oracle.uniform(n * n, 3, np.float32)
+    want = C.copy()
+    assert oracle.gemm(COL, NOTRANS, NOTRANS, n, n, n, 1.0, A, 0, n, B, 0, n, 0.0, want, 0, n) == 0
+    st, got = gpu.gemm(COL, NOTRANS, NOTRANS, n, n, n, 1.0, A, 0, n, B, 0, n, 0.0, C, 0, n)
+    assert st == 0
+    A64, B64 = A.reshape(n, n).T.astype(np.float64), B.reshape(n, n).T.astype(np.float64)
+    exact = A64 @ B64
+    mag = np.abs(A64) @ np.abs(B64)
+    bound = gemm_bound(n, mag, np.float32)
+    assert np.all(np.abs(got.reshape(n, n).T - exact) <= bound)
+    assert np.all(np.abs(want.reshape(n, n).T - exact) <= bound)      # the oracle sits inside the same bound
+    assert np.all(np.abs(got.astype(np.float64) - want) <= 2 * bound.T.ravel())
+
+
+def test_beta_zero_never_reads_c_and_alpha_zero(gpu):
+    for dtype in (np.float32, np.float64):
+        M, N, K = 70, 90, 50
+        A, B = oracle.uniform(M * K, 1, dtype), oracle.uniform(K * N, 2, dtype)
+        C = np.full(M * N, np.nan, dtype=dtype)
+        want = C.copy()
+        oracle.gemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 0.0, want, 0, M)
+        st, got = gpu.gemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 0.0, C, 0, M)
+        assert st == 0 and np.isfinite(got).all()
+        np.testing.assert_allclose(got, want, rtol=0, atol=4 * K * np.finfo(dtype).eps)
+        C1 = oracle.uniform(M * N, 3, dtype)
+        st, got = gpu.gemm(COL, NOTRANS, NOTRANS, M, N, K, 0.0, A, 0, M, B, 0, K, 1.0, C1, 0, M)
+        assert st == 0
+        np.testing.assert_array_equal(got, C1)
+        # K == 0: C <- beta * C (documented deviation from a reference bug); beta == 0 clears NaNs
+        st, got = gpu.gemm(COL, NOTRANS, NOTRANS, M, N, 0, 1.0, A, 0, M, B, 0, 1, 0.5, C1, 0, M)
+        assert st == 0
+        np.testing.assert_array_equal(got, (0.5 * C1).astype(dtype))
+        st, got = gpu.gemm(COL, NOTRANS, NOTRANS, M, N, 0, 1.0, A, 0, M, B, 0, 1, 0.0, C, 0, M)
+        assert st == 0 and (got == 0).all()
+
+
+EDGE_SHAPES = [(4097, 4095, 1031), (65536, 64, 4096), (64, 65536, 4096), (127, 129, 8192)]
+
+
+@pytest.mark.parametrize("M,N,K", EDGE_SHAPES)
+def test_config3_sgemm_edge_sweep(gpu, M, N, K):
+    """BASELINE config 3: alpha=0.7, beta=-1.3, all four transposes, ld = rows+3, offsets
+    5/7/11, uniform[-1,1).  Sampled elements (borders included) against the exact product;
+    everything outside the M x N window of C must be bit-identical to the input."""
+    dtype = np.float32
+    alpha, beta = 0.7, -1.3
+    offs = (5, 7, 11)
+    for tA, tB in itertools.product([NOTRANS, TRANS], [NOTRANS, TRANS]):
+        lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 3, offs)
+        A, B, C = oracle.uniform(na, 1, dtype), oracle.uniform(nb, 2, dtype), oracle.uniform(nc, 3, dtype)
+        st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc)
+        assert st == 0
+        _check_sampled(dtype, tA != NOTRANS, tB != NOTRANS, M, N, K, alpha, beta, A[offs[0]:], lda, B[offs[1]:], ldb,
+                       C[offs[2]:], got[offs[2]:], ldc)
+        mask = np.zeros(nc, dtype=bool)
+        logical_view(mask, COL, NOTRANS, M, N, offs[2], ldc)[:] = True
+        np.testing.assert_array_equal(got[~mask], C[~mask])
+        assert not np.array_equal(got[mask], C[mask])
+
+
+def _freivalds(torch, dA, dB, dC0, dC, tA, tB, n, alpha, beta):
+    """C v == alpha opA (opB v) + beta C0 v in fp64 on the device; returns the relative defect."""
+    v = torch.randn(n, dtype=torch.float64, device="cuda")
+    A = dA.view(n, n).T.double() if not tA else dA.view(n, n).double()
+    Bv = (dB.view(n, n).T.double() if not tB else dB.view(n, n).double()) @ v
+    rhs = alpha * (A @ Bv) + beta * (dC0.view(n, n).T.double() @ v)
+    lhs = dC.view(n, n).T.double() @ v
+    return float((lhs - rhs).abs().max() / rhs.abs().max())
+
+
+@pytest.mark.parametrize("cfg", ["config2_sgemm", "config4_dgemm"])
+def test_full_size_8192(gpu, cfg):
+    """BASELINE configs 2 and 4 at full size: sampled elements against the exact product, and
+    a size-independent linearity check C v = alpha A (B v) + beta C0 v."""
+    import torch
+    import clblas_amd
+    n = 8192
+    if cfg == "config2_sgemm":
+        dtype, tA, tB, alpha, beta = np.float32, NOTRANS, NOTRANS, 1.0, 1.0
+        A, B, C = (oracle.uniform(n * n, s, dtype) for s in (1, 2, 3))
+        fn = clblas_amd.sgemm
+    else:
+        dtype, tA, tB, alpha, beta = np.float64, NOTRANS, TRANS, 1.0, 0.5
+        A, B, C = (oracle.normal(n * n, s, dtype) for s in (1, 2, 3))
+        fn = clblas_amd.dgemm
+    dA, dB, dC0 = (torch.from_numpy(x).cuda() for x in (A, B, C))
+    dC = dC0.clone()
+    st = fn(COL, tA, tB, n, n, n, alpha, dA, 0, n, dB, 0, n, beta, dC, 0, n)
+    torch.cuda.synchronize()
+    assert st == 0
+    got = dC.cpu().numpy()
+    _check_sampled(dtype, tA != NOTRANS, tB != NOTRANS, n, n, n, alpha, beta, A, n, B, n, C, got, n, nsamp=6000)
+    defect = _freivalds(torch, dA, dB, dC0, dC, tA != NOTRANS, tB != NOTRANS, n, alpha, beta)
+    assert defect <= 64 * n * np.finfo(dtype).eps, defect
+
+
+def test_wide_leading_dimension_path(gpu):
+    """Leading dimensions beyond the 32-bit panel offsets take the plain 64-bit kernel."""
+    M, N, K = 4, 3, 5
+    lda = 3 * 1024 * 1024
+    A = oracle.integers(K * lda, 1, 10, np.float32)
+    B = oracle.integers(K * N, 2, 10, np.float32)
+    C = oracle.integers(M * N, 3, 10, np.float32)
+    want = C.copy()
+    oracle.gemm(COL, NOTRANS, NOTRANS, M, N, K, 2.0, A, 0, lda, B, 0, K, 3.0, want, 0, M)
+    st, got = gpu.gemm(COL, NOTRANS, NOTRANS, M, N, K, 2.0, A, 0, lda, B, 0, K, 3.0, C, 0, M)
+    assert st == 0
+    np.testing.assert_array_equal(got, want)

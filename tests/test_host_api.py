@@ -1,0 +1,109 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol the header declares,
+and its argument validation returns the same status as the oracle's restatement of the
+reference checks.  No kernel is launched here (every call fails validation first)."""
+import ctypes
+import itertools
+import os
+import re
+
+import pytest
+
+import clblas_amd
+import oracle
+from helpers import COL, ROW, NOTRANS, TRANS, CONJ, LEFT, RIGHT, UPPER, LOWER, UNIT, NONUNIT
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FAKE = 0x1000  # non-null "device pointer"; never dereferenced because validation fails first
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, "include", "clblas_amd.h")).read()
+    return sorted(set(re.findall(r"\b(clblas[A-Z]\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = clblas_amd.load_library()
+    syms = header_symbols()
+    assert set(syms) == set(clblas_amd.EXPORTED_SYMBOLS)
+    for s in syms:
+        assert hasattr(lib, s), s
+
+
+def test_header_compiles_as_c_and_cxx(tmp_path):
+    import subprocess
+    src = tmp_path / "t.c"
+    src.write_text('#include "clblas_amd.h"\nint main(void){return clblasSuccess + clblasColumnMajor - 1;}\n')
+    inc = os.path.join(ROOT, "include")
+    subprocess.check_call(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-I", inc, "-c", str(src), "-o",
+                           str(tmp_path / "t.o")])
+    subprocess.check_call(["g++", "-std=c++11", "-Wall", "-Werror", "-x", "c++", "-I", inc, "-c", str(src), "-o",
+                           str(tmp_path / "t2.o")])
+
+
+def test_version_and_status_values():
+    assert clblas_amd.get_version() == (0, 1, 0)
+    S = clblas_amd.Status
+    # numeric values of src/clBLAS.h:123-155
+    assert (S.NotImplemented, S.NotInitialized, S.InvalidMatA, S.InvalidMatB, S.InvalidMatC) == (-1024, -1023, -1022,
+                                                                                                 -1021, -1020)
+    assert (S.InvalidDim, S.InvalidLeadDimA, S.InvalidLeadDimB, S.InvalidLeadDimC) == (-1017, -1016, -1015, -1014)
+    assert (S.InsufficientMemMatA, S.InsufficientMemMatB, S.InsufficientMemMatC) == (-1011, -1010, -1009)
+    assert (clblas_amd.Order.RowMajor, clblas_amd.Order.ColumnMajor) == (0, 1)
+    assert (clblas_amd.Uplo.Upper, clblas_amd.Diag.Unit, clblas_amd.Side.Left) == (0, 0, 0)
+
+
+GEMM_BAD = []
+for order, tA, tB in itertools.product([ROW, COL], [NOTRANS, TRANS, CONJ], [NOTRANS, TRANS]):
+    for (M, N, K, lda, ldb, ldc) in [(0, 4, 4, 8, 8, 8), (4, 0, 4, 8, 8, 8), (5, 6, 7, 4, 9, 9), (5, 6, 7, 9, 5, 9),
+                                     (5, 6, 7, 9, 9, 4), (5, 6, 7, 4, 4, 4), (5, 6, 7, 6, 6, 5), (7, 5, 6, 6, 5, 6),
+                                     (0, 0, 0, 1, 1, 1), (3, 3, 0, 0, 0, 2)]:
+        GEMM_BAD.append((order, tA, tB, M, N, K, lda, ldb, ldc))
+
+
+@pytest.mark.parametrize("fn", ["sgemm", "dgemm"])
+def test_gemm_validation_matches_reference_checks(fn):
+    f = getattr(clblas_amd, fn)
+    hit = set()
+    for (order, tA, tB, M, N, K, lda, ldb, ldc) in GEMM_BAD:
+        want = oracle.check_gemm(order, tA, tB, M, N, K, 1, 0, lda, 0, 1, 0, ldb, 0, 1, 0, ldc, 0)
+        if want == 0:
+            continue  # valid arguments would launch; not for a CPU test
+        got = f(order, tA, tB, M, N, K, 1.0, FAKE, 0, lda, FAKE, 0, ldb, 0.0, FAKE, 0, ldc, stream=0)
+        assert got == want, (order, tA, tB, M, N, K, lda, ldb, ldc)
+        hit.add(want)
+    assert {-1017, -1016, -1015, -1014} <= hit
+    # null objects, in A, B, C order (src/tests/functional/func-error.cpp:58-104)
+    assert f(COL, 0, 0, 4, 4, 4, 1.0, None, 0, 4, None, 0, 4, 0.0, None, 0, 4, stream=0) == -1022
+    assert f(COL, 0, 0, 4, 4, 4, 1.0, FAKE, 0, 4, None, 0, 4, 0.0, None, 0, 4, stream=0) == -1021
+    assert f(COL, 0, 0, 4, 4, 4, 1.0, FAKE, 0, 4, FAKE, 0, 4, 0.0, None, 0, 4, stream=0) == -1020
+    # enum values outside the reference's enums
+    assert f(7, 0, 0, 4, 4, 4, 1.0, FAKE, 0, 4, FAKE, 0, 4, 0.0, FAKE, 0, 4, stream=0) == clblas_amd.Status.InvalidValue
+    assert f(COL, 3, 0, 4, 4, 4, 1.0, FAKE, 0, 4, FAKE, 0, 4, 0.0, FAKE, 0, 4, stream=0) == clblas_amd.Status.InvalidValue
+
+
+@pytest.mark.parametrize("fn", ["strsm", "dtrsm"])
+def test_trsm_validation_matches_reference_checks(fn):
+    f = getattr(clblas_amd, fn)
+    hit = set()
+    for order, side, tA in itertools.product([ROW, COL], [LEFT, RIGHT], [NOTRANS, TRANS]):
+        for (M, N, lda, ldb) in [(0, 4, 8, 8), (4, 0, 8, 8), (6, 4, 5, 8), (4, 6, 5, 8), (6, 4, 8, 3), (4, 6, 8, 3),
+                                 (6, 6, 5, 5)]:
+            want = oracle.check_trsm(order, side, tA, M, N, 1, 0, lda, 0, 1, 0, ldb, 0)
+            if want == 0:
+                continue
+            got = f(order, side, LOWER, tA, NONUNIT, M, N, 1.0, FAKE, 0, lda, FAKE, 0, ldb, stream=0)
+            assert got == want, (order, side, tA, M, N, lda, ldb)
+            hit.add(want)
+    assert {-1017, -1016, -1015} <= hit
+    assert f(COL, LEFT, LOWER, NOTRANS, NONUNIT, 4, 4, 1.0, None, 0, 4, None, 0, 4, stream=0) == -1022
+    assert f(COL, LEFT, LOWER, NOTRANS, NONUNIT, 4, 4, 1.0, FAKE, 0, 4, None, 0, 4, stream=0) == -1021
+    assert f(COL, 5, LOWER, NOTRANS, NONUNIT, 4, 4, 1.0, FAKE, 0, 4, FAKE, 0, 4, stream=0) == clblas_amd.Status.InvalidValue
+
+
+def test_product_package_does_not_touch_the_oracle():
+    pkg = os.path.join(ROOT, "clblas_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for fn in files:
+            if fn.endswith((".py", ".cpp", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, fn)).read()
+                assert "oracle" not in text.lower(), os.path.join(dirpath, fn)

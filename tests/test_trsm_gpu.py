@@ -1,0 +1,140 @@
+"""GPU parity tests for clblasStrsm / clblasDtrsm through the C ABI.
+
+The reference solves with explicit inverses of 128x128 diagonal blocks; this library solves
+the diagonal blocks by substitution.  The two are not bit-comparable, so parity is judged as
+the task states: normwise backward error
+    ||op(A) X - alpha B|| / (||A|| ||X|| + |alpha| ||B||) <= 2 n eps        (inf-norms)
+plus elementwise agreement with the oracle's restatement of the reference algorithm within
+a forward bound for these well-conditioned inputs, plus the reference tests' own devices:
+NaN-poisoned unused triangle / unit diagonal, closed-form Extratest, untouched padding."""
+import itertools
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import (COL, ROW, NOTRANS, TRANS, CONJ, UPPER, LOWER, UNIT, NONUNIT, LEFT, RIGHT, golden_cases,
+                     logical_view)
+
+pytestmark = pytest.mark.gpu
+
+DT = {"f32": np.float32, "f64": np.float64}
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import gpu_util
+    import torch
+    assert torch.cuda.is_available()
+    return gpu_util
+
+
+@pytest.mark.parametrize("name", ["sample_strsm_offsets", "extratest_f32", "extratest_f64"])
+def test_golden(gpu, name):
+    c = golden_cases()[name]
+    dt = DT[c["dtype"]]
+    A, B = np.array(c["A"], dtype=dt), np.array(c["B"], dtype=dt)
+    st, out = gpu.trsm(c["order"], c["side"], c["uplo"], c["transA"], c["diag"], c["M"], c["N"], c["alpha"], A,
+                       c["offA"], c["lda"], B, c["offB"], c["ldb"])
+    assert st == 0
+    tol = c.get("tol", 16 * np.finfo(dt).eps)   # Extratest: the reference's own 1e-5
+    np.testing.assert_allclose(out.astype(np.float64), np.array(c["expected"]), rtol=tol, atol=tol)
+
+
+def make_inputs(order, side, uplo, diag, M, N, dtype, seed, offA=5, offB=7):
+    n = M if side == LEFT else N
+    lda = n + 3
+    lower_in_memory = (uplo == LOWER) == (order == COL)
+    A = oracle.triangular(n, lda, lower_in_memory, seed, dtype, poison_diag=(diag == UNIT))
+    A = np.concatenate([np.full(offA, np.nan, dtype=dtype), A])
+    ib, ob = (M, N) if order == COL else (N, M)
+    ldb = ib + 2
+    B = oracle.uniform(offB + ob * ldb, seed + 1, dtype)
+    return A, lda, B, ldb
+
+
+def backward_error(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B0, X, offB, ldb):
+    n = M if side == LEFT else N
+    Am = np.nan_to_num(logical_view(A, order, NOTRANS, n, n, offA, lda).astype(np.float64))
+    Am = np.triu(Am) if uplo == UPPER else np.tril(Am)
+    if diag == UNIT:
+        np.fill_diagonal(Am, 1.0)
+    if tA != NOTRANS:
+        Am = Am.T
+    Xm = logical_view(X, order, NOTRANS, M, N, offB, ldb).astype(np.float64)
+    Bm = logical_view(B0, order, NOTRANS, M, N, offB, ldb).astype(np.float64)
+    R = (Am @ Xm if side == LEFT else Xm @ Am) - alpha * Bm
+    nrm = lambda Z: np.abs(Z).sum(axis=1).max()
+    return nrm(R) / (nrm(Am) * nrm(Xm) + abs(alpha) * nrm(Bm))
+
+
+VARIANTS = list(itertools.product([LEFT, RIGHT], [UPPER, LOWER], [NOTRANS, TRANS], [UNIT, NONUNIT]))
+SIZES = [(1, 1), (5, 3), (37, 29), (130, 17), (23, 300), (257, 64), (300, 520)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("order", [ROW, COL])
+@pytest.mark.parametrize("side,uplo,tA,diag", VARIANTS)
+def test_all_variants(gpu, dtype, order, side, uplo, tA, diag):
+    eps = np.finfo(dtype).eps
+    for (M, N) in SIZES:
+        alpha = 0.75
+        A, lda, B, ldb = make_inputs(order, side, uplo, diag, M, N, dtype, 11)
+        want = B.copy()
+        assert oracle.trsm_blocked(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, want, 7, ldb) == 0
+        st, got = gpu.trsm(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, B, 7, ldb)
+        assert st == 0
+        n = M if side == LEFT else N
+        Xg = logical_view(got, order, NOTRANS, M, N, 7, ldb)
+        assert not np.isnan(Xg).any(), "poisoned triangle or unit diagonal was read (%d,%d)" % (M, N)
+        be = backward_error(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, B, got, 7, ldb)
+        assert be <= 2 * n * eps, ((M, N), be)
+        Xw = logical_view(want, order, NOTRANS, M, N, 7, ldb)
+        scale = np.abs(Xw).max()
+        assert np.abs(Xg - Xw).max() <= 32 * n * eps * scale, (M, N)
+        mask = np.ones(B.size, dtype=bool)
+        logical_view(mask, order, NOTRANS, M, N, 7, ldb)[:] = False
+        np.testing.assert_array_equal(got[mask], B[mask])
+
+
+def test_conjtrans_is_trans_and_alpha_zero(gpu):
+    M, N = 70, 33
+    A, lda, B, ldb = make_inputs(COL, LEFT, LOWER, NONUNIT, M, N, np.float64, 3)
+    st, x1 = gpu.trsm(COL, LEFT, LOWER, TRANS, NONUNIT, M, N, 1.0, A, 5, lda, B, 7, ldb)
+    st2, x2 = gpu.trsm(COL, LEFT, LOWER, CONJ, NONUNIT, M, N, 1.0, A, 5, lda, B, 7, ldb)
+    assert st == 0 and st2 == 0
+    np.testing.assert_array_equal(x1, x2)
+    st, x0 = gpu.trsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, M, N, 0.0, A, 5, lda, B, 7, ldb)
+    assert st == 0
+    assert (logical_view(x0, COL, NOTRANS, M, N, 7, ldb) == 0).all()
+
+
+def test_config5_dtrsm_8192(gpu):
+    """BASELINE config 5 at full size: Left/Lower/NoTrans/NonUnit, M=N=8192, alpha=1.
+    (a) backward error on sampled right-hand sides, computed in fp64 on the host;
+    (b) size-independent: the leading 1024 rows of X solve the leading 1024x1024 system, so
+        they must agree with the oracle's solve of that sub-problem."""
+    import torch
+    import clblas_amd
+    n = 8192
+    A = oracle.triangular(n, n, True, 21, np.float64)
+    B = oracle.normal(n * n, 22, np.float64)
+    dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    st = clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, dA, 0, n, dB, 0, n)
+    torch.cuda.synchronize()
+    assert st == 0
+    X = dB.cpu().numpy().reshape(n, n).T        # X[r, c]
+    assert np.isfinite(X).all()
+    L = np.tril(np.nan_to_num(A.reshape(n, n).T))
+    B0 = B.reshape(n, n).T
+    cols = np.r_[0, 1, 63, 64, 4095, 4096, 8190, 8191, np.random.default_rng(0).integers(0, n, 24)]
+    R = L @ X[:, cols] - B0[:, cols]
+    nrm_L = np.abs(L).sum(axis=1).max()
+    be = np.abs(R).max(axis=0) / (nrm_L * np.abs(X[:, cols]).max(axis=0) + np.abs(B0[:, cols]).max(axis=0))
+    assert be.max() <= 2 * n * np.finfo(np.float64).eps, be.max()
+    k, nc = 1024, 96
+    sub = np.ascontiguousarray(B0[:k, :nc].T).ravel()            # column-major k x nc
+    Asub = np.ascontiguousarray(A.reshape(n, n)[:k, :k]).ravel()  # columns 0..k-1, rows 0..k-1, ld k
+    assert oracle.trsm_blocked(COL, LEFT, LOWER, NOTRANS, NONUNIT, k, nc, 1.0, Asub, 0, k, sub, 0, k) == 0
+    want = sub.reshape(nc, k).T
+    assert np.abs(X[:k, :nc] - want).max() <= 32 * k * np.finfo(np.float64).eps * np.abs(want).max()
