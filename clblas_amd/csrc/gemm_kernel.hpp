@@ -71,7 +71,7 @@ template <> struct Mma<double> {
         return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
     }
     static __device__ __forceinline__ int row(int v, int lane) {
-        return 4 * (lane >> 4) + v;
+        return (lane >> 4) + 4 * v;
     }
 };
 
