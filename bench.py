@@ -58,7 +58,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm or dtrsm (profiling)")
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, or copy (profiling; copy = a plain "
+                    "1 GiB device copy used to scale the HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (one MI355X per box); use --gpus 1")
@@ -77,6 +78,14 @@ def main():
     gen.manual_seed(1234)
     extra = {}
     result = None
+
+    if args.only == "copy":
+        src = torch.rand(1 << 28, device="cuda", dtype=torch.float32, generator=gen)  # 1 GiB
+        dst = torch.empty_like(src)
+        wall, ev_ms = timed_calls(torch, lambda: dst.copy_(src), steps, warmup)
+        print(json.dumps({"metric": "plain device copy, 1 GiB read + 1 GiB written per launch", "launch_ms": ev_ms,
+                          "GBps": round(2 * 2 ** 30 / (ev_ms * 1e-3) / 1e9, 1)}))
+        return
 
     # ---- SGEMM, BASELINE config 2 -------------------------------------------------------
     if args.only in ("", "sgemm"):
@@ -163,7 +172,7 @@ def main():
     if not args.no_cpu and args.only == "":
         import numpy as np
         import oracle
-        m_s, n_s, k_s = 2048, 1024, n     # same K (same per-element work) on a block of C
+        m_s, n_s, k_s = n, n // 2, n      # same K (same per-element work) on half of the columns of C
         a = oracle.uniform(m_s * k_s, 1, np.float32)
         b = oracle.uniform(k_s * n_s, 2, np.float32)
         c = oracle.uniform(m_s * n_s, 3, np.float32)
