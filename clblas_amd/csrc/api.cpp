@@ -26,12 +26,6 @@ int forced_gemm_tile() {
     return std::atoi(s);
 }
 
-int forced_trsm_nb() {
-    const char *s = std::getenv("CLBLAS_AMD_TRSM_NB");
-    if (!s || !*s) return 0;
-    return std::atoi(s);
-}
-
 namespace {
 struct WsSlot {
     void *ptr = nullptr;

@@ -12,9 +12,6 @@ namespace cba {
 // from the environment variable CLBLAS_AMD_GEMM_TILE, or -1.
 int forced_gemm_tile();
 
-// Debug-only override of the TRSM leaf block size (CLBLAS_AMD_TRSM_NB), or 0.
-int forced_trsm_nb();
-
 // Library-owned device scratch for `stream` on the current device, at least `bytes` long.
 // Grown on demand; earlier, smaller buffers stay alive until clblasTeardown so that work
 // already enqueued on them remains valid.  Returns nullptr if the allocation fails.

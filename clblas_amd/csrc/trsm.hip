@@ -5,9 +5,10 @@
 // for STRSM, the legacy block solver (src/library/blas/gens/trsm.c:1213-1456).  The
 // reference inverts every 128x128 diagonal block (trtri kernels) and then alternates
 // "X_i = inv(A_ii) B_i" with a trailing DGEMM update, using an M x N temporary.  Here the
-// diagonal blocks are solved directly by substitution (one wavefront lane per right-hand
-// side, the block's triangle broadcast from LDS), the sweep is recursive so that almost all
-// flops land in large-K GEMM updates, and B is solved in place without a temporary.
+// diagonal blocks (128 x 128) are solved directly by substitution inside one kernel (eight
+// wavefronts, one lane per right-hand side, the block's triangle broadcast from LDS), the
+// sweep is recursive so that almost all flops land in large-K GEMM updates, and B is solved
+// in place without a temporary.
 // The block sweep directions are those of xtrsm.cc:1226-1477; alpha is applied exactly once
 // to every element of B (xtrsm.cc:1236-1240).
 //
@@ -20,102 +21,238 @@
 
 namespace cba {
 
-// Solves one diagonal block against every right-hand side it touches.
+// Solves one diagonal block (up to 128 x 128) against 64 right-hand sides per workgroup.
 //
-// The block is the nb x nb (nb <= NBL) triangle at A(i0,i0).  "Equation order" p = 0..nb-1
-// walks the block forward (index p) or backward (index nb-1-p) so that equation p only
-// involves unknowns q < p.  coef(p,q) is the factor of unknown q in equation p:
-//   left :  op(A)(ip, iq)        right:  op(A)(iq, ip)
-// so with teff = trans XOR right it is A[ip + iq*lda] (teff false) or A[iq + ip*lda].
-// Right-hand side j (a column of B for side=left, a row of B for side=right) has its
-// element r at B[(i0+r)*sr + j*sj].
-template <typename T, int NBL, bool RIGHT, bool FORWARD>
-__global__ void __launch_bounds__(64)
+// The block is the nb x nb (nb <= NB) triangle at A(i0,i0).  "Equation order" P = 0..nb-1
+// walks the block forward (index P) or backward (index nb-1-P) so that equation P only
+// involves unknowns Q < P.  coef(P,Q) is the factor of unknown Q in equation P:
+//   left :  op(A)(iP, iQ)        right:  op(A)(iQ, iP)
+// so with teff = trans XOR right it is A[iP + iQ*lda] (teff false) or A[iQ + iP*lda].
+// Right-hand side j is a column of B for side=left (element r at B[r + j*ldb]) and a row
+// of B for side=right (element r at B[j + r*ldb]).
+//
+// Work split: 8 wavefronts, wavefront w owns equations [16w, 16w+16) and keeps them in
+// registers, one lane per right-hand side.  Step s: wavefront s finishes its 16 unknowns
+// by substitution (each new unknown is folded into the remaining equations at once, so
+// the FMAs of one step are independent) and publishes them through LDS; after the
+// barrier every later wavefront subtracts the 16 x 16 coupling block times those unknowns.
+// The triangle sits in LDS as 36 blocks of 16 x 16, read as wave-uniform broadcasts one
+// column ahead of the FMAs that use them.
+// Only the referenced triangle of A is read (never the other one, nor a unit diagonal).
+// For side=left a right-hand side is a column of B, so giving each lane "its" column
+// directly would make every load touch 64 different columns; the panel is instead moved
+// between HBM and registers through an LDS staging area with lanes running along the
+// contiguous direction (the area reuses the triangle's LDS before and after the solve).
+template <typename T> struct TrsmLeaf {
+    static constexpr int NB = 128, IB = 16, NBLK = NB / IB, CW = 64, THREADS = 64 * NBLK;
+    static constexpr int EP = IB + 16 / (int)sizeof(T);   // column pitch of an E block: columns stay 16-byte aligned
+    static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;  // blocks (bi,bj), bi >= bj, at bi*(bi+1)/2 + bj
+    static constexpr int E_ELEMS = N_EBLK * IB * EP;
+    static constexpr int X_ELEMS = 2 * IB * CW;
+    static constexpr int SP = NB + 2;                     // pitch of the right-hand-side staging area
+    static constexpr int S_ELEMS = CW * SP;               // shares LDS with E (used before and after it)
+    static_assert(S_ELEMS <= E_ELEMS + X_ELEMS, "staging area must fit in the E/X region");
+    static constexpr size_t SMEM = (size_t)(E_ELEMS + X_ELEMS + NB) * sizeof(T);
+};
+
+// IB values of one E-block column (16-byte LDS reads; the address is wave-uniform).
+template <typename T, int IB> static __device__ __forceinline__ void load_e_column(const T *src, T (&dst)[IB]) {
+    constexpr int V = 16 / (int)sizeof(T);
+    typedef T VT __attribute__((ext_vector_type(V)));
+#pragma unroll
+    for (int p = 0; p < IB; p += V) {
+        VT v = *reinterpret_cast<const VT *>(src + p);
+#pragma unroll
+        for (int e = 0; e < V; ++e) dst[p + e] = v[e];
+    }
+}
+
+template <typename T, bool RIGHT, bool FORWARD>
+__global__ void __launch_bounds__(TrsmLeaf<T>::THREADS)
 trsm_diag_kernel(const T *__restrict__ Ablk, int64_t lda, bool teff, bool unit, int nb, T alpha,
                  T *__restrict__ Bblk, int64_t ldb, int nrhs) {
-    __shared__ __attribute__((aligned(16))) T E[NBL * NBL];
-    __shared__ T Dinv[NBL];
-    constexpr int TP = NBL + 2;  // pitch of the transposed right-hand-side staging (left side)
-    __shared__ __attribute__((aligned(16))) T stage[RIGHT ? 1 : 64 * TP];
+    typedef TrsmLeaf<T> L;
+    constexpr int IB = L::IB, CW = L::CW, EP = L::EP, NT = L::THREADS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    T *E = reinterpret_cast<T *>(smem_raw);
+    T *X = E + L::E_ELEMS;
+    T *Dinv = X + L::X_ELEMS;
 
-    const int lane = threadIdx.x;
-    // ---- triangle into LDS in equation order; only the referenced triangle is read ----
-    for (int e = lane; e < NBL * NBL; e += 64) {
-        // Make the index that is contiguous in memory vary fastest across lanes.
-        int p, q;
-        if (teff != !FORWARD) { q = e % NBL; p = e / NBL; } else { p = e % NBL; q = e / NBL; }
-        T val = (T)0;
-        if (q < p && p < nb) {
-            int ip = FORWARD ? p : nb - 1 - p, iq = FORWARD ? q : nb - 1 - q;
-            val = teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+
+    const int64_t j0 = (int64_t)blockIdx.x * CW;
+    const int64_t j = j0 + lane;
+    const bool col_ok = j < nrhs;
+    T y[IB];
+
+    // ---- this wavefront's 16 equations of right-hand side j into registers ----
+    if (RIGHT) {
+#pragma unroll
+        for (int p = 0; p < IB; ++p) {
+            const int P = wave * IB + p;
+            const int r = FORWARD ? P : nb - 1 - P;
+            T v = (T)0;
+            if (P < nb && col_ok) v = Bblk[j + (int64_t)r * ldb];
+            y[p] = alpha * v;
         }
-        E[p * NBL + q] = val;
+    } else {
+        T *S = E;  // staging area, overwritten by the triangle afterwards
+        // All loads are issued before the first LDS write so that their latencies overlap.
+        constexpr int NLD = CW * (L::NB / 2) / NT;
+        T v0[NLD], v1[NLD];
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            const int e = tid + u * NT;
+            const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
+            v0[u] = (T)0;
+            v1[u] = (T)0;
+            if (j0 + c < nrhs) {
+                const T *src = Bblk + r + (j0 + c) * ldb;
+                if (r < nb) v0[u] = src[0];
+                if (r + 1 < nb) v1[u] = src[1];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            const int e = tid + u * NT;
+            const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
+            S[c * L::SP + r] = v0[u];
+            S[c * L::SP + r + 1] = v1[u];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < IB; ++p) {
+            const int P = wave * IB + p;
+            const int r = FORWARD ? P : (nb - 1 - P < 0 ? 0 : nb - 1 - P);
+            y[p] = (P < nb) ? alpha * S[lane * L::SP + r] : (T)0;
+        }
+        __syncthreads();
     }
-    if (lane < NBL) {
+
+    // ---- triangle into LDS, block by block, in equation order (loads batched) ----
+    constexpr int E_ITERS = L::N_EBLK * IB * IB / NT, E_BATCH = 6;
+    static_assert(L::N_EBLK * IB * IB % NT == 0 && E_ITERS % E_BATCH == 0, "triangle fill must divide into batches");
+#pragma unroll 1
+    for (int it = 0; it < E_ITERS; it += E_BATCH) {
+        T val[E_BATCH];
+        int dst[E_BATCH];
+#pragma unroll
+        for (int u = 0; u < E_BATCH; ++u) {
+            const int e = tid + (it + u) * NT;
+            const int blk = e / (IB * IB), w = e % (IB * IB);
+            int bi = 0;
+            while ((bi + 1) * (bi + 2) / 2 <= blk) ++bi;
+            const int bj = blk - bi * (bi + 1) / 2;
+            // Let the index that is contiguous in memory vary fastest across lanes.
+            int p, q;
+            if (teff) { q = w % IB; p = w / IB; } else { p = w % IB; q = w / IB; }
+            const int P = bi * IB + p, Q = bj * IB + q;
+            val[u] = (T)0;
+            if (Q < P && P < nb) {
+                const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
+                val[u] = teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
+            }
+            dst[u] = blk * (IB * EP) + q * EP + p;
+        }
+#pragma unroll
+        for (int u = 0; u < E_BATCH; ++u) E[dst[u]] = val[u];
+    }
+    if (tid < L::NB) {
         T d = (T)1;
-        if (!unit && lane < nb) {
-            int ip = FORWARD ? lane : nb - 1 - lane;
+        if (!unit && tid < nb) {
+            const int ip = FORWARD ? tid : nb - 1 - tid;
             d = (T)1 / Ablk[ip + (int64_t)ip * lda];
         }
-        Dinv[lane] = d;
+        Dinv[tid] = d;
     }
+    __syncthreads();
 
-    const int64_t j0 = (int64_t)blockIdx.x * 64;
-    const int64_t j = j0 + lane;
-    T x[NBL];
+#pragma unroll 1
+    for (int s = 0; s < L::NBLK; ++s) {
+        T *Xs = X + (s & 1) * (IB * CW);
+        if (wave == s) {
+            const T *Ed = E + (s * (s + 1) / 2 + s) * (IB * EP);
+            T dinv[IB];
+            load_e_column<T, IB>(Dinv + s * IB, dinv);
+            T ea[IB], eb[IB];
+            load_e_column<T, IB>(Ed, ea);
+#pragma unroll
+            for (int q = 0; q < IB; q += 2) {
+                load_e_column<T, IB>(Ed + (q + 1) * EP, eb);
+                __builtin_amdgcn_sched_barrier(0);
+                {
+                    const T x = y[q] * dinv[q];
+                    y[q] = x;
+                    Xs[q * CW + lane] = x;
+#pragma unroll
+                    for (int p = q + 1; p < IB; ++p) y[p] = fma(-ea[p], x, y[p]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if (q + 2 < IB) load_e_column<T, IB>(Ed + (q + 2) * EP, ea);
+                __builtin_amdgcn_sched_barrier(0);
+                {
+                    const T x = y[q + 1] * dinv[q + 1];
+                    y[q + 1] = x;
+                    Xs[(q + 1) * CW + lane] = x;
+#pragma unroll
+                    for (int p = q + 2; p < IB; ++p) y[p] = fma(-eb[p], x, y[p]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        __syncthreads();
+        if (wave > s && wave * IB < nb) {
+            const T *Eo = E + (wave * (wave + 1) / 2 + s) * (IB * EP);
+            T xs[IB];
+#pragma unroll
+            for (int q = 0; q < IB; ++q) xs[q] = Xs[q * CW + lane];
+            T ea[IB], eb[IB];
+            load_e_column<T, IB>(Eo, ea);
+#pragma unroll
+            for (int q = 0; q < IB; q += 2) {
+                load_e_column<T, IB>(Eo + (q + 1) * EP, eb);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int p = 0; p < IB; ++p) y[p] = fma(-ea[p], xs[q], y[p]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (q + 2 < IB) load_e_column<T, IB>(Eo + (q + 2) * EP, ea);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int p = 0; p < IB; ++p) y[p] = fma(-eb[p], xs[q + 1], y[p]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    }
 
     if (RIGHT) {
-        // element r of rhs j: Bblk[j + r*ldb]; lanes run along j: coalesced.
 #pragma unroll
-        for (int p = 0; p < NBL; ++p) {
-            int r = FORWARD ? p : nb - 1 - p;
-            x[p] = (p < nb && j < nrhs) ? Bblk[j + (int64_t)r * ldb] : (T)0;
-        }
-        __syncthreads();
-    } else {
-        // element r of rhs j: Bblk[r + j*ldb]; contiguous along r, so go through LDS:
-        // lanes read runs along r, then each lane picks up its own column.
-        for (int e = lane; e < 64 * NBL; e += 64) {
-            int r = e % NBL, c = e / NBL;
-            T v = (T)0;
-            if (r < nb && j0 + c < nrhs) v = Bblk[r + (j0 + c) * ldb];
-            stage[c * TP + r] = v;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int p = 0; p < NBL; ++p) {
-            // p >= nb are padding equations (x = 0); clamp the index, the value is unused.
-            int r = FORWARD ? p : (nb - 1 - p < 0 ? 0 : nb - 1 - p);
-            x[p] = (p < nb) ? stage[lane * TP + r] : (T)0;
-        }
-    }
-
-    // ---- substitution, all in registers; E and Dinv are wave-uniform LDS broadcasts ----
-#pragma unroll
-    for (int p = 0; p < NBL; ++p) {
-        T acc = alpha * x[p];
-#pragma unroll
-        for (int q = 0; q < p; ++q) acc = fma(-E[p * NBL + q], x[q], acc);
-        x[p] = acc * Dinv[p];
-    }
-
-    if (RIGHT) {
-#pragma unroll
-        for (int p = 0; p < NBL; ++p) {
-            int r = FORWARD ? p : nb - 1 - p;
-            if (p < nb && j < nrhs) Bblk[j + (int64_t)r * ldb] = x[p];
+        for (int p = 0; p < IB; ++p) {
+            const int P = wave * IB + p;
+            const int r = FORWARD ? P : nb - 1 - P;
+            if (P < nb && col_ok) Bblk[j + (int64_t)r * ldb] = y[p];
         }
     } else {
-        __syncthreads();
+        T *S = E;
+        __syncthreads();  // every wavefront is done with the triangle
 #pragma unroll
-        for (int p = 0; p < NBL; ++p) {
-            int r = FORWARD ? p : (nb - 1 - p < 0 ? 0 : nb - 1 - p);
-            if (p < nb) stage[lane * TP + r] = x[p];
+        for (int p = 0; p < IB; ++p) {
+            const int P = wave * IB + p;
+            const int r = FORWARD ? P : (nb - 1 - P < 0 ? 0 : nb - 1 - P);
+            if (P < nb) S[lane * L::SP + r] = y[p];
         }
         __syncthreads();
-        for (int e = lane; e < 64 * NBL; e += 64) {
-            int r = e % NBL, c = e / NBL;
-            if (r < nb && j0 + c < nrhs) Bblk[r + (j0 + c) * ldb] = stage[c * TP + r];
+        constexpr int NLD = CW * (L::NB / 2) / NT;
+#pragma unroll
+        for (int u = 0; u < NLD; ++u) {
+            const int e = tid + u * NT;
+            const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
+            if (j0 + c < nrhs) {
+                T *dst = Bblk + r + (j0 + c) * ldb;
+                if (r < nb) dst[0] = S[c * L::SP + r];
+                if (r + 1 < nb) dst[1] = S[c * L::SP + r + 1];
+            }
         }
     }
 }
@@ -134,7 +271,8 @@ template <> struct GemmOf<double> {
     }
 };
 
-template <typename T, int NBL> struct TrsmDriver {
+template <typename T> struct TrsmDriver {
+    static constexpr int NBL = TrsmLeaf<T>::NB;
     bool right, trans, unit, forward, teff;
     int M, N;
     const T *A;
@@ -147,22 +285,16 @@ template <typename T, int NBL> struct TrsmDriver {
         const T *Ablk = A + i0 + (int64_t)i0 * lda;
         const int nrhs = right ? M : N;
         T *Bblk = right ? B + (int64_t)i0 * ldb : B + i0;
-        dim3 grid((unsigned)((nrhs + 63) / 64)), block(64);
-        if (right) {
-            if (forward)
-                hipLaunchKernelGGL((trsm_diag_kernel<T, NBL, true, true>), grid, block, 0, stream, Ablk, lda, teff,
-                                   unit, nb, alpha, Bblk, ldb, nrhs);
-            else
-                hipLaunchKernelGGL((trsm_diag_kernel<T, NBL, true, false>), grid, block, 0, stream, Ablk, lda, teff,
-                                   unit, nb, alpha, Bblk, ldb, nrhs);
-        } else {
-            if (forward)
-                hipLaunchKernelGGL((trsm_diag_kernel<T, NBL, false, true>), grid, block, 0, stream, Ablk, lda, teff,
-                                   unit, nb, alpha, Bblk, ldb, nrhs);
-            else
-                hipLaunchKernelGGL((trsm_diag_kernel<T, NBL, false, false>), grid, block, 0, stream, Ablk, lda,
-                                   teff, unit, nb, alpha, Bblk, ldb, nrhs);
+        typedef TrsmLeaf<T> L;
+        void (*fn)(const T *, int64_t, bool, bool, int, T, T *, int64_t, int);
+        if (right) fn = forward ? trsm_diag_kernel<T, true, true> : trsm_diag_kernel<T, true, false>;
+        else fn = forward ? trsm_diag_kernel<T, false, true> : trsm_diag_kernel<T, false, false>;
+        if (L::SMEM > 64 * 1024) {
+            hipError_t e = ensure_dynamic_lds((const void *)fn, L::SMEM);
+            if (e != hipSuccess) return e;
         }
+        dim3 grid((unsigned)((nrhs + L::CW - 1) / L::CW)), block(L::THREADS);
+        hipLaunchKernelGGL(fn, grid, block, L::SMEM, stream, Ablk, lda, teff, unit, nb, alpha, Bblk, ldb, nrhs);
         return hipGetLastError();
     }
 
@@ -203,7 +335,7 @@ template <typename T, int NBL> struct TrsmDriver {
 template <typename T>
 static hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool unit, int M, int N, T alpha, const T *A,
                                 int64_t lda, T *B, int64_t ldb, hipStream_t stream) {
-    TrsmDriver<T, 32> d;
+    TrsmDriver<T> d;
     d.right = right; d.trans = trans; d.unit = unit;
     // Left: equations run forward when op(A) is lower triangular; right: when it is upper.
     d.forward = right ? (lower == trans) : (lower != trans);
