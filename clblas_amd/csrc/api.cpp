@@ -26,6 +26,12 @@ int forced_gemm_tile() {
     return std::atoi(s);
 }
 
+int debug_env_int(const char *name, int dflt) {
+    const char *s = std::getenv(name);
+    if (!s || !*s) return dflt;
+    return std::atoi(s);
+}
+
 namespace {
 struct WsSlot {
     void *ptr = nullptr;

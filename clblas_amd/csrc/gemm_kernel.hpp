@@ -85,6 +85,7 @@ template <typename T> struct GemmParams {
     T alpha, beta;
     int tiles_m, tiles_n;
     int group_m;      // tile rows walked together (L2 locality)
+    int xcd_remap;    // 1: give each XCD a contiguous chunk of the tile list
     int k_per_split;  // multiple of BK; >= K when the K loop is not split
     T *ws;            // split-K partial sums: ws[split * ws_slice + n * ws_ld + m]
     int64_t ws_ld, ws_slice;
@@ -202,7 +203,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         const int id = blockIdx.x;
         const int xcd = id & 7, q = id >> 3;
         const int per = nwg >> 3, rem = nwg & 7;
-        tile = xcd * per + (xcd < rem ? xcd : rem) + q;
+        tile = p.xcd_remap ? xcd * per + (xcd < rem ? xcd : rem) + q : id;
     }
     int tm, tn;
     {

@@ -112,7 +112,10 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     p.alpha = alpha; p.beta = beta;
     p.tiles_m = (int)ceil_div64(M, e.bm);
     p.tiles_n = (int)ceil_div64(N, e.bn);
-    p.group_m = p.tiles_m < 8 ? p.tiles_m : 8;
+    p.group_m = debug_env_int("CLBLAS_AMD_GEMM_GROUP_M", 4);
+    if (p.group_m > p.tiles_m) p.group_m = p.tiles_m;
+    if (p.group_m < 1) p.group_m = 1;
+    p.xcd_remap = debug_env_int("CLBLAS_AMD_GEMM_XCD", 1);
     p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
     p.k_per_split = K;
     const int idx = (tA ? 2 : 0) | (tB ? 1 : 0);

@@ -12,6 +12,9 @@ namespace cba {
 // from the environment variable CLBLAS_AMD_GEMM_TILE, or -1.
 int forced_gemm_tile();
 
+// Debug-only integer knob from the environment (tile walk order experiments), or `dflt`.
+int debug_env_int(const char *name, int dflt);
+
 // Library-owned device scratch for `stream` on the current device, at least `bytes` long.
 // Grown on demand; earlier, smaller buffers stay alive until clblasTeardown so that work
 // already enqueued on them remains valid.  Returns nullptr if the allocation fails.
