@@ -24,6 +24,13 @@ if ROOT not in sys.path:
 PEAK_FP32_MATRIX = 157.3  # TFLOP/s, MI355X dense MFMA
 PEAK_FP64_MATRIX = 78.6
 
+# HBM-side bytes per launch of the SGEMM 8192^3 kernel, from two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a plain 1 GiB
+# device copy (profiles/bench_8192_counters.md: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
+# Counters cannot be read from inside this process, so the figure is carried as a constant
+# and only reported when the workload is the one it was measured on.
+SGEMM_8192_TRAFFIC_BYTES = 8.67e9
+
 COL, NOTRANS, TRANS = 1, 0, 1
 LEFT, LOWER, NONUNIT = 0, 1, 1
 
@@ -111,7 +118,8 @@ def main():
             "config": {"workload": "BASELINE config 2: SGEMM column-major NN M=N=K=%d, tight ld, alpha=1, beta=1, "
                                    "uniform[-1,1)" % n},
             "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MATRIX,
-                         "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MATRIX, 4), "traffic": None,
+                         "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MATRIX, 4),
+                         "traffic": SGEMM_8192_TRAFFIC_BYTES if n == 8192 else None,
                          "kernel": "gemm_mfma_kernel<float,256,128,16,...> (one launch per call)",
                          "launch_ms": round(ev_ms, 4)},
         }
