@@ -28,6 +28,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace cba {
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -107,8 +109,8 @@ template <typename T, int BX, int BK, int NT, bool KC> struct PanelLoader {
     static_assert(NVEC % NT == 0 && PER >= 1, "panel does not divide over the workgroup");
     static constexpr int LDS_PITCH = BX + 4;
 
+    struct Regs { u32x4 v[PER]; };  // one panel's worth of data in flight
     uint32_t voff[PER];
-    u32x4 reg[PER];
 
     __device__ __forceinline__ void init(int tid, int64_t ld) {
 #pragma unroll
@@ -125,21 +127,21 @@ template <typename T, int BX, int BK, int NT, bool KC> struct PanelLoader {
     }
 
     // base: first element of the panel; bytes_left: footprint bytes from `base` on.
-    __device__ __forceinline__ void fetch(const T *base, int64_t bytes_left) {
+    __device__ __forceinline__ void fetch(const T *base, int64_t bytes_left, Regs &reg) const {
         __amdgpu_buffer_rsrc_t r = make_rsrc(base, bytes_left);
 #pragma unroll
-        for (int i = 0; i < PER; ++i) reg[i] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff[i], 0, 0);
+        for (int i = 0; i < PER; ++i) reg.v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff[i], 0, 0);
     }
 
     // k_valid: number of valid k rows in this panel (>= BK for a full panel).
-    __device__ __forceinline__ void store(T *lds, int tid, int k_valid) {
+    __device__ __forceinline__ void store(T *lds, int tid, int k_valid, const Regs &reg) const {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             int idx = tid + i * NT;
             if (KC) {
                 int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
                 union { u32x4 u; T e[VEC]; } cv;
-                cv.u = reg[i];
+                cv.u = reg.v[i];
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     // Past-K elements of a k-contiguous operand are real memory (the next
@@ -151,7 +153,7 @@ template <typename T, int BX, int BK, int NT, bool KC> struct PanelLoader {
                 int k = idx / (BX / VEC), x = (idx % (BX / VEC)) * VEC;
                 // Rows k >= K lie past the operand's footprint: the range check already
                 // returned zeros for them.
-                *reinterpret_cast<u32x4 *>(&lds[k * LDS_PITCH + x]) = reg[i];
+                *reinterpret_cast<u32x4 *>(&lds[k * LDS_PITCH + x]) = reg.v[i];
             }
         }
     }
@@ -243,66 +245,89 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             for (int v = 0; v < NACC; ++v) acc[bn][bm][v] = (T)0;
 
     if (n_panels > 0) {
-        {
-            const int64_t ao = a_off(k_begin), bo = b_off(k_begin);
-            la.fetch(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
-            lb.fetch(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
-            la.store(smem, tid, k_end - k_begin);
-            lb.store(smem + BK * PITCH_A, tid, k_end - k_begin);
-        }
+        // Software pipeline over panels.  Two register sets hold panels in flight from HBM:
+        // at the top of panel kp the loads of panel kp+2 are issued, in the middle of its
+        // MFMAs panel kp+1 (issued a whole panel earlier) is written into the idle LDS stage,
+        // and the single barrier at the end publishes it.
+        typename Cfg::LoaderA::Regs ra[2];
+        typename Cfg::LoaderB::Regs rb[2];
+        auto fetch_panel = [&](int kp, typename Cfg::LoaderA::Regs &xa, typename Cfg::LoaderB::Regs &xb) {
+            const int k0 = k_begin + kp * BK;
+            const int64_t ao = a_off(k0), bo = b_off(k0);
+            la.fetch(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T), xa);
+            lb.fetch(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T), xb);
+        };
+        auto store_panel = [&](int kp, const typename Cfg::LoaderA::Regs &xa, const typename Cfg::LoaderB::Regs &xb) {
+            T *dst = smem + (kp & 1) * STAGE;
+            const int k_valid = k_end - (k_begin + kp * BK);
+            la.store(dst, tid, k_valid, xa);
+            lb.store(dst + BK * PITCH_A, tid, k_valid, xb);
+        };
+
+        fetch_panel(0, ra[0], rb[0]);
+        if (n_panels > 1) fetch_panel(1, ra[1], rb[1]);
+        store_panel(0, ra[0], rb[0]);
         __syncthreads();
 
         const int a_frag = wm * WM + j * VM;
         const int b_frag = wn * WN + j * VN;
+        constexpr int STEPS = BK / KS;
+        constexpr int STORE_AT = STEPS / 2;  // MFMA step after which the next panel goes to LDS
 
-        for (int kp = 0; kp < n_panels; ++kp) {
-            const int cur = kp & 1;
-            const bool more = kp + 1 < n_panels;
-            const int k_next = k_begin + (kp + 1) * BK;
-            if (more) {
-                const int64_t ao = a_off(k_next), bo = b_off(k_next);
-                la.fetch(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
-                lb.fetch(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
-            }
+        // One panel: `par` is kp & 1, known at compile time so that the register sets are
+        // addressed statically.
+        auto do_panel = [&](int kp, auto par_tag) {
+            constexpr int PAR = decltype(par_tag)::value;
+            if (kp + 2 < n_panels) fetch_panel(kp + 2, ra[PAR], rb[PAR]);
 
-            const T *As = smem + cur * STAGE;
+            const T *As = smem + PAR * STAGE;
             const T *Bs = As + BK * PITCH_A;
-#pragma unroll
-            for (int s = 0; s < BK / KS; ++s) {
+            // Fragments for MFMA step s+1 are read from LDS while the MFMAs of step s run.
+            T a[2][TM], b[2][TN];
+            auto read_frags = [&](int s, T (&af)[TM], T (&bf)[TN]) {
                 const int krow = s * KS + g;
-                T a[TM], b[TN];
 #pragma unroll
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     typename Vec<T, VM>::type av =
                         *reinterpret_cast<const typename Vec<T, VM>::type *>(&As[krow * PITCH_A + a_frag + ga * MB * VM]);
-                    if constexpr (VM == 1) a[ga] = av;
+                    if constexpr (VM == 1) af[ga] = av;
                     else {
 #pragma unroll
-                        for (int e = 0; e < VM; ++e) a[ga * VM + e] = av[e];
+                        for (int e = 0; e < VM; ++e) af[ga * VM + e] = av[e];
                     }
                 }
 #pragma unroll
                 for (int gb = 0; gb < TN / VN; ++gb) {
                     typename Vec<T, VN>::type bv =
                         *reinterpret_cast<const typename Vec<T, VN>::type *>(&Bs[krow * PITCH_B + b_frag + gb * MB * VN]);
-                    if constexpr (VN == 1) b[gb] = bv;
+                    if constexpr (VN == 1) bf[gb] = bv;
                     else {
 #pragma unroll
-                        for (int e = 0; e < VN; ++e) b[gb * VN + e] = bv[e];
+                        for (int e = 0; e < VN; ++e) bf[gb * VN + e] = bv[e];
                     }
                 }
+            };
+            read_frags(0, a[0], b[0]);
+#pragma unroll
+            for (int s = 0; s < STEPS; ++s) {
+                if (s + 1 < STEPS) read_frags(s + 1, a[(s + 1) & 1], b[(s + 1) & 1]);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int bn = 0; bn < TN; ++bn)
 #pragma unroll
-                    for (int bm = 0; bm < TM; ++bm) acc[bn][bm] = M::run(b[bn], a[bm], acc[bn][bm]);
-            }
-
-            if (more) {
-                T *nxt = smem + (cur ^ 1) * STAGE;
-                la.store(nxt, tid, k_end - k_next);
-                lb.store(nxt + BK * PITCH_A, tid, k_end - k_next);
+                    for (int bm = 0; bm < TM; ++bm) acc[bn][bm] = M::run(b[s & 1][bn], a[s & 1][bm], acc[bn][bm]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (s + 1 == STORE_AT) {
+                    if (kp + 1 < n_panels) store_panel(kp + 1, ra[PAR ^ 1], rb[PAR ^ 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             __syncthreads();
+        };
+
+        for (int kp = 0; kp < n_panels; kp += 2) {
+            do_panel(kp, std::integral_constant<int, 0>());
+            if (kp + 1 < n_panels) do_panel(kp + 1, std::integral_constant<int, 1>());
         }
     }
 
