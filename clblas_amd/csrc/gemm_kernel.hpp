@@ -102,12 +102,16 @@ static __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p
 
 // Fetches one BX x BK operand panel.  KC == true: memory is contiguous along k
 // (element (x,k) at x*ld + k); KC == false: contiguous along x (element at k*ld + x).
-template <typename T, int BX, int BK, int NT, bool KC> struct PanelLoader {
+// KLAY selects the LDS layout: false: [k][x] (row pitch BX+4); true (only with KC): [x][k]
+// (row pitch BK + one 16-byte vector), written with one 16-byte store per loaded vector.
+template <typename T, int BX, int BK, int NT, bool KC, bool KLAY> struct PanelLoader {
+    static_assert(!KLAY || KC, "[x][k] layout is for k-contiguous operands");
     static constexpr int VEC = 16 / (int)sizeof(T);
     static constexpr int NVEC = BX * BK / VEC;
     static constexpr int PER = NVEC / NT;
     static_assert(NVEC % NT == 0 && PER >= 1, "panel does not divide over the workgroup");
-    static constexpr int LDS_PITCH = BX + 4;
+    static constexpr int LDS_PITCH = KLAY ? BK + VEC : BX + 4;
+    static constexpr int LDS_ELEMS = KLAY ? BX * LDS_PITCH : BK * LDS_PITCH;
 
     struct Regs { u32x4 v[PER]; };  // one panel's worth of data in flight
     uint32_t voff[PER];
@@ -142,12 +146,15 @@ template <typename T, int BX, int BK, int NT, bool KC> struct PanelLoader {
                 int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
                 union { u32x4 u; T e[VEC]; } cv;
                 cv.u = reg.v[i];
+                // Past-K elements of a k-contiguous operand are real memory (the next
+                // column), not out of range, so they are cleared here.
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    // Past-K elements of a k-contiguous operand are real memory (the next
-                    // column), not out of range, so they are cleared here.
-                    T val = (kv + e < k_valid) ? cv.e[e] : (T)0;
-                    lds[(kv + e) * LDS_PITCH + x] = val;
+                for (int e = 0; e < VEC; ++e) cv.e[e] = (kv + e < k_valid) ? cv.e[e] : (T)0;
+                if (KLAY) {
+                    *reinterpret_cast<u32x4 *>(&lds[x * LDS_PITCH + kv]) = cv.u;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) lds[(kv + e) * LDS_PITCH + x] = cv.e[e];
                 }
             } else {
                 int k = idx / (BX / VEC), x = (idx % (BX / VEC)) * VEC;
@@ -170,10 +177,20 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static constexpr int VN = TN < VEC ? TN : VEC;
     static_assert(BM % WM == 0 && BN % WN == 0 && WM % MB == 0 && WN % MB == 0, "tile shape");
     static_assert(TM % VM == 0 && TN % VN == 0 && BK % KS == 0, "tile shape");
-    typedef PanelLoader<T, BM, BK, NT, A_KC> LoaderA;
-    typedef PanelLoader<T, BN, BK, NT, B_KC> LoaderB;
+    // A k-contiguous B panel (transB == N) is kept as Bs[n][k]; a k-contiguous A panel is
+    // still transposed into As[k][m] so that C keeps its 16-byte row-interleaved stores.
+    static constexpr bool B_KLAY = B_KC;
+    static constexpr int VNM = B_KLAY ? 1 : VN;  // n interleave used by the fragment/epilogue mapping
+    static constexpr int NG = 64 / MB;           // lane groups along k
+    static_assert(BK % (VEC * NG) == 0, "panel depth must hold whole k groups");
+    typedef PanelLoader<T, BM, BK, NT, A_KC, false> LoaderA;
+    typedef PanelLoader<T, BN, BK, NT, B_KC, B_KLAY> LoaderB;
     static constexpr int PITCH_A = LoaderA::LDS_PITCH, PITCH_B = LoaderB::LDS_PITCH;
-    static constexpr int STAGE = BK * (PITCH_A + PITCH_B);  // elements per LDS stage
+    static constexpr int A_ELEMS = LoaderA::LDS_ELEMS;
+    static constexpr int STAGE = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;  // elements per LDS stage
+    // Panels in flight from HBM (register sets).  Two everywhere except FP64 with a [n][k] B
+    // panel, where the second set would push the kernel over 256 VGPRs.
+    static constexpr int DEPTH = (sizeof(T) == 8 && B_KLAY && TM * TN >= 16) ? 1 : 2;
     static constexpr size_t SMEM = 2 * (size_t)STAGE * sizeof(T);
 };
 
@@ -185,6 +202,8 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     constexpr int MB = Cfg::MB, KS = Cfg::KS, NACC = Cfg::NACC;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, VM = Cfg::VM, VN = Cfg::VN;
     constexpr int PITCH_A = Cfg::PITCH_A, PITCH_B = Cfg::PITCH_B, STAGE = Cfg::STAGE;
+    constexpr int VEC = Cfg::VEC, NG = Cfg::NG, A_ELEMS = Cfg::A_ELEMS, VNM = Cfg::VNM;
+    constexpr bool B_KLAY = Cfg::B_KLAY;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *smem = reinterpret_cast<T *>(smem_raw);
@@ -245,12 +264,14 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             for (int v = 0; v < NACC; ++v) acc[bn][bm][v] = (T)0;
 
     if (n_panels > 0) {
-        // Software pipeline over panels.  Two register sets hold panels in flight from HBM:
-        // at the top of panel kp the loads of panel kp+2 are issued, in the middle of its
-        // MFMAs panel kp+1 (issued a whole panel earlier) is written into the idle LDS stage,
-        // and the single barrier at the end publishes it.
-        typename Cfg::LoaderA::Regs ra[2];
-        typename Cfg::LoaderB::Regs rb[2];
+        // Software pipeline over panels.  DEPTH register sets hold panels in flight from HBM.
+        // DEPTH 2: at the top of panel kp the loads of panel kp+2 are issued, in the middle of
+        // its MFMAs panel kp+1 (issued a whole panel earlier) is written into the idle LDS
+        // stage, and the single barrier at the end publishes it.  DEPTH 1: panel kp+1 is
+        // requested at the top of panel kp and written after its last MFMA.
+        constexpr int DEPTH = Cfg::DEPTH;
+        typename Cfg::LoaderA::Regs ra[DEPTH];
+        typename Cfg::LoaderB::Regs rb[DEPTH];
         auto fetch_panel = [&](int kp, typename Cfg::LoaderA::Regs &xa, typename Cfg::LoaderB::Regs &xb) {
             const int k0 = k_begin + kp * BK;
             const int64_t ao = a_off(k0), bo = b_off(k0);
@@ -261,31 +282,40 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             T *dst = smem + (kp & 1) * STAGE;
             const int k_valid = k_end - (k_begin + kp * BK);
             la.store(dst, tid, k_valid, xa);
-            lb.store(dst + BK * PITCH_A, tid, k_valid, xb);
+            lb.store(dst + A_ELEMS, tid, k_valid, xb);
         };
 
         fetch_panel(0, ra[0], rb[0]);
-        if (n_panels > 1) fetch_panel(1, ra[1], rb[1]);
+        if (DEPTH == 2 && n_panels > 1) fetch_panel(1, ra[DEPTH - 1], rb[DEPTH - 1]);
         store_panel(0, ra[0], rb[0]);
         __syncthreads();
 
         const int a_frag = wm * WM + j * VM;
         const int b_frag = wn * WN + j * VN;
         constexpr int STEPS = BK / KS;
-        constexpr int STORE_AT = STEPS / 2;  // MFMA step after which the next panel goes to LDS
+        // MFMA step after which the next panel goes to LDS: mid-way when it was requested a
+        // whole panel earlier, at the end when it was requested at the top of this panel.
+        constexpr int STORE_AT = DEPTH == 2 ? STEPS / 2 : STEPS;
 
         // One panel: `par` is kp & 1, known at compile time so that the register sets are
         // addressed statically.
         auto do_panel = [&](int kp, auto par_tag) {
             constexpr int PAR = decltype(par_tag)::value;
-            if (kp + 2 < n_panels) fetch_panel(kp + 2, ra[PAR], rb[PAR]);
+            constexpr int R_IN = DEPTH == 2 ? PAR : 0;       // set receiving the new loads
+            constexpr int R_OUT = DEPTH == 2 ? PAR ^ 1 : 0;  // set written to LDS during this panel
+            if (kp + DEPTH < n_panels) fetch_panel(kp + DEPTH, ra[R_IN], rb[R_IN]);
 
             const T *As = smem + PAR * STAGE;
-            const T *Bs = As + BK * PITCH_A;
-            // Fragments for MFMA step s+1 are read from LDS while the MFMAs of step s run.
-            T a[2][TM], b[2][TN];
-            auto read_frags = [&](int s, T (&af)[TM], T (&bf)[TN]) {
-                const int krow = s * KS + g;
+            const T *Bs = As + A_ELEMS;
+            // MFMA step s of a panel consumes, in lane group g, the k index
+            //   kmap(s,g) = (s / VEC) * VEC * NG + g * VEC + s % VEC,
+            // i.e. VEC consecutive steps walk VEC consecutive k: a k-major panel row is read
+            // per step, a [n][k] panel is read as one 16-byte vector per VEC steps.
+            // Fragments are read one step (one VEC-step group for [n][k]) ahead of their use.
+            T a[2][TM], b[2][TN], bk[2][TN][VEC];
+            auto kmap = [&](int s) { return (s / VEC) * (VEC * NG) + g * VEC + (s % VEC); };
+            auto read_a = [&](int s, T (&af)[TM]) {
+                const int krow = kmap(s);
 #pragma unroll
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     typename Vec<T, VM>::type av =
@@ -296,6 +326,9 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                         for (int e = 0; e < VM; ++e) af[ga * VM + e] = av[e];
                     }
                 }
+            };
+            auto read_b = [&](int s, T (&bf)[TN]) {  // k-major B panel
+                const int krow = kmap(s);
 #pragma unroll
                 for (int gb = 0; gb < TN / VN; ++gb) {
                     typename Vec<T, VN>::type bv =
@@ -307,18 +340,37 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     }
                 }
             };
-            read_frags(0, a[0], b[0]);
+            auto read_bk = [&](int grp, T (&bf)[TN][VEC]) {  // [n][k] B panel, VEC steps at once
+#pragma unroll
+                for (int bn = 0; bn < TN; ++bn) {
+                    typename Vec<T, VEC>::type bv = *reinterpret_cast<const typename Vec<T, VEC>::type *>(
+                        &Bs[(wn * WN + bn * MB + j) * PITCH_B + grp * (VEC * NG) + g * VEC]);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) bf[bn][e] = bv[e];
+                }
+            };
+            read_a(0, a[0]);
+            if constexpr (B_KLAY) read_bk(0, bk[0]); else read_b(0, b[0]);
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
-                if (s + 1 < STEPS) read_frags(s + 1, a[(s + 1) & 1], b[(s + 1) & 1]);
+                if (s + 1 < STEPS) {
+                    read_a(s + 1, a[(s + 1) & 1]);
+                    if constexpr (B_KLAY) {
+                        if ((s + 1) % VEC == 0) read_bk((s + 1) / VEC, bk[((s + 1) / VEC) & 1]);
+                    } else {
+                        read_b(s + 1, b[(s + 1) & 1]);
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int bn = 0; bn < TN; ++bn)
+                for (int bn = 0; bn < TN; ++bn) {
+                    const T bval = B_KLAY ? bk[(s / VEC) & 1][bn][s % VEC] : b[s & 1][bn];
 #pragma unroll
-                    for (int bm = 0; bm < TM; ++bm) acc[bn][bm] = M::run(b[s & 1][bn], a[s & 1][bm], acc[bn][bm]);
+                    for (int bm = 0; bm < TM; ++bm) acc[bn][bm] = M::run(bval, a[s & 1][bm], acc[bn][bm]);
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 if (s + 1 == STORE_AT) {
-                    if (kp + 1 < n_panels) store_panel(kp + 1, ra[PAR ^ 1], rb[PAR ^ 1]);
+                    if (kp + 1 < n_panels) store_panel(kp + 1, ra[R_OUT], rb[R_OUT]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -347,7 +399,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     for (int bn = 0; bn < TN; ++bn) {
 #pragma unroll
         for (int v = 0; v < NACC; ++v) {
-            const int n = n0 + wn * WN + (bn / VN) * (MB * VN) + M::row(v, lane) * VN + (bn % VN);
+            const int n = n0 + wn * WN + (bn / VNM) * (MB * VNM) + M::row(v, lane) * VNM + (bn % VNM);
             if (n >= p.N) continue;
             T *col = Cout + (int64_t)n * ldc;
 #pragma unroll

@@ -13,7 +13,8 @@ namespace cba {
 
 template <typename T> struct TileEntry {
     int bm, bn, bk, threads;
-    size_t smem;
+    size_t smem;     // largest of the four variants (for the residency estimate)
+    size_t smem_of[4];
     bool has_splitk;
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
     void (*plain[4])(const GemmParams<T>);
@@ -22,9 +23,16 @@ template <typename T> struct TileEntry {
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK>
 TileEntry<T> make_tile_entry() {
-    typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;  // smem / threads do not depend on transposes
+    typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
-    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.smem = Cfg::SMEM; e.has_splitk = WITH_SPLITK;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK;
+    // LDS need depends on the layout of the B panel (transB): index as plain[].
+    e.smem_of[0] = GemmCfg<T, BM, BN, BK, WM, WN, false, true>::SMEM;
+    e.smem_of[1] = GemmCfg<T, BM, BN, BK, WM, WN, false, false>::SMEM;
+    e.smem_of[2] = GemmCfg<T, BM, BN, BK, WM, WN, true, true>::SMEM;
+    e.smem_of[3] = GemmCfg<T, BM, BN, BK, WM, WN, true, false>::SMEM;
+    e.smem = e.smem_of[0];
+    for (int i = 1; i < 4; ++i) e.smem = e.smem_of[i] > e.smem ? e.smem_of[i] : e.smem;
     // A is k-contiguous when transposed; B is k-contiguous when NOT transposed.
     e.plain[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, false, MINW>;   // NN
     e.plain[1] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, false, false, MINW>;  // NT
@@ -136,11 +144,12 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             fn = e.splitk[idx];
         }
     }
-    if (e.smem > 64 * 1024) {
-        hipError_t err = ensure_dynamic_lds((const void *)fn, e.smem);
+    const size_t smem = e.smem_of[idx];
+    if (smem > 64 * 1024) {
+        hipError_t err = ensure_dynamic_lds((const void *)fn, smem);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)splits), dim3(e.threads), e.smem, stream, p);
+    hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)splits), dim3(e.threads), smem, stream, p);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
     if (splits > 1) {
