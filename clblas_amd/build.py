@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libclblas_amd.so")
+CLIENT_PATH = os.path.join(HERE, "client", "clblas_amd-client")
 
 SOURCES = ["api.cpp", "gemm_f32.hip", "gemm_f64.hip", "trsm.hip"]
 
@@ -50,7 +51,20 @@ def build_library(verbose=True):
         raise RuntimeError("link failed: %s\n%s" % (" ".join(cmd), res.stderr))
     if verbose:
         print("built", LIB_PATH)
+    build_client(verbose)
     return LIB_PATH
+
+
+def build_client(verbose=True):
+    """Benchmark command line (CSV in the schema of the reference's published results)."""
+    cmd = [_hipcc()] + COMMON_FLAGS + [os.path.join(HERE, "client", "client.cpp"), "-o", CLIENT_PATH,
+                                      "-L" + HERE, "-lclblas_amd", "-Wl,-rpath,$ORIGIN/.."]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("client build failed: %s\n%s" % (" ".join(cmd), res.stderr))
+    if verbose:
+        print("built", CLIENT_PATH)
+    return CLIENT_PATH
 
 
 if __name__ == "__main__":
