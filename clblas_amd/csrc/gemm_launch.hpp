@@ -16,16 +16,17 @@ template <typename T> struct TileEntry {
     size_t smem;     // largest of the four variants (for the residency estimate)
     size_t smem_of[4];
     bool has_splitk;
+    double eff;      // measured fraction of MFMA peak on large problems (tile choice model)
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
     void (*plain[4])(const GemmParams<T>);
     void (*splitk[4])(const GemmParams<T>);
 };
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK>
-TileEntry<T> make_tile_entry() {
+TileEntry<T> make_tile_entry(double eff) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
-    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
     e.smem_of[0] = GemmCfg<T, BM, BN, BK, WM, WN, false, true>::SMEM;
     e.smem_of[1] = GemmCfg<T, BM, BN, BK, WM, WN, false, false>::SMEM;
@@ -52,9 +53,13 @@ TileEntry<T> make_tile_entry() {
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Chooses tile and split count.  The reference keys its choice on M*N brackets and
-// divisibility (AutoGemmParameters.py:8-55); here remainders are handled in-kernel, so
-// the only question is how to fill 256 CUs: the largest tile that still yields enough
-// workgroups, and a K split when even the smallest tile cannot.
+// divisibility (AutoGemmParameters.py:8-55); here remainders are handled in-kernel, so the
+// question is only how well a tile shape fills 256 CUs.  Workgroups that share a CU share
+// its MFMA pipes, so time is quantised per CU, not per resident workgroup:
+//     time ~ ceil(tiles / 256) * BM * BN / eff
+// with eff the measured MFMA efficiency of that tile shape on large problems (padding is
+// paid for automatically because whole tiles are counted).  The smallest tile adds a K
+// split when even it cannot give every CU a workgroup.
 template <typename T>
 static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, int *tile_out,
                         int *splits_out) {
@@ -63,12 +68,11 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
     if (force >= 0 && force < ntab) {
         pick = force;
     } else {
+        double best = 0;
         for (int i = 0; i < ntab; ++i) {
-            int64_t t = ceil_div64(M, tab[i].bm) * ceil_div64(N, tab[i].bn);
-            // Work actually computed vs. useful work: avoid tiles that are mostly padding.
-            double useful = ((double)M * N) / ((double)t * tab[i].bm * tab[i].bn);
-            int64_t resident = (tab[i].smem * 2 <= 160 * 1024 && tab[i].threads <= 256) ? 2 : 1;
-            if (t >= kCUs * resident && useful >= 0.80) { pick = i; break; }
+            const int64_t t = ceil_div64(M, tab[i].bm) * ceil_div64(N, tab[i].bn);
+            const double cost = (double)ceil_div64(t, kCUs) * tab[i].bm * tab[i].bn / tab[i].eff;
+            if (i == 0 || cost < best) { best = cost; pick = i; }
         }
     }
     int splits = 1;

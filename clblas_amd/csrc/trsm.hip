@@ -87,6 +87,43 @@ trsm_diag_kernel(const T *__restrict__ Ablk, int64_t lda, bool teff, bool unit, 
     const bool col_ok = j < nrhs;
     T y[IB];
 
+    // ---- triangle: issue its loads first so that they overlap the right-hand-side traffic.
+    //      Element e of the (block, q, p) enumeration; only the referenced triangle is read. ----
+    constexpr int E_ITERS = L::N_EBLK * IB * IB / NT;
+    static_assert(L::N_EBLK * IB * IB % NT == 0, "triangle fill must divide over the workgroup");
+    auto e_coords = [&](int u, int &blk, int &p, int &q) {
+        const int e = tid + u * NT;
+        blk = e / (IB * IB);
+        const int w = e % (IB * IB);
+        // Let the index that is contiguous in memory vary fastest across lanes.
+        if (teff) { q = w % IB; p = w / IB; } else { p = w % IB; q = w / IB; }
+    };
+    auto e_slot = [&](int u) {
+        int blk, p, q;
+        e_coords(u, blk, p, q);
+        return blk * (IB * EP) + q * EP + p;
+    };
+    T eval[E_ITERS];
+#pragma unroll
+    for (int u = 0; u < E_ITERS; ++u) {
+        int blk, p, q;
+        e_coords(u, blk, p, q);
+        int bi = 0;
+        while ((bi + 1) * (bi + 2) / 2 <= blk) ++bi;
+        const int bj = blk - bi * (bi + 1) / 2;
+        const int P = bi * IB + p, Q = bj * IB + q;
+        eval[u] = (T)0;
+        if (Q < P && P < nb) {
+            const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
+            eval[u] = teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
+        }
+    }
+    T dval = (T)1;
+    if (tid < L::NB && !unit && tid < nb) {
+        const int ip = FORWARD ? tid : nb - 1 - tid;
+        dval = Ablk[ip + (int64_t)ip * lda];
+    }
+
     // ---- this wavefront's 16 equations of right-hand side j into registers ----
     if (RIGHT) {
 #pragma unroll
@@ -131,42 +168,10 @@ trsm_diag_kernel(const T *__restrict__ Ablk, int64_t lda, bool teff, bool unit, 
         __syncthreads();
     }
 
-    // ---- triangle into LDS, block by block, in equation order (loads batched) ----
-    constexpr int E_ITERS = L::N_EBLK * IB * IB / NT, E_BATCH = 6;
-    static_assert(L::N_EBLK * IB * IB % NT == 0 && E_ITERS % E_BATCH == 0, "triangle fill must divide into batches");
-#pragma unroll 1
-    for (int it = 0; it < E_ITERS; it += E_BATCH) {
-        T val[E_BATCH];
-        int dst[E_BATCH];
+    // ---- triangle into LDS (its loads were issued first, see above) ----
 #pragma unroll
-        for (int u = 0; u < E_BATCH; ++u) {
-            const int e = tid + (it + u) * NT;
-            const int blk = e / (IB * IB), w = e % (IB * IB);
-            int bi = 0;
-            while ((bi + 1) * (bi + 2) / 2 <= blk) ++bi;
-            const int bj = blk - bi * (bi + 1) / 2;
-            // Let the index that is contiguous in memory vary fastest across lanes.
-            int p, q;
-            if (teff) { q = w % IB; p = w / IB; } else { p = w % IB; q = w / IB; }
-            const int P = bi * IB + p, Q = bj * IB + q;
-            val[u] = (T)0;
-            if (Q < P && P < nb) {
-                const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
-                val[u] = teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
-            }
-            dst[u] = blk * (IB * EP) + q * EP + p;
-        }
-#pragma unroll
-        for (int u = 0; u < E_BATCH; ++u) E[dst[u]] = val[u];
-    }
-    if (tid < L::NB) {
-        T d = (T)1;
-        if (!unit && tid < nb) {
-            const int ip = FORWARD ? tid : nb - 1 - tid;
-            d = (T)1 / Ablk[ip + (int64_t)ip * lda];
-        }
-        Dinv[tid] = d;
-    }
+    for (int u = 0; u < E_ITERS; ++u) E[e_slot(u)] = eval[u];
+    if (tid < L::NB) Dinv[tid] = (T)1 / dval;
     __syncthreads();
 
 #pragma unroll 1
