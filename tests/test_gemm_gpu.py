@@ -209,3 +209,52 @@ def test_wide_leading_dimension_path(gpu):
     st, got = gpu.gemm(COL, NOTRANS, NOTRANS, M, N, K, 2.0, A, 0, lda, B, 0, K, 3.0, C, 0, M)
     assert st == 0
     np.testing.assert_array_equal(got, want)
+
+
+def test_padding_of_inputs_is_never_used(gpu):
+    """Everything outside the logical windows of A and B (leading-dimension padding, offsets,
+    tails) is NaN: tile remainders in M, N and K must neither fault nor leak into C."""
+    for dtype in (np.float32, np.float64):
+        for (M, N, K) in [(70, 45, 37), (257, 130, 19), (33, 300, 130)]:
+            for order, tA, tB in itertools.product([ROW, COL], [NOTRANS, TRANS], [NOTRANS, TRANS]):
+                offs = (9, 3, 6)
+                lda, ldb, ldc, na, nb, nc = _layout(order, tA, tB, M, N, K, 5, offs)
+                A = np.full(na + 7, np.nan, dtype=dtype)
+                B = np.full(nb + 7, np.nan, dtype=dtype)
+                logical_view(A, order, tA, M, K, offs[0], lda)[:] = oracle.integers(M * K, 1, 9, dtype).reshape(M, K)
+                logical_view(B, order, tB, K, N, offs[1], ldb)[:] = oracle.integers(K * N, 2, 9, dtype).reshape(K, N)
+                C = oracle.integers(nc, 3, 9, dtype)
+                want = C.copy()
+                assert oracle.gemm(order, tA, tB, M, N, K, 2.0, A, offs[0], lda, B, offs[1], ldb, 1.0, want, offs[2],
+                                   ldc) == 0
+                st, got = gpu.gemm(order, tA, tB, M, N, K, 2.0, A, offs[0], lda, B, offs[1], ldb, 1.0, C, offs[2], ldc)
+                assert st == 0
+                np.testing.assert_array_equal(got, want, err_msg=str((dtype, M, N, K, order, tA, tB)))
+
+
+def test_two_streams_and_teardown(gpu):
+    """Calls on different streams are independent (each has its own split-K scratch), and the
+    library keeps working after clblasTeardown released that scratch."""
+    import torch
+    import clblas_amd
+    M, N, K = 100, 90, 4096            # few tiles, deep K: takes the split-K path
+    la, lc = exact_int_limits(K, 1.0, 1.0, np.float32)
+    A1, B1, C1 = (oracle.integers(n, s, la, np.float32) for n, s in ((M * K, 1), (K * N, 2), (M * N, 3)))
+    A2, B2, C2 = (oracle.integers(n, s, la, np.float32) for n, s in ((M * K, 4), (K * N, 5), (M * N, 6)))
+    w1, w2 = C1.copy(), C2.copy()
+    oracle.gemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A1, 0, M, B1, 0, K, 1.0, w1, 0, M)
+    oracle.gemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A2, 0, M, B2, 0, K, 1.0, w2, 0, M)
+    for rep in range(2):
+        d = [torch.from_numpy(x).cuda() for x in (A1, B1, C1, A2, B2, C2)]
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        torch.cuda.synchronize()
+        for _ in range(1):
+            assert clblas_amd.sgemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, d[0], 0, M, d[1], 0, K, 1.0, d[2], 0, M,
+                                    stream=s1) == 0
+            assert clblas_amd.sgemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, d[3], 0, M, d[4], 0, K, 1.0, d[5], 0, M,
+                                    stream=s2) == 0
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(d[2].cpu().numpy(), w1)
+        np.testing.assert_array_equal(d[5].cpu().numpy(), w2)
+        clblas_amd.teardown()          # second pass runs after the scratch was released
+    assert clblas_amd.setup() == 0
