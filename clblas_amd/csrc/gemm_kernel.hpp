@@ -7,20 +7,24 @@
 // alpha/beta applied once in the epilogue, beta == 0 never reads C.
 //
 // Structure of one workgroup (BM x BN macro tile of C, waves arranged WAVES_M x WAVES_N):
-//   * A and B panels of depth BK are fetched with 16-byte raw buffer loads into registers
-//     while the MFMAs of the previous panel run, then written to one of two LDS stages
-//     (double buffering, one barrier per panel).  Buffer descriptors are re-based every
-//     panel and sized to the exact footprint of the operand, so the hardware range check
-//     turns every access past the end of the matrix into a zero: no extra launch and no
-//     per-element branch is needed for M/N/K remainders.
-//   * LDS always holds the panels "k-major": As[k][m], Bs[k][n].  Operands whose
-//     contiguous direction in memory is k (transA == T, transB == N) are transposed on the
-//     way into LDS; a row pitch of tile+4 elements makes both the transposing scalar
-//     writes and the 16-byte fragment reads bank-conflict free.
+//   * Panels of depth BK travel HBM -> LDS without passing through registers wherever the
+//     LDS image is a plain copy of memory: `buffer_load_dwordx4 ... lds` writes each wave's
+//     64 x 16 bytes to consecutive LDS addresses.  That covers operands contiguous along the
+//     tile edge (As[k][m], Bs[k][n]) and a k-contiguous B panel, kept as Bs[n][k] with its
+//     16-byte slots XOR-swizzled by the row so that fragment reads stay bank-conflict free.
+//     Only a k-contiguous A panel (transA == T) is still staged through registers and
+//     transposed into As[k][m] (pitch BM+4), so that C keeps its 16-byte row stores.
+//   * NSTAGE LDS stages form a ring; the loads of panel p+NSTAGE-1 are issued at the top of
+//     panel p and one barrier per panel publishes the next stage.  Buffer descriptors are
+//     re-based every panel and sized to the exact footprint of the operand, so the hardware
+//     range check turns every access past the end of the matrix into a zero (also on the
+//     LDS path): no extra launch and no per-element branch is needed for M/N remainders or
+//     for the K remainder of tile-edge-contiguous operands; the K remainder of a
+//     k-contiguous panel is real memory and is cleared in LDS before it is used.
 //   * Each wave owns a WM x WN sub-tile as TM x TN MFMA blocks
 //     (v_mfma_f32_32x32x2_f32 / v_mfma_f64_16x16x4_f64).  The MFMA "B" operand carries the
 //     A matrix and the "A" operand carries the B matrix, so that the lane index of the
-//     result runs along m, the contiguous direction of C.  The m (and n) coordinates are
+//     result runs along m, the contiguous direction of C.  The m coordinates are
 //     interleaved between blocks so that one 16-byte LDS read feeds VM blocks and one
 //     16-byte global store writes VM consecutive rows of C.
 #pragma once
@@ -100,68 +104,112 @@ static __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)n, 0x00020000);
 }
 
-// Fetches one BX x BK operand panel.  KC == true: memory is contiguous along k
-// (element (x,k) at x*ld + k); KC == false: contiguous along x (element at k*ld + x).
-// KLAY selects the LDS layout: false: [k][x] (row pitch BX+4); true (only with KC): [x][k]
-// (row pitch BK + one 16-byte vector), written with one 16-byte store per loaded vector.
-template <typename T, int BX, int BK, int NT, bool KC, bool KLAY> struct PanelLoader {
-    static_assert(!KLAY || KC, "[x][k] layout is for k-contiguous operands");
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// s_waitcnt immediate that waits for vmcnt <= n only (gfx9 encoding: vmcnt in bits 3:0 and
+// 15:14, expcnt 6:4, lgkmcnt 11:8; the other counters are left at "don't wait").
+#define CBA_VMCNT_ONLY(n) ((((n) & 0xf) | ((((n) >> 4) & 0x3) << 14) | (0x7 << 4) | (0xf << 8)))
+
+// How an operand panel gets from memory into LDS.
+//   LM_DMA_X: memory contiguous along the tile edge x; LDS image [k][x], pitch BX.
+//   LM_DMA_K: memory contiguous along k; LDS image [x][k], pitch BK, 16-byte slots of row x
+//             stored at slot ^ swz(x)  (B operand with transB == N).
+//   LM_REG_T: memory contiguous along k; staged through registers and transposed into
+//             [k][x], pitch BX+4 (A operand with transA == T).
+enum LoadMode { LM_DMA_X = 0, LM_DMA_K = 1, LM_REG_T = 2 };
+
+template <typename T, int BX, int BK, int NT, int MODE> struct PanelLoader {
     static constexpr int VEC = 16 / (int)sizeof(T);
     static constexpr int NVEC = BX * BK / VEC;
-    static constexpr int PER = NVEC / NT;
+    static constexpr int PER = NVEC / NT;  // 16-byte vectors per thread = wave-wide loads per wave
     static_assert(NVEC % NT == 0 && PER >= 1, "panel does not divide over the workgroup");
-    static constexpr int LDS_PITCH = KLAY ? BK + VEC : BX + 4;
-    static constexpr int LDS_ELEMS = KLAY ? BX * LDS_PITCH : BK * LDS_PITCH;
+    static constexpr int NW = NT / 64;
+    static constexpr int CHUNK = 64 * VEC;  // elements written by one wave-wide LDS load (1 KiB)
+    // LM_DMA_X: every 1 KiB chunk (CHUNK / BX rows of the [k][x] image) is followed by a small
+    // gap, sized so that the rows read together by the lane groups of one fragment read
+    // (VEC rows apart) start 64 bytes = 16 banks apart.
+    static constexpr int ROWS_PER_CHUNK = CHUNK / BX > 0 ? CHUNK / BX : 1;
+    static constexpr int CHUNKS_APART = VEC / ROWS_PER_CHUNK > 0 ? VEC / ROWS_PER_CHUNK : 1;
+    static constexpr int CHUNK_PAD = MODE == LM_DMA_X ? (64 / (int)sizeof(T)) / CHUNKS_APART : 0;  // elements
+    static constexpr int CHUNK_PITCH = CHUNK + CHUNK_PAD;
+    static constexpr int LDS_PITCH = MODE == LM_DMA_X ? BX : (MODE == LM_DMA_K ? BK : BX + 4);
+    static constexpr int LDS_ELEMS = MODE == LM_REG_T ? BK * LDS_PITCH : (NVEC / 64) * CHUNK_PITCH;
+    // LM_DMA_X: LDS element offset of image element (k, x).
+    static __device__ __forceinline__ int lds_at(int k, int x) {
+        const int e = k * BX + x;
+        return e + (e / CHUNK) * CHUNK_PAD;
+    }
+    static constexpr bool DMA = MODE != LM_REG_T;
+    // LM_DMA_K swizzle: S slots per row; rows x and x + 16/S start in the same bank.
+    static constexpr int S = BK / VEC;
+    static_assert(MODE != LM_DMA_K || (S <= 16 && 16 % S == 0), "swizzle needs S | 16");
+    static __device__ __forceinline__ int swz(int x) { return (x / (16 / S)) % S; }
 
-    struct Regs { u32x4 v[PER]; };  // one panel's worth of data in flight
+    struct Regs { u32x4 v[DMA ? 1 : PER]; };  // LM_REG_T: one panel's worth of data in flight
     uint32_t voff[PER];
 
     __device__ __forceinline__ void init(int tid, int64_t ld) {
+        const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            int idx = tid + i * NT;
-            if (KC) {
-                int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
-                voff[i] = (uint32_t)(((int64_t)x * ld + kv) * (int64_t)sizeof(T));
-            } else {
-                int k = idx / (BX / VEC), x = (idx % (BX / VEC)) * VEC;
+            if (MODE == LM_DMA_X) {
+                const int e = (wave + i * NW) * CHUNK + lane * VEC;  // element index in the [k][x] image
+                const int k = e / BX, x = e % BX;
                 voff[i] = (uint32_t)(((int64_t)k * ld + x) * (int64_t)sizeof(T));
+            } else if (MODE == LM_DMA_K) {
+                const int x = (wave + i * NW) * (64 / S) + lane / S;
+                const int slot = (lane % S) ^ swz(x);  // logical slot stored in this lane's place
+                voff[i] = (uint32_t)(((int64_t)x * ld + slot * VEC) * (int64_t)sizeof(T));
+            } else {
+                const int idx = tid + i * NT;
+                const int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
+                voff[i] = (uint32_t)(((int64_t)x * ld + kv) * (int64_t)sizeof(T));
             }
         }
     }
 
-    // base: first element of the panel; bytes_left: footprint bytes from `base` on.
-    __device__ __forceinline__ void fetch(const T *base, int64_t bytes_left, Regs &reg) const {
+    // Starts the transfer of one panel.  base: first element of the panel; bytes_left:
+    // footprint bytes from `base` on; lds: this operand's image in the receiving stage.
+    __device__ __forceinline__ void issue(const T *base, int64_t bytes_left, T *lds, int wave_u, Regs &reg) const {
         __amdgpu_buffer_rsrc_t r = make_rsrc(base, bytes_left);
 #pragma unroll
-        for (int i = 0; i < PER; ++i) reg.v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff[i], 0, 0);
+        for (int i = 0; i < PER; ++i) {
+            if (DMA) {
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH), 16,
+                                                         (int)voff[i], 0, 0, 0);
+            } else {
+                reg.v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff[i], 0, 0);
+            }
+        }
     }
 
-    // k_valid: number of valid k rows in this panel (>= BK for a full panel).
+    // LM_REG_T: registers -> LDS, transposing; elements past K are cleared (they are real
+    // memory - the next column - not out of range).
     __device__ __forceinline__ void store(T *lds, int tid, int k_valid, const Regs &reg) const {
+        if (DMA) return;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            int idx = tid + i * NT;
-            if (KC) {
-                int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
-                union { u32x4 u; T e[VEC]; } cv;
-                cv.u = reg.v[i];
-                // Past-K elements of a k-contiguous operand are real memory (the next
-                // column), not out of range, so they are cleared here.
+            const int idx = tid + i * NT;
+            const int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
+            union { u32x4 u; T e[VEC]; } cv;
+            cv.u = reg.v[i];
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) cv.e[e] = (kv + e < k_valid) ? cv.e[e] : (T)0;
-                if (KLAY) {
-                    *reinterpret_cast<u32x4 *>(&lds[x * LDS_PITCH + kv]) = cv.u;
-                } else {
+            for (int e = 0; e < VEC; ++e) lds[(kv + e) * LDS_PITCH + x] = (kv + e < k_valid) ? cv.e[e] : (T)0;
+        }
+    }
+
+    // LM_DMA_K: clears the elements past K of a partial panel, each thread in the 16 bytes
+    // its own loads delivered (call after waiting for those loads).
+    __device__ __forceinline__ void clear_k_tail(T *lds, int tid, int k_valid) const {
+        if (MODE != LM_DMA_K) return;
+        const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) lds[(kv + e) * LDS_PITCH + x] = cv.e[e];
-                }
-            } else {
-                int k = idx / (BX / VEC), x = (idx % (BX / VEC)) * VEC;
-                // Rows k >= K lie past the operand's footprint: the range check already
-                // returned zeros for them.
-                *reinterpret_cast<u32x4 *>(&lds[k * LDS_PITCH + x]) = reg.v[i];
-            }
+        for (int i = 0; i < PER; ++i) {
+            const int x = (wave + i * NW) * (64 / S) + lane / S;
+            const int place = lane % S, slot = place ^ swz(x);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                if (slot * VEC + e >= k_valid) lds[x * BK + place * VEC + e] = (T)0;
         }
     }
 };
@@ -178,20 +226,21 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static_assert(BM % WM == 0 && BN % WN == 0 && WM % MB == 0 && WN % MB == 0, "tile shape");
     static_assert(TM % VM == 0 && TN % VN == 0 && BK % KS == 0, "tile shape");
     // A k-contiguous B panel (transB == N) is kept as Bs[n][k]; a k-contiguous A panel is
-    // still transposed into As[k][m] so that C keeps its 16-byte row-interleaved stores.
+    // transposed into As[k][m] so that C keeps its 16-byte row-interleaved stores.
     static constexpr bool B_KLAY = B_KC;
     static constexpr int VNM = B_KLAY ? 1 : VN;  // n interleave used by the fragment/epilogue mapping
     static constexpr int NG = 64 / MB;           // lane groups along k
     static_assert(BK % (VEC * NG) == 0, "panel depth must hold whole k groups");
-    typedef PanelLoader<T, BM, BK, NT, A_KC, false> LoaderA;
-    typedef PanelLoader<T, BN, BK, NT, B_KC, B_KLAY> LoaderB;
+    typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_REG_T : LM_DMA_X> LoaderA;
+    typedef PanelLoader<T, BN, BK, NT, B_KC ? LM_DMA_K : LM_DMA_X> LoaderB;
     static constexpr int PITCH_A = LoaderA::LDS_PITCH, PITCH_B = LoaderB::LDS_PITCH;
     static constexpr int A_ELEMS = LoaderA::LDS_ELEMS;
     static constexpr int STAGE = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;  // elements per LDS stage
-    // Panels in flight from HBM (register sets).  Two everywhere except FP64 with a [n][k] B
-    // panel, where the second set would push the kernel over 256 VGPRs.
-    static constexpr int DEPTH = (sizeof(T) == 8 && B_KLAY && TM * TN >= 16) ? 1 : 2;
-    static constexpr size_t SMEM = 2 * (size_t)STAGE * sizeof(T);
+    // Three stages (loads two panels ahead) when two workgroups of them still share a CU's
+    // 160 KiB, otherwise two (loads one panel ahead).
+    static constexpr int NSTAGE = (2 * 3 * STAGE * (int)sizeof(T) <= 150 * 1024) ? 3 : 2;
+    static constexpr int DEPTH = NSTAGE - 1;
+    static constexpr size_t SMEM = (size_t)NSTAGE * STAGE * sizeof(T);
 };
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, bool SPLITK, int MINW>
@@ -203,6 +252,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, VM = Cfg::VM, VN = Cfg::VN;
     constexpr int PITCH_A = Cfg::PITCH_A, PITCH_B = Cfg::PITCH_B, STAGE = Cfg::STAGE;
     constexpr int VEC = Cfg::VEC, NG = Cfg::NG, A_ELEMS = Cfg::A_ELEMS, VNM = Cfg::VNM;
+    constexpr int NSTAGE = Cfg::NSTAGE, DEPTH = Cfg::DEPTH;
     constexpr bool B_KLAY = Cfg::B_KLAY;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -211,6 +261,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // same value, known to be wave-uniform
     const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
     const int j = lane % MB;  // position along the block edge
     const int g = lane / MB;  // k sub-step supplied by this lane
@@ -264,37 +315,48 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             for (int v = 0; v < NACC; ++v) acc[bn][bm][v] = (T)0;
 
     if (n_panels > 0) {
-        // Software pipeline over panels.  DEPTH register sets hold panels in flight from HBM.
-        // DEPTH 2: at the top of panel kp the loads of panel kp+2 are issued, in the middle of
-        // its MFMAs panel kp+1 (issued a whole panel earlier) is written into the idle LDS
-        // stage, and the single barrier at the end publishes it.  DEPTH 1: panel kp+1 is
-        // requested at the top of panel kp and written after its last MFMA.
-        constexpr int DEPTH = Cfg::DEPTH;
-        typename Cfg::LoaderA::Regs ra[DEPTH];
-        typename Cfg::LoaderB::Regs rb[DEPTH];
-        auto fetch_panel = [&](int kp, typename Cfg::LoaderA::Regs &xa, typename Cfg::LoaderB::Regs &xb) {
+        // Software pipeline over panels: a ring of NSTAGE LDS stages, loads issued DEPTH =
+        // NSTAGE-1 panels ahead.  Panel kp lives in stage kp % NSTAGE.  The loads of panel
+        // kp+DEPTH go out at the top of panel kp into the stage whose last readers finished
+        // before the barrier that ended panel kp-1.  Before the barrier that ends panel kp,
+        // each wave waits for its own loads of panel kp+1 (issued a panel earlier when
+        // DEPTH is 2); the register-staged operand is written into that stage mid-way.
+        typedef typename Cfg::LoaderA LA;
+        typedef typename Cfg::LoaderB LB;
+        constexpr int RSETS = DEPTH;  // register sets of a staged operand
+        typename LA::Regs ra[RSETS];
+        typename LB::Regs rb[RSETS];
+        constexpr int LOADS_PER_PANEL = LA::PER + LB::PER;  // vector-memory instructions per wave and panel
+
+        auto stage_ptr = [&](int kp) -> T * { return smem + (kp % NSTAGE) * STAGE; };
+        auto issue_panel = [&](int kp, typename LA::Regs &xa, typename LB::Regs &xb) {
             const int k0 = k_begin + kp * BK;
             const int64_t ao = a_off(k0), bo = b_off(k0);
-            la.fetch(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T), xa);
-            lb.fetch(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T), xb);
+            T *dst = stage_ptr(kp);
+            la.issue(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T), dst, wave_u, xa);
+            lb.issue(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T), dst + A_ELEMS, wave_u, xb);
         };
-        auto store_panel = [&](int kp, const typename Cfg::LoaderA::Regs &xa, const typename Cfg::LoaderB::Regs &xb) {
-            T *dst = smem + (kp & 1) * STAGE;
+        // Makes panel kp (already requested) readable by the whole workgroup: own loads
+        // complete, staged registers written, K tail cleared, barrier.
+        auto publish_panel = [&](int kp, bool newer_in_flight, const typename LA::Regs &xa, bool store_a) {
+            T *dst = stage_ptr(kp);
             const int k_valid = k_end - (k_begin + kp * BK);
-            la.store(dst, tid, k_valid, xa);
-            lb.store(dst + A_ELEMS, tid, k_valid, xb);
+            if (store_a) la.store(dst, tid, k_valid, xa);
+            if (newer_in_flight) __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(LOADS_PER_PANEL));
+            else __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0));
+            if (k_valid < BK) lb.clear_k_tail(dst + A_ELEMS, tid, k_valid);
+            __syncthreads();
         };
 
-        fetch_panel(0, ra[0], rb[0]);
-        if (DEPTH == 2 && n_panels > 1) fetch_panel(1, ra[DEPTH - 1], rb[DEPTH - 1]);
-        store_panel(0, ra[0], rb[0]);
-        __syncthreads();
+        issue_panel(0, ra[0], rb[0]);
+        if (DEPTH == 2 && n_panels > 1) issue_panel(1, ra[RSETS - 1], rb[RSETS - 1]);
+        publish_panel(0, DEPTH == 2 && n_panels > 1, ra[0], true);
 
         const int a_frag = wm * WM + j * VM;
         const int b_frag = wn * WN + j * VN;
         constexpr int STEPS = BK / KS;
-        // MFMA step after which the next panel goes to LDS: mid-way when it was requested a
-        // whole panel earlier, at the end when it was requested at the top of this panel.
+        // MFMA step after which a register-staged A panel goes to LDS: mid-way when it was
+        // requested a whole panel earlier, after the last step otherwise.
         constexpr int STORE_AT = DEPTH == 2 ? STEPS / 2 : STEPS;
 
         // One panel: `par` is kp & 1, known at compile time so that the register sets are
@@ -303,9 +365,10 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             constexpr int PAR = decltype(par_tag)::value;
             constexpr int R_IN = DEPTH == 2 ? PAR : 0;       // set receiving the new loads
             constexpr int R_OUT = DEPTH == 2 ? PAR ^ 1 : 0;  // set written to LDS during this panel
-            if (kp + DEPTH < n_panels) fetch_panel(kp + DEPTH, ra[R_IN], rb[R_IN]);
+            const bool issued = kp + DEPTH < n_panels;
+            if (issued) issue_panel(kp + DEPTH, ra[R_IN], rb[R_IN]);
 
-            const T *As = smem + PAR * STAGE;
+            const T *As = stage_ptr(kp);
             const T *Bs = As + A_ELEMS;
             // MFMA step s of a panel consumes, in lane group g, the k index
             //   kmap(s,g) = (s / VEC) * VEC * NG + g * VEC + s % VEC,
@@ -313,13 +376,14 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             // per step, a [n][k] panel is read as one 16-byte vector per VEC steps.
             // Fragments are read one step (one VEC-step group for [n][k]) ahead of their use.
             T a[2][TM], b[2][TN], bk[2][TN][VEC];
+            auto a_at = [&](int k, int x) { return LA::DMA ? LA::lds_at(k, x) : k * PITCH_A + x; };
             auto kmap = [&](int s) { return (s / VEC) * (VEC * NG) + g * VEC + (s % VEC); };
             auto read_a = [&](int s, T (&af)[TM]) {
                 const int krow = kmap(s);
 #pragma unroll
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     typename Vec<T, VM>::type av =
-                        *reinterpret_cast<const typename Vec<T, VM>::type *>(&As[krow * PITCH_A + a_frag + ga * MB * VM]);
+                        *reinterpret_cast<const typename Vec<T, VM>::type *>(&As[a_at(krow, a_frag + ga * MB * VM)]);
                     if constexpr (VM == 1) af[ga] = av;
                     else {
 #pragma unroll
@@ -332,7 +396,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 #pragma unroll
                 for (int gb = 0; gb < TN / VN; ++gb) {
                     typename Vec<T, VN>::type bv =
-                        *reinterpret_cast<const typename Vec<T, VN>::type *>(&Bs[krow * PITCH_B + b_frag + gb * MB * VN]);
+                        *reinterpret_cast<const typename Vec<T, VN>::type *>(&Bs[LB::lds_at(krow, b_frag + gb * MB * VN)]);
                     if constexpr (VN == 1) bf[gb] = bv;
                     else {
 #pragma unroll
@@ -343,8 +407,10 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             auto read_bk = [&](int grp, T (&bf)[TN][VEC]) {  // [n][k] B panel, VEC steps at once
 #pragma unroll
                 for (int bn = 0; bn < TN; ++bn) {
-                    typename Vec<T, VEC>::type bv = *reinterpret_cast<const typename Vec<T, VEC>::type *>(
-                        &Bs[(wn * WN + bn * MB + j) * PITCH_B + grp * (VEC * NG) + g * VEC]);
+                    const int n_loc = wn * WN + bn * MB + j;
+                    const int place = (grp * NG + g) ^ LB::swz(n_loc);
+                    typename Vec<T, VEC>::type bv =
+                        *reinterpret_cast<const typename Vec<T, VEC>::type *>(&Bs[n_loc * PITCH_B + place * VEC]);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) bf[bn][e] = bv[e];
                 }
@@ -369,12 +435,14 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     for (int bm = 0; bm < TM; ++bm) acc[bn][bm] = M::run(bval, a[s & 1][bm], acc[bn][bm]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (s + 1 == STORE_AT) {
-                    if (kp + 1 < n_panels) store_panel(kp + 1, ra[R_OUT], rb[R_OUT]);
+                if (!LA::DMA && s + 1 == STORE_AT && s + 1 < STEPS) {
+                    if (kp + 1 < n_panels)
+                        la.store(stage_ptr(kp + 1), tid, k_end - (k_begin + (kp + 1) * BK), ra[R_OUT]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
-            __syncthreads();
+            if (kp + 1 < n_panels) publish_panel(kp + 1, DEPTH == 2 && issued, ra[R_OUT], !LA::DMA && STORE_AT == STEPS);
+            else __syncthreads();
         };
 
         for (int kp = 0; kp < n_panels; kp += 2) {
