@@ -236,9 +236,10 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static constexpr int PITCH_A = LoaderA::LDS_PITCH, PITCH_B = LoaderB::LDS_PITCH;
     static constexpr int A_ELEMS = LoaderA::LDS_ELEMS;
     static constexpr int STAGE = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;  // elements per LDS stage
-    // Three stages (loads two panels ahead) when two workgroups of them still share a CU's
-    // 160 KiB, otherwise two (loads one panel ahead).
-    static constexpr int NSTAGE = (2 * 3 * STAGE * (int)sizeof(T) <= 150 * 1024) ? 3 : 2;
+    // Two stages: the loads of panel p+1 are issued at the top of panel p.  A third stage
+    // (loads two panels ahead) was measured 1-5 % slower on every tile shape; the kernel
+    // keeps the general ring so that the depth stays a one-line choice.
+    static constexpr int NSTAGE = 2;
     static constexpr int DEPTH = NSTAGE - 1;
     static constexpr size_t SMEM = (size_t)NSTAGE * STAGE * sizeof(T);
 };
@@ -463,45 +464,63 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     }
     const bool read_c = !(beta == (T)0);
 
+    // C is read in batches of CH accumulator rows per lane before any of them is written
+    // back, so that the load latencies of a batch overlap instead of queueing behind each
+    // store (loads and stores go to the same array, so the compiler keeps their order).
+    typedef typename Vec<T, VM>::utype UV;
+    constexpr int CH = NACC < 8 ? NACC : 8;
 #pragma unroll
     for (int bn = 0; bn < TN; ++bn) {
 #pragma unroll
-        for (int v = 0; v < NACC; ++v) {
-            const int n = n0 + wn * WN + (bn / VNM) * (MB * VNM) + M::row(v, lane) * VNM + (bn % VNM);
-            if (n >= p.N) continue;
-            T *col = Cout + (int64_t)n * ldc;
+        for (int v0 = 0; v0 < NACC; v0 += CH) {
+            UV cold[CH][TM / VM];
+            if (read_c) {
 #pragma unroll
-            for (int ga = 0; ga < TM / VM; ++ga) {
-                const int m = m0 + wm * WM + ga * (MB * VM) + j * VM;
-                if (m + VM <= p.M) {
-                    typedef typename Vec<T, VM>::utype UV;
-                    T r[VM];
-                    if (read_c) {
-                        UV cv = *reinterpret_cast<const UV *>(col + m);
+                for (int dv = 0; dv < CH; ++dv) {
+                    const int n = n0 + wn * WN + (bn / VNM) * (MB * VNM) + M::row(v0 + dv, lane) * VNM + (bn % VNM);
+                    const T *col = Cout + (int64_t)n * ldc;
+#pragma unroll
+                    for (int ga = 0; ga < TM / VM; ++ga) {
+                        const int m = m0 + wm * WM + ga * (MB * VM) + j * VM;
+                        if (n < p.N && m + VM <= p.M) cold[dv][ga] = *reinterpret_cast<const UV *>(col + m);
+                    }
+                }
+            }
+#pragma unroll
+            for (int dv = 0; dv < CH; ++dv) {
+                const int v = v0 + dv;
+                const int n = n0 + wn * WN + (bn / VNM) * (MB * VNM) + M::row(v, lane) * VNM + (bn % VNM);
+                if (n >= p.N) continue;
+                T *col = Cout + (int64_t)n * ldc;
+#pragma unroll
+                for (int ga = 0; ga < TM / VM; ++ga) {
+                    const int m = m0 + wm * WM + ga * (MB * VM) + j * VM;
+                    if (m + VM <= p.M) {
+                        T r[VM];
 #pragma unroll
                         for (int e = 0; e < VM; ++e) {
-                            T c_old;
-                            if constexpr (VM == 1) c_old = cv; else c_old = cv[e];
-                            r[e] = alpha * acc[bn][ga * VM + e][v] + beta * c_old;
+                            r[e] = alpha * acc[bn][ga * VM + e][v];
+                            if (read_c) {
+                                T c_old;
+                                if constexpr (VM == 1) c_old = cold[dv][ga]; else c_old = cold[dv][ga][e];
+                                r[e] += beta * c_old;
+                            }
                         }
+                        UV ov;
+                        if constexpr (VM == 1) ov = r[0];
+                        else {
+#pragma unroll
+                            for (int e = 0; e < VM; ++e) ov[e] = r[e];
+                        }
+                        *reinterpret_cast<UV *>(col + m) = ov;
                     } else {
 #pragma unroll
-                        for (int e = 0; e < VM; ++e) r[e] = alpha * acc[bn][ga * VM + e][v];
-                    }
-                    UV ov;
-                    if constexpr (VM == 1) ov = r[0];
-                    else {
-#pragma unroll
-                        for (int e = 0; e < VM; ++e) ov[e] = r[e];
-                    }
-                    *reinterpret_cast<UV *>(col + m) = ov;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < VM; ++e) {
-                        if (m + e < p.M) {
-                            T r = alpha * acc[bn][ga * VM + e][v];
-                            if (read_c) r += beta * col[m + e];
-                            col[m + e] = r;
+                        for (int e = 0; e < VM; ++e) {
+                            if (m + e < p.M) {
+                                T r = alpha * acc[bn][ga * VM + e][v];
+                                if (read_c) r += beta * col[m + e];
+                                col[m + e] = r;
+                            }
                         }
                     }
                 }
