@@ -10,17 +10,18 @@
 //   * Panels of depth BK travel HBM -> LDS without passing through registers wherever the
 //     LDS image is a plain copy of memory: `buffer_load_dwordx4 ... lds` writes each wave's
 //     64 x 16 bytes to consecutive LDS addresses.  That covers operands contiguous along the
-//     tile edge (As[k][m], Bs[k][n]) and a k-contiguous B panel, kept as Bs[n][k] with its
-//     16-byte slots XOR-swizzled by the row so that fragment reads stay bank-conflict free.
-//     Only a k-contiguous A panel (transA == T) is still staged through registers and
-//     transposed into As[k][m] (pitch BM+4), so that C keeps its 16-byte row stores.
+//     tile edge (As[k][m], Bs[k][n]) and k-contiguous panels, kept as As[m][k] / Bs[n][k]
+//     with their 16-byte slots XOR-swizzled by the row so that fragment reads stay
+//     bank-conflict free.  Each lane of such a load names its own source address, so the rows
+//     of As[m][k] are stored block by block (all rows of MFMA block 0, then block 1, ...)
+//     while a lane still owns VM consecutive rows of C for its 16-byte stores.
 //   * NSTAGE LDS stages form a ring; the loads of panel p+NSTAGE-1 are issued at the top of
 //     panel p and one barrier per panel publishes the next stage.  Buffer descriptors are
 //     re-based every panel and sized to the exact footprint of the operand, so the hardware
 //     range check turns every access past the end of the matrix into a zero (also on the
 //     LDS path): no extra launch and no per-element branch is needed for M/N remainders or
 //     for the K remainder of tile-edge-contiguous operands; the K remainder of a
-//     k-contiguous panel is real memory and is cleared in LDS before it is used.
+//     k-contiguous panel is real memory (the next column) and is cleared in LDS before use.
 //   * Each wave owns a WM x WN sub-tile as TM x TN MFMA blocks
 //     (v_mfma_f32_32x32x2_f32 / v_mfma_f64_16x16x4_f64).  The MFMA "B" operand carries the
 //     A matrix and the "A" operand carries the B matrix, so that the lane index of the
@@ -110,15 +111,15 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 // 15:14, expcnt 6:4, lgkmcnt 11:8; the other counters are left at "don't wait").
 #define CBA_VMCNT_ONLY(n) ((((n) & 0xf) | ((((n) >> 4) & 0x3) << 14) | (0x7 << 4) | (0xf << 8)))
 
-// How an operand panel gets from memory into LDS.
+// How an operand panel gets from memory into LDS (always `buffer_load_dwordx4 ... lds`).
 //   LM_DMA_X: memory contiguous along the tile edge x; LDS image [k][x], pitch BX.
-//   LM_DMA_K: memory contiguous along k; LDS image [x][k], pitch BK, 16-byte slots of row x
-//             stored at slot ^ swz(x)  (B operand with transB == N).
-//   LM_REG_T: memory contiguous along k; staged through registers and transposed into
-//             [k][x], pitch BX+4 (A operand with transA == T).
-enum LoadMode { LM_DMA_X = 0, LM_DMA_K = 1, LM_REG_T = 2 };
+//   LM_DMA_K: memory contiguous along k; LDS image [x'][k], pitch BK, 16-byte slots of row x'
+//             stored at slot ^ swz(x').  Row x' of the image holds tile row perm(x'): with
+//             interleave IL and block edge MBLK, image rows [e*MBLK, (e+1)*MBLK) of every
+//             span of IL*MBLK rows hold the tile rows j*IL + e (IL == 1: identity).
+enum LoadMode { LM_DMA_X = 0, LM_DMA_K = 1 };
 
-template <typename T, int BX, int BK, int NT, int MODE> struct PanelLoader {
+template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1> struct PanelLoader {
     static constexpr int VEC = 16 / (int)sizeof(T);
     static constexpr int NVEC = BX * BK / VEC;
     static constexpr int PER = NVEC / NT;  // 16-byte vectors per thread = wave-wide loads per wave
@@ -132,20 +133,25 @@ template <typename T, int BX, int BK, int NT, int MODE> struct PanelLoader {
     static constexpr int CHUNKS_APART = VEC / ROWS_PER_CHUNK > 0 ? VEC / ROWS_PER_CHUNK : 1;
     static constexpr int CHUNK_PAD = MODE == LM_DMA_X ? (64 / (int)sizeof(T)) / CHUNKS_APART : 0;  // elements
     static constexpr int CHUNK_PITCH = CHUNK + CHUNK_PAD;
-    static constexpr int LDS_PITCH = MODE == LM_DMA_X ? BX : (MODE == LM_DMA_K ? BK : BX + 4);
-    static constexpr int LDS_ELEMS = MODE == LM_REG_T ? BK * LDS_PITCH : (NVEC / 64) * CHUNK_PITCH;
+    static constexpr int LDS_PITCH = MODE == LM_DMA_X ? BX : BK;
+    static constexpr int LDS_ELEMS = (NVEC / 64) * CHUNK_PITCH;
     // LM_DMA_X: LDS element offset of image element (k, x).
     static __device__ __forceinline__ int lds_at(int k, int x) {
         const int e = k * BX + x;
         return e + (e / CHUNK) * CHUNK_PAD;
     }
-    static constexpr bool DMA = MODE != LM_REG_T;
     // LM_DMA_K swizzle: S slots per row; rows x and x + 16/S start in the same bank.
     static constexpr int S = BK / VEC;
     static_assert(MODE != LM_DMA_K || (S <= 16 && 16 % S == 0), "swizzle needs S | 16");
+    static_assert(MODE != LM_DMA_K || BX % (IL * MBLK) == 0, "row interleave must tile the panel");
     static __device__ __forceinline__ int swz(int x) { return (x / (16 / S)) % S; }
+    // LM_DMA_K: tile row held by image row x.
+    static __device__ __forceinline__ int perm(int x) {
+        if (IL == 1) return x;
+        const int span = IL * MBLK, r = x % span;
+        return (x / span) * span + (r % MBLK) * IL + r / MBLK;
+    }
 
-    struct Regs { u32x4 v[DMA ? 1 : PER]; };  // LM_REG_T: one panel's worth of data in flight
     uint32_t voff[PER];
 
     __device__ __forceinline__ void init(int tid, int64_t ld) {
@@ -156,46 +162,22 @@ template <typename T, int BX, int BK, int NT, int MODE> struct PanelLoader {
                 const int e = (wave + i * NW) * CHUNK + lane * VEC;  // element index in the [k][x] image
                 const int k = e / BX, x = e % BX;
                 voff[i] = (uint32_t)(((int64_t)k * ld + x) * (int64_t)sizeof(T));
-            } else if (MODE == LM_DMA_K) {
+            } else {
                 const int x = (wave + i * NW) * (64 / S) + lane / S;
                 const int slot = (lane % S) ^ swz(x);  // logical slot stored in this lane's place
-                voff[i] = (uint32_t)(((int64_t)x * ld + slot * VEC) * (int64_t)sizeof(T));
-            } else {
-                const int idx = tid + i * NT;
-                const int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
-                voff[i] = (uint32_t)(((int64_t)x * ld + kv) * (int64_t)sizeof(T));
+                voff[i] = (uint32_t)(((int64_t)perm(x) * ld + slot * VEC) * (int64_t)sizeof(T));
             }
         }
     }
 
     // Starts the transfer of one panel.  base: first element of the panel; bytes_left:
     // footprint bytes from `base` on; lds: this operand's image in the receiving stage.
-    __device__ __forceinline__ void issue(const T *base, int64_t bytes_left, T *lds, int wave_u, Regs &reg) const {
+    __device__ __forceinline__ void issue(const T *base, int64_t bytes_left, T *lds, int wave_u) const {
         __amdgpu_buffer_rsrc_t r = make_rsrc(base, bytes_left);
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            if (DMA) {
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH), 16,
-                                                         (int)voff[i], 0, 0, 0);
-            } else {
-                reg.v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff[i], 0, 0);
-            }
-        }
-    }
-
-    // LM_REG_T: registers -> LDS, transposing; elements past K are cleared (they are real
-    // memory - the next column - not out of range).
-    __device__ __forceinline__ void store(T *lds, int tid, int k_valid, const Regs &reg) const {
-        if (DMA) return;
-#pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int idx = tid + i * NT;
-            const int x = idx / (BK / VEC), kv = (idx % (BK / VEC)) * VEC;
-            union { u32x4 u; T e[VEC]; } cv;
-            cv.u = reg.v[i];
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) lds[(kv + e) * LDS_PITCH + x] = (kv + e < k_valid) ? cv.e[e] : (T)0;
-        }
+        for (int i = 0; i < PER; ++i)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH), 16,
+                                                     (int)voff[i], 0, 0, 0);
     }
 
     // LM_DMA_K: clears the elements past K of a partial panel, each thread in the 16 bytes
@@ -225,13 +207,14 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static constexpr int VN = TN < VEC ? TN : VEC;
     static_assert(BM % WM == 0 && BN % WN == 0 && WM % MB == 0 && WN % MB == 0, "tile shape");
     static_assert(TM % VM == 0 && TN % VN == 0 && BK % KS == 0, "tile shape");
-    // A k-contiguous B panel (transB == N) is kept as Bs[n][k]; a k-contiguous A panel is
-    // transposed into As[k][m] so that C keeps its 16-byte row-interleaved stores.
-    static constexpr bool B_KLAY = B_KC;
+    // k-contiguous panels (transA == T, transB == N) are kept as As[m][k] / Bs[n][k].  The m
+    // interleave of the C mapping is the same for both A layouts (the [m][k] image permutes
+    // its rows instead); n is interleaved only for a k-major B panel.
+    static constexpr bool A_KLAY = A_KC, B_KLAY = B_KC;
     static constexpr int VNM = B_KLAY ? 1 : VN;  // n interleave used by the fragment/epilogue mapping
     static constexpr int NG = 64 / MB;           // lane groups along k
     static_assert(BK % (VEC * NG) == 0, "panel depth must hold whole k groups");
-    typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_REG_T : LM_DMA_X> LoaderA;
+    typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_DMA_K : LM_DMA_X, VM, MB> LoaderA;
     typedef PanelLoader<T, BN, BK, NT, B_KC ? LM_DMA_K : LM_DMA_X> LoaderB;
     static constexpr int PITCH_A = LoaderA::LDS_PITCH, PITCH_B = LoaderB::LDS_PITCH;
     static constexpr int A_ELEMS = LoaderA::LDS_ELEMS;
@@ -254,7 +237,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     constexpr int PITCH_A = Cfg::PITCH_A, PITCH_B = Cfg::PITCH_B, STAGE = Cfg::STAGE;
     constexpr int VEC = Cfg::VEC, NG = Cfg::NG, A_ELEMS = Cfg::A_ELEMS, VNM = Cfg::VNM;
     constexpr int NSTAGE = Cfg::NSTAGE, DEPTH = Cfg::DEPTH;
-    constexpr bool B_KLAY = Cfg::B_KLAY;
+    constexpr bool A_KLAY = Cfg::A_KLAY, B_KLAY = Cfg::B_KLAY;
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *smem = reinterpret_cast<T *>(smem_raw);
@@ -321,70 +304,60 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         // kp+DEPTH go out at the top of panel kp into the stage whose last readers finished
         // before the barrier that ended panel kp-1.  Before the barrier that ends panel kp,
         // each wave waits for its own loads of panel kp+1 (issued a panel earlier when
-        // DEPTH is 2); the register-staged operand is written into that stage mid-way.
+        // DEPTH is 2).
         typedef typename Cfg::LoaderA LA;
         typedef typename Cfg::LoaderB LB;
-        constexpr int RSETS = DEPTH;  // register sets of a staged operand
-        typename LA::Regs ra[RSETS];
-        typename LB::Regs rb[RSETS];
         constexpr int LOADS_PER_PANEL = LA::PER + LB::PER;  // vector-memory instructions per wave and panel
 
         auto stage_ptr = [&](int kp) -> T * { return smem + (kp % NSTAGE) * STAGE; };
-        auto issue_panel = [&](int kp, typename LA::Regs &xa, typename LB::Regs &xb) {
+        auto issue_panel = [&](int kp) {
             const int k0 = k_begin + kp * BK;
             const int64_t ao = a_off(k0), bo = b_off(k0);
             T *dst = stage_ptr(kp);
-            la.issue(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T), dst, wave_u, xa);
-            lb.issue(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T), dst + A_ELEMS, wave_u, xb);
+            la.issue(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T), dst, wave_u);
+            lb.issue(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T), dst + A_ELEMS, wave_u);
         };
         // Makes panel kp (already requested) readable by the whole workgroup: own loads
-        // complete, staged registers written, K tail cleared, barrier.
-        auto publish_panel = [&](int kp, bool newer_in_flight, const typename LA::Regs &xa, bool store_a) {
+        // complete, K tail cleared, barrier.
+        auto publish_panel = [&](int kp, bool newer_in_flight) {
             T *dst = stage_ptr(kp);
             const int k_valid = k_end - (k_begin + kp * BK);
-            if (store_a) la.store(dst, tid, k_valid, xa);
             if (newer_in_flight) __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(LOADS_PER_PANEL));
             else __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0));
-            if (k_valid < BK) lb.clear_k_tail(dst + A_ELEMS, tid, k_valid);
+            if (k_valid < BK) {
+                la.clear_k_tail(dst, tid, k_valid);
+                lb.clear_k_tail(dst + A_ELEMS, tid, k_valid);
+            }
             __syncthreads();
         };
 
-        issue_panel(0, ra[0], rb[0]);
-        if (DEPTH == 2 && n_panels > 1) issue_panel(1, ra[RSETS - 1], rb[RSETS - 1]);
-        publish_panel(0, DEPTH == 2 && n_panels > 1, ra[0], true);
+        issue_panel(0);
+        if (DEPTH == 2 && n_panels > 1) issue_panel(1);
+        publish_panel(0, DEPTH == 2 && n_panels > 1);
 
         const int a_frag = wm * WM + j * VM;
         const int b_frag = wn * WN + j * VN;
         constexpr int STEPS = BK / KS;
-        // MFMA step after which a register-staged A panel goes to LDS: mid-way when it was
-        // requested a whole panel earlier, after the last step otherwise.
-        constexpr int STORE_AT = DEPTH == 2 ? STEPS / 2 : STEPS;
 
-        // One panel: `par` is kp & 1, known at compile time so that the register sets are
-        // addressed statically.
-        auto do_panel = [&](int kp, auto par_tag) {
-            constexpr int PAR = decltype(par_tag)::value;
-            constexpr int R_IN = DEPTH == 2 ? PAR : 0;       // set receiving the new loads
-            constexpr int R_OUT = DEPTH == 2 ? PAR ^ 1 : 0;  // set written to LDS during this panel
+        auto do_panel = [&](int kp) {
             const bool issued = kp + DEPTH < n_panels;
-            if (issued) issue_panel(kp + DEPTH, ra[R_IN], rb[R_IN]);
+            if (issued) issue_panel(kp + DEPTH);
 
             const T *As = stage_ptr(kp);
             const T *Bs = As + A_ELEMS;
             // MFMA step s of a panel consumes, in lane group g, the k index
             //   kmap(s,g) = (s / VEC) * VEC * NG + g * VEC + s % VEC,
             // i.e. VEC consecutive steps walk VEC consecutive k: a k-major panel row is read
-            // per step, a [n][k] panel is read as one 16-byte vector per VEC steps.
-            // Fragments are read one step (one VEC-step group for [n][k]) ahead of their use.
-            T a[2][TM], b[2][TN], bk[2][TN][VEC];
-            auto a_at = [&](int k, int x) { return LA::DMA ? LA::lds_at(k, x) : k * PITCH_A + x; };
+            // per step, a [x][k] panel is read as one 16-byte vector per VEC steps.
+            // Fragments are read one step (one VEC-step group for [x][k]) ahead of their use.
+            T a[2][TM], b[2][TN], ak[2][TM][VEC], bk[2][TN][VEC];
             auto kmap = [&](int s) { return (s / VEC) * (VEC * NG) + g * VEC + (s % VEC); };
-            auto read_a = [&](int s, T (&af)[TM]) {
+            auto read_a = [&](int s, T (&af)[TM]) {  // k-major A panel
                 const int krow = kmap(s);
 #pragma unroll
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     typename Vec<T, VM>::type av =
-                        *reinterpret_cast<const typename Vec<T, VM>::type *>(&As[a_at(krow, a_frag + ga * MB * VM)]);
+                        *reinterpret_cast<const typename Vec<T, VM>::type *>(&As[LA::lds_at(krow, a_frag + ga * MB * VM)]);
                     if constexpr (VM == 1) af[ga] = av;
                     else {
 #pragma unroll
@@ -405,6 +378,17 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     }
                 }
             };
+            auto read_ak = [&](int grp, T (&af)[TM][VEC]) {  // [m'][k] A panel, VEC steps at once
+#pragma unroll
+                for (int bm = 0; bm < TM; ++bm) {
+                    const int m_img = wm * WM + bm * MB + j;  // image row of block bm, lane j
+                    const int place = (grp * NG + g) ^ LA::swz(m_img);
+                    typename Vec<T, VEC>::type av =
+                        *reinterpret_cast<const typename Vec<T, VEC>::type *>(&As[m_img * PITCH_A + place * VEC]);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) af[bm][e] = av[e];
+                }
+            };
             auto read_bk = [&](int grp, T (&bf)[TN][VEC]) {  // [n][k] B panel, VEC steps at once
 #pragma unroll
                 for (int bn = 0; bn < TN; ++bn) {
@@ -416,12 +400,16 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     for (int e = 0; e < VEC; ++e) bf[bn][e] = bv[e];
                 }
             };
-            read_a(0, a[0]);
+            if constexpr (A_KLAY) read_ak(0, ak[0]); else read_a(0, a[0]);
             if constexpr (B_KLAY) read_bk(0, bk[0]); else read_b(0, b[0]);
 #pragma unroll
             for (int s = 0; s < STEPS; ++s) {
                 if (s + 1 < STEPS) {
-                    read_a(s + 1, a[(s + 1) & 1]);
+                    if constexpr (A_KLAY) {
+                        if ((s + 1) % VEC == 0) read_ak((s + 1) / VEC, ak[((s + 1) / VEC) & 1]);
+                    } else {
+                        read_a(s + 1, a[(s + 1) & 1]);
+                    }
                     if constexpr (B_KLAY) {
                         if ((s + 1) % VEC == 0) read_bk((s + 1) / VEC, bk[((s + 1) / VEC) & 1]);
                     } else {
@@ -433,22 +421,20 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 for (int bn = 0; bn < TN; ++bn) {
                     const T bval = B_KLAY ? bk[(s / VEC) & 1][bn][s % VEC] : b[s & 1][bn];
 #pragma unroll
-                    for (int bm = 0; bm < TM; ++bm) acc[bn][bm] = M::run(bval, a[s & 1][bm], acc[bn][bm]);
+                    for (int bm = 0; bm < TM; ++bm) {
+                        const T aval = A_KLAY ? ak[(s / VEC) & 1][bm][s % VEC] : a[s & 1][bm];
+                        acc[bn][bm] = M::run(bval, aval, acc[bn][bm]);
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (!LA::DMA && s + 1 == STORE_AT && s + 1 < STEPS) {
-                    if (kp + 1 < n_panels)
-                        la.store(stage_ptr(kp + 1), tid, k_end - (k_begin + (kp + 1) * BK), ra[R_OUT]);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
             }
-            if (kp + 1 < n_panels) publish_panel(kp + 1, DEPTH == 2 && issued, ra[R_OUT], !LA::DMA && STORE_AT == STEPS);
+            if (kp + 1 < n_panels) publish_panel(kp + 1, DEPTH == 2 && issued);
             else __syncthreads();
         };
-
+        // Two panels per trip, so that the stage addresses of each copy are loop-invariant.
         for (int kp = 0; kp < n_panels; kp += 2) {
-            do_panel(kp, std::integral_constant<int, 0>());
-            if (kp + 1 < n_panels) do_panel(kp + 1, std::integral_constant<int, 1>());
+            do_panel(kp);
+            if (kp + 1 < n_panels) do_panel(kp + 1);
         }
     }
 
