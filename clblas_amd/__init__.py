@@ -2,8 +2,9 @@
 behind clBLAS's call surface.
 
 The product is the shared library (C ABI declared in include/clblas_amd.h).  This module
-only loads it with ctypes and mirrors the four entry points with the reference's argument
-order (src/clBLAS.h:7382-7405, 7463-7486, 7988-8008, 8063-8083); matrices are passed as
+only loads it with ctypes and mirrors the entry points with the reference's argument
+order (src/clBLAS.h:7382-7405, 7463-7486, 7538-7561, 7622-7645, 7988-8008, 8063-8083);
+matrices are passed as
 torch CUDA tensors (used purely as device allocations) or as integer device addresses.
 
 There is no CPU fallback: if the library has not been built, loading raises.
@@ -68,11 +69,23 @@ EXPORTED_SYMBOLS = (
     "clblasTeardown",
     "clblasSgemm",
     "clblasDgemm",
+    "clblasCgemm",
+    "clblasZgemm",
     "clblasStrsm",
     "clblasDtrsm",
 )
 
 _lib = None
+
+
+class FloatComplex(ctypes.Structure):
+    """By-value complex scalar of clblasCgemm (two floats, one SSE register on x86-64)."""
+    _fields_ = [("re", ctypes.c_float), ("im", ctypes.c_float)]
+
+
+class DoubleComplex(ctypes.Structure):
+    """By-value complex scalar of clblasZgemm."""
+    _fields_ = [("re", ctypes.c_double), ("im", ctypes.c_double)]
 
 
 def _declare(lib):
@@ -81,6 +94,10 @@ def _declare(lib):
         fn = getattr(lib, name)
         fn.restype = i
         fn.argtypes = [i, i, i, sz, sz, sz, real, vp, sz, sz, vp, sz, sz, real, vp, sz, sz, vp]
+    for name, cplx in (("clblasCgemm", FloatComplex), ("clblasZgemm", DoubleComplex)):
+        fn = getattr(lib, name)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, sz, cplx, vp, sz, sz, vp, sz, sz, cplx, vp, sz, sz, vp]
     for name, real in (("clblasStrsm", ctypes.c_float), ("clblasDtrsm", ctypes.c_double)):
         fn = getattr(lib, name)
         fn.restype = i
@@ -149,6 +166,22 @@ def sgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, bet
 def dgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
     return load_library().clblasDgemm(int(order), int(transA), int(transB), M, N, K, alpha, _ptr(A), offA, lda,
                                       _ptr(B), offB, ldb, beta, _ptr(C), offC, ldc, _stream(stream))
+
+
+def cgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    """alpha / beta: Python complex; A, B, C: complex64 tensors (or device addresses)."""
+    a, b = complex(alpha), complex(beta)
+    return load_library().clblasCgemm(int(order), int(transA), int(transB), M, N, K, FloatComplex(a.real, a.imag),
+                                      _ptr(A), offA, lda, _ptr(B), offB, ldb, FloatComplex(b.real, b.imag),
+                                      _ptr(C), offC, ldc, _stream(stream))
+
+
+def zgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    """alpha / beta: Python complex; A, B, C: complex128 tensors (or device addresses)."""
+    a, b = complex(alpha), complex(beta)
+    return load_library().clblasZgemm(int(order), int(transA), int(transB), M, N, K, DoubleComplex(a.real, a.imag),
+                                      _ptr(A), offA, lda, _ptr(B), offB, ldb, DoubleComplex(b.real, b.imag),
+                                      _ptr(C), offC, ldc, _stream(stream))
 
 
 def strsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):

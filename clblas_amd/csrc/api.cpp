@@ -1,7 +1,7 @@
 // C ABI of libclblas_amd.so: argument validation, row-major folding and dispatch.
 //
 // This is the host front end that stands where the reference has
-//   src/library/blas/xgemm.cc:667-783  (clblasSgemm / clblasDgemm),
+//   src/library/blas/xgemm.cc:667-905  (clblasSgemm / clblasDgemm / clblasCgemm / clblasZgemm),
 //   src/library/blas/xgemm.cc:341-383  (clblasGemm<T>: ConjTrans and row-major folding),
 //   src/library/blas/xtrsm.cc:1600-1785 (clblasStrsm / clblasDtrsm),
 //   src/library/blas/functor/functor_xtrsm.cc:57-75 (doTrsm validation),
@@ -148,20 +148,36 @@ clblasStatus gemm_front(Fn launch, clblasOrder order, clblasTranspose transA, cl
     if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldc, MAT_C)) != clblasSuccess) return st;
     if (M > kMaxDim || N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
 
-    // Real types: ConjTrans is Trans (xgemm.cc:330-335).
+    // Real types: ConjTrans is Trans (xgemm.cc:330-335); the real launchers ignore cA / cB.
     bool tA = transA != clblasNoTrans, tB = transB != clblasNoTrans;
+    bool cA = transA == clblasConjTrans, cB = transB == clblasConjTrans;
     const T *pa = A + offA, *pb = B + offB;
     // Row major is the column-major product C^T = op(B)^T op(A)^T (xgemm.cc:40-61):
     // swap the operands, their transposes, leading dimensions, and M with N.
     if (order == clblasRowMajor) {
         std::swap(tA, tB);
+        std::swap(cA, cB);
         std::swap(M, N);
         std::swap(lda, ldb);
         std::swap(pa, pb);
     }
-    return map_hip_error(launch(tA, tB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb, (int64_t)ldb, beta,
-                                C + offC, (int64_t)ldc, stream));
+    return map_hip_error(launch(tA, tB, cA, cB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb, (int64_t)ldb,
+                                beta, C + offC, (int64_t)ldc, stream));
 }
+
+hipError_t sgemm_real(bool tA, bool tB, bool, bool, int M, int N, int K, float alpha, const float *A, int64_t lda,
+                      const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream) {
+    return cba::sgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+hipError_t dgemm_real(bool tA, bool tB, bool, bool, int M, int N, int K, double alpha, const double *A, int64_t lda,
+                      const double *B, int64_t ldb, double beta, double *C, int64_t ldc, hipStream_t stream) {
+    return cba::dgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+}
+
+static_assert(sizeof(FloatComplex) == sizeof(cba::Cx<float>) && sizeof(DoubleComplex) == sizeof(cba::Cx<double>),
+              "complex layouts must agree");
+inline cba::Cx<float> cx(FloatComplex z) { return cba::Cx<float>{z.s[0], z.s[1]}; }
+inline cba::Cx<double> cx(DoubleComplex z) { return cba::Cx<double>{z.s[0], z.s[1]}; }
 
 template <typename T, typename Fn>
 clblasStatus trsm_front(Fn launch, clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
@@ -228,7 +244,7 @@ clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B,
                          size_t offB, size_t ldb, float beta, float *C, size_t offC, size_t ldc,
                          hipStream_t stream) {
-    return gemm_front<float>(cba::sgemm_colmajor, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb,
+    return gemm_front<float>(sgemm_real, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb,
                              beta, C, offC, ldc, stream);
 }
 
@@ -236,8 +252,28 @@ clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          size_t K, double alpha, const double *A, size_t offA, size_t lda, const double *B,
                          size_t offB, size_t ldb, double beta, double *C, size_t offC, size_t ldc,
                          hipStream_t stream) {
-    return gemm_front<double>(cba::dgemm_colmajor, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB,
+    return gemm_front<double>(dgemm_real, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB,
                               ldb, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasCgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
+                         size_t K, FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                         const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta, FloatComplex *C,
+                         size_t offC, size_t ldc, hipStream_t stream) {
+    typedef cba::Cx<float> E;
+    return gemm_front<E>(cba::cgemm_colmajor, order, transA, transB, M, N, K, cx(alpha),
+                         reinterpret_cast<const E *>(A), offA, lda, reinterpret_cast<const E *>(B), offB, ldb,
+                         cx(beta), reinterpret_cast<E *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasZgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
+                         size_t K, DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                         const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta, DoubleComplex *C,
+                         size_t offC, size_t ldc, hipStream_t stream) {
+    typedef cba::Cx<double> E;
+    return gemm_front<E>(cba::zgemm_colmajor, order, transA, transB, M, N, K, cx(alpha),
+                         reinterpret_cast<const E *>(A), offA, lda, reinterpret_cast<const E *>(B), offB, ldb,
+                         cx(beta), reinterpret_cast<E *>(C), offC, ldc, stream);
 }
 
 clblasStatus clblasStrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,

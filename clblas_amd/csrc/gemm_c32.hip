@@ -1,0 +1,29 @@
+// Complex FP32 GEMM: tile table and entry point.
+#include "gemm_launch.hpp"
+
+namespace cba {
+
+// Ordered from the largest tile to the smallest.  A complex element carries four times the
+// flops of a real one for twice the bytes, so these tiles match the real 256x128 / 128x128
+// ones in arithmetic intensity at half the panel depth.
+//   0: 128x128x8, wave 64x64 (2 workgroups of 4 waves per CU)
+//   1:  64x64x8,  wave 32x32, split-K capable
+static const TileEntry<Cx<float>> *c32_tiles(int *n) {
+    static const TileEntry<Cx<float>> tab[] = {
+        make_tile_entry<Cx<float>, 128, 128, 8, 64, 64, 2, false>(0.88),
+        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true>(0.78),
+    };
+    *n = (int)(sizeof(tab) / sizeof(tab[0]));
+    return tab;
+}
+
+hipError_t cgemm_colmajor(bool transA, bool transB, bool conjA, bool conjB, int M, int N, int K, Cx<float> alpha,
+                          const Cx<float> *A, int64_t lda, const Cx<float> *B, int64_t ldb, Cx<float> beta,
+                          Cx<float> *C, int64_t ldc, hipStream_t stream) {
+    int n;
+    const TileEntry<Cx<float>> *tab = c32_tiles(&n);
+    return run_gemm_colmajor<Cx<float>>(tab, n, transA, transB, conjA, conjB, M, N, K, alpha, A, lda, B, ldb, beta,
+                                        C, ldc, stream);
+}
+
+}  // namespace cba

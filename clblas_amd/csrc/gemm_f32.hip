@@ -21,7 +21,7 @@ hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float a
                           const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream) {
     int n;
     const TileEntry<float> *tab = f32_tiles(&n);
-    return run_gemm_colmajor<float>(tab, n, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+    return run_gemm_colmajor<float>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
 }
 
 }  // namespace cba

@@ -20,7 +20,7 @@ hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double 
                           hipStream_t stream) {
     int n;
     const TileEntry<double> *tab = f64_tiles(&n);
-    return run_gemm_colmajor<double>(tab, n, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+    return run_gemm_colmajor<double>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
 }
 
 }  // namespace cba

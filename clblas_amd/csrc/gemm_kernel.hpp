@@ -28,12 +28,21 @@
 //     result runs along m, the contiguous direction of C.  The m coordinates are
 //     interleaved between blocks so that one 16-byte LDS read feeds VM blocks and one
 //     16-byte global store writes VM consecutive rows of C.
+//   * Complex types (interleaved re/im, src/library/blas/AutoGemm/KernelOpenCL.py:106-165)
+//     run on the same real MFMAs: the lane groups that a real MFMA spreads over consecutive
+//     k carry the real and the imaginary part of ONE k instead, so with the B-side operand
+//     (br | bi) a block of Re C accumulates from the A-side operand (ar | -ai) and the block
+//     of Im C from (ai | ar): two MFMAs per complex k and block, every MFMA flop useful.
+//     Lanes pick their part out of the (re, im) pair they read from LDS; conjugation is a
+//     sign flip of the imaginary lanes.
 #pragma once
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
 #include <type_traits>
+
+#include "internal.h"
 
 namespace cba {
 
@@ -44,14 +53,92 @@ typedef double f64x2 __attribute__((ext_vector_type(2)));
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-// Vector of N elements of T with only element alignment (global C may be misaligned by
-// offC / ldc) and with natural alignment (LDS).
+template <typename T> struct Elem { typedef T Real; static constexpr bool CPLX = false; };
+template <typename R> struct Elem<Cx<R>> { typedef R Real; static constexpr bool CPLX = true; };
+
+// Element arithmetic shared by the kernels.  The complex forms follow the operation order
+// of the reference's TYPE_MAD / TYPE_MAD_WRITE macros (KernelOpenCL.py:106-165).
+template <typename T> __host__ __device__ __forceinline__ T el_one() { return (T)1; }
+template <> __host__ __device__ __forceinline__ Cx<float> el_one<Cx<float>>() { return Cx<float>{1.f, 0.f}; }
+template <> __host__ __device__ __forceinline__ Cx<double> el_one<Cx<double>>() { return Cx<double>{1.0, 0.0}; }
+__host__ __device__ __forceinline__ bool el_is_zero(float x) { return x == 0.f; }
+__host__ __device__ __forceinline__ bool el_is_zero(double x) { return x == 0.0; }
+template <typename R> __host__ __device__ __forceinline__ bool el_is_zero(Cx<R> x) { return x.re == (R)0 && x.im == (R)0; }
+__device__ __forceinline__ float el_add(float a, float b) { return a + b; }
+__device__ __forceinline__ double el_add(double a, double b) { return a + b; }
+template <typename R> __device__ __forceinline__ Cx<R> el_add(Cx<R> a, Cx<R> b) { return Cx<R>{a.re + b.re, a.im + b.im}; }
+// alpha * x
+__device__ __forceinline__ float el_scale(float alpha, float x) { return alpha * x; }
+__device__ __forceinline__ double el_scale(double alpha, double x) { return alpha * x; }
+template <typename R> __device__ __forceinline__ Cx<R> el_scale(Cx<R> alpha, Cx<R> x) {
+    R re = x.re * alpha.re;
+    re = fma(-alpha.im, x.im, re);
+    R im = x.im * alpha.re;
+    im = fma(alpha.im, x.re, im);
+    return Cx<R>{re, im};
+}
+// r + beta * c
+__device__ __forceinline__ float el_axpy(float beta, float c, float r) { return r + beta * c; }
+__device__ __forceinline__ double el_axpy(double beta, double c, double r) { return r + beta * c; }
+template <typename R> __device__ __forceinline__ Cx<R> el_axpy(Cx<R> beta, Cx<R> c, Cx<R> r) {
+    R re = fma(beta.re, c.re, r.re);
+    re = fma(-beta.im, c.im, re);
+    R im = fma(beta.im, c.re, r.im);
+    im = fma(beta.re, c.im, im);
+    return Cx<R>{re, im};
+}
+// s + op(a) * op(b), op = conjugate where flagged (flags are ignored for real types)
+__device__ __forceinline__ float el_mad(float a, bool, float b, bool, float s) { return fmaf(a, b, s); }
+__device__ __forceinline__ double el_mad(double a, bool, double b, bool, double s) { return fma(a, b, s); }
+template <typename R> __device__ __forceinline__ Cx<R> el_mad(Cx<R> a, bool ca, Cx<R> b, bool cb, Cx<R> s) {
+    const R ai = ca ? -a.im : a.im, bi = cb ? -b.im : b.im;
+    R re = fma(a.re, b.re, s.re);
+    re = fma(-ai, bi, re);
+    R im = fma(a.re, bi, s.im);
+    im = fma(ai, b.re, im);
+    return Cx<R>{re, im};
+}
+
+// Vector of N elements of T: `type` with natural alignment (LDS), `utype` with only element
+// alignment (global C may be misaligned by offC / ldc); get/set address element e.
 template <typename T, int N> struct Vec;
-template <> struct Vec<float, 1> { typedef float type; typedef float utype; };
-template <> struct Vec<float, 2> { typedef f32x2 type; typedef float utype __attribute__((ext_vector_type(2), aligned(4))); };
-template <> struct Vec<float, 4> { typedef f32x4 type; typedef float utype __attribute__((ext_vector_type(4), aligned(4))); };
-template <> struct Vec<double, 1> { typedef double type; typedef double utype; };
-template <> struct Vec<double, 2> { typedef f64x2 type; typedef double utype __attribute__((ext_vector_type(2), aligned(8))); };
+template <> struct Vec<float, 1> {
+    typedef float type; typedef float utype;
+    template <typename V> static __device__ __forceinline__ float get(const V &v, int) { return v; }
+    template <typename V> static __device__ __forceinline__ void set(V &v, int, float x) { v = x; }
+};
+template <> struct Vec<double, 1> {
+    typedef double type; typedef double utype;
+    template <typename V> static __device__ __forceinline__ double get(const V &v, int) { return v; }
+    template <typename V> static __device__ __forceinline__ void set(V &v, int, double x) { v = x; }
+};
+#define CBA_REAL_VEC(T, N, BASE, ALIGN)                                                          \
+    template <> struct Vec<T, N> {                                                               \
+        typedef BASE type;                                                                       \
+        typedef T utype __attribute__((ext_vector_type(N), aligned(ALIGN)));                     \
+        template <typename V> static __device__ __forceinline__ T get(const V &v, int e) { return v[e]; }   \
+        template <typename V> static __device__ __forceinline__ void set(V &v, int e, T x) { v[e] = x; }    \
+    };
+CBA_REAL_VEC(float, 2, f32x2, 4)
+CBA_REAL_VEC(float, 4, f32x4, 4)
+CBA_REAL_VEC(double, 2, f64x2, 8)
+#undef CBA_REAL_VEC
+#define CBA_CPLX_VEC(R, N, BASE, ALIGN)                                                          \
+    template <> struct Vec<Cx<R>, N> {                                                           \
+        typedef BASE type;                                                                       \
+        typedef R utype __attribute__((ext_vector_type(2 * N), aligned(ALIGN)));                 \
+        template <typename V> static __device__ __forceinline__ Cx<R> get(const V &v, int e) {   \
+            return Cx<R>{v[2 * e], v[2 * e + 1]};                                                \
+        }                                                                                        \
+        template <typename V> static __device__ __forceinline__ void set(V &v, int e, Cx<R> x) { \
+            v[2 * e] = x.re;                                                                     \
+            v[2 * e + 1] = x.im;                                                                 \
+        }                                                                                        \
+    };
+CBA_CPLX_VEC(float, 1, f32x2, 4)
+CBA_CPLX_VEC(float, 2, f32x4, 4)
+CBA_CPLX_VEC(double, 1, f64x2, 8)
+#undef CBA_CPLX_VEC
 
 template <typename T> struct Mma;
 
@@ -89,6 +176,7 @@ template <typename T> struct GemmParams {
     int64_t lda, ldb, ldc;
     int64_t a_bytes, b_bytes;  // exact footprint of op-A / op-B storage, from A / B
     int M, N, K;
+    int conj_a, conj_b;  // complex types: conjugate op-A / op-B elements
     T alpha, beta;
     int tiles_m, tiles_n;
     int group_m;      // tile rows walked together (L2 locality)
@@ -191,15 +279,17 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
             const int place = lane % S, slot = place ^ swz(x);
 #pragma unroll
             for (int e = 0; e < VEC; ++e)
-                if (slot * VEC + e >= k_valid) lds[x * BK + place * VEC + e] = (T)0;
+                if (slot * VEC + e >= k_valid) lds[x * BK + place * VEC + e] = T();
         }
     }
 };
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC> struct GemmCfg {
-    typedef Mma<T> M;
+    typedef Mma<typename Elem<T>::Real> M;
+    static constexpr bool CPLX = Elem<T>::CPLX;
     static constexpr int VEC = 16 / (int)sizeof(T);
-    static constexpr int MB = M::MB, KS = M::KS, NACC = M::NACC;
+    // Complex: two lane groups (re, im) per k, so an MFMA covers half as many k.
+    static constexpr int MB = M::MB, KS = CPLX ? M::KS / 2 : M::KS, NACC = M::NACC;
     static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
     static constexpr int NT = 64 * WAVES_M * WAVES_N;
     static constexpr int TM = WM / MB, TN = WN / MB;
@@ -212,7 +302,7 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     // its rows instead); n is interleaved only for a k-major B panel.
     static constexpr bool A_KLAY = A_KC, B_KLAY = B_KC;
     static constexpr int VNM = B_KLAY ? 1 : VN;  // n interleave used by the fragment/epilogue mapping
-    static constexpr int NG = 64 / MB;           // lane groups along k
+    static constexpr int NG = KS;                // lane groups along k
     static_assert(BK % (VEC * NG) == 0, "panel depth must hold whole k groups");
     typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_DMA_K : LM_DMA_X, VM, MB> LoaderA;
     typedef PanelLoader<T, BN, BK, NT, B_KC ? LM_DMA_K : LM_DMA_X> LoaderB;
@@ -231,7 +321,10 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64, MINW)
 gemm_mfma_kernel(const GemmParams<T> p) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, A_KC, B_KC> Cfg;
-    typedef Mma<T> M;
+    typedef typename Elem<T>::Real R;
+    typedef Mma<R> M;
+    constexpr bool CPLX = Cfg::CPLX;
+    constexpr int NP = CPLX ? 2 : 1;  // MFMA accumulator blocks per C block (re, im)
     constexpr int MB = Cfg::MB, KS = Cfg::KS, NACC = Cfg::NACC;
     constexpr int TM = Cfg::TM, TN = Cfg::TN, VM = Cfg::VM, VN = Cfg::VN;
     constexpr int PITCH_A = Cfg::PITCH_A, PITCH_B = Cfg::PITCH_B, STAGE = Cfg::STAGE;
@@ -247,8 +340,31 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     const int wave = tid >> 6;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // same value, known to be wave-uniform
     const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
-    const int j = lane % MB;  // position along the block edge
-    const int g = lane / MB;  // k sub-step supplied by this lane
+    const int j = lane % MB;                            // position along the block edge
+    const int g = CPLX ? lane / (2 * MB) : lane / MB;  // k sub-step supplied by this lane
+    const int part = CPLX ? (lane / MB) & 1 : 0;        // complex: 0 = lane carries re, 1 = im
+    // Sign flips (on the sign bit) that turn the part a lane picked into its MFMA operand:
+    //   B side (br | bi'), A side for Re C (ar | -ai'), for Im C (ai' | ar), x' = conjugated.
+    const uint32_t sgn_b = (CPLX && part && p.conj_b) ? 0x80000000u : 0u;
+    const uint32_t sgn_an = (CPLX && part && !p.conj_a) ? 0x80000000u : 0u;
+    const uint32_t sgn_as = (CPLX && !part && p.conj_a) ? 0x80000000u : 0u;
+    auto flip = [](R x, uint32_t m) -> R {
+        if constexpr (sizeof(R) == 4) return __builtin_bit_cast(R, __builtin_bit_cast(uint32_t, x) ^ m);
+        else return __builtin_bit_cast(R, __builtin_bit_cast(uint64_t, x) ^ ((uint64_t)m << 32));
+    };
+    // Element read from LDS -> MFMA operand(s) of this lane.
+    auto ops_a = [&](T x, R (&o)[NP]) {
+        if constexpr (CPLX) {
+            o[0] = flip(part ? x.im : x.re, sgn_an);
+            o[1] = flip(part ? x.re : x.im, sgn_as);
+        } else {
+            o[0] = x;
+        }
+    };
+    auto op_b = [&](T x) -> R {
+        if constexpr (CPLX) return flip(part ? x.im : x.re, sgn_b);
+        else return x;
+    };
 
     // ---- tile assignment: contiguous chunk of the tile list per XCD, then walk
     //      `group_m` tile rows at a time so that concurrently running workgroups of one
@@ -290,13 +406,15 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     auto a_off = [&](int k0) -> int64_t { return A_KC ? (int64_t)m0 * p.lda + k0 : (int64_t)k0 * p.lda + m0; };
     auto b_off = [&](int k0) -> int64_t { return B_KC ? (int64_t)n0 * p.ldb + k0 : (int64_t)k0 * p.ldb + n0; };
 
-    typename M::Acc acc[TN][TM];
+    typename M::Acc acc[TN][TM][NP];
 #pragma unroll
     for (int bn = 0; bn < TN; ++bn)
 #pragma unroll
         for (int bm = 0; bm < TM; ++bm)
 #pragma unroll
-            for (int v = 0; v < NACC; ++v) acc[bn][bm][v] = (T)0;
+            for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+                for (int v = 0; v < NACC; ++v) acc[bn][bm][pp][v] = (R)0;
 
     if (n_panels > 0) {
         // Software pipeline over panels: a ring of NSTAGE LDS stages, loads issued DEPTH =
@@ -350,35 +468,29 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             // i.e. VEC consecutive steps walk VEC consecutive k: a k-major panel row is read
             // per step, a [x][k] panel is read as one 16-byte vector per VEC steps.
             // Fragments are read one step (one VEC-step group for [x][k]) ahead of their use.
-            T a[2][TM], b[2][TN], ak[2][TM][VEC], bk[2][TN][VEC];
+            R a[2][TM][NP], b[2][TN], ak[2][TM][VEC][NP], bk[2][TN][VEC];
             auto kmap = [&](int s) { return (s / VEC) * (VEC * NG) + g * VEC + (s % VEC); };
-            auto read_a = [&](int s, T (&af)[TM]) {  // k-major A panel
+            auto read_a = [&](int s, R (&af)[TM][NP]) {  // k-major A panel
                 const int krow = kmap(s);
 #pragma unroll
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     typename Vec<T, VM>::type av =
                         *reinterpret_cast<const typename Vec<T, VM>::type *>(&As[LA::lds_at(krow, a_frag + ga * MB * VM)]);
-                    if constexpr (VM == 1) af[ga] = av;
-                    else {
 #pragma unroll
-                        for (int e = 0; e < VM; ++e) af[ga * VM + e] = av[e];
-                    }
+                    for (int e = 0; e < VM; ++e) ops_a(Vec<T, VM>::get(av, e), af[ga * VM + e]);
                 }
             };
-            auto read_b = [&](int s, T (&bf)[TN]) {  // k-major B panel
+            auto read_b = [&](int s, R (&bf)[TN]) {  // k-major B panel
                 const int krow = kmap(s);
 #pragma unroll
                 for (int gb = 0; gb < TN / VN; ++gb) {
                     typename Vec<T, VN>::type bv =
                         *reinterpret_cast<const typename Vec<T, VN>::type *>(&Bs[LB::lds_at(krow, b_frag + gb * MB * VN)]);
-                    if constexpr (VN == 1) bf[gb] = bv;
-                    else {
 #pragma unroll
-                        for (int e = 0; e < VN; ++e) bf[gb * VN + e] = bv[e];
-                    }
+                    for (int e = 0; e < VN; ++e) bf[gb * VN + e] = op_b(Vec<T, VN>::get(bv, e));
                 }
             };
-            auto read_ak = [&](int grp, T (&af)[TM][VEC]) {  // [m'][k] A panel, VEC steps at once
+            auto read_ak = [&](int grp, R (&af)[TM][VEC][NP]) {  // [m'][k] A panel, VEC steps at once
 #pragma unroll
                 for (int bm = 0; bm < TM; ++bm) {
                     const int m_img = wm * WM + bm * MB + j;  // image row of block bm, lane j
@@ -386,10 +498,10 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     typename Vec<T, VEC>::type av =
                         *reinterpret_cast<const typename Vec<T, VEC>::type *>(&As[m_img * PITCH_A + place * VEC]);
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) af[bm][e] = av[e];
+                    for (int e = 0; e < VEC; ++e) ops_a(Vec<T, VEC>::get(av, e), af[bm][e]);
                 }
             };
-            auto read_bk = [&](int grp, T (&bf)[TN][VEC]) {  // [n][k] B panel, VEC steps at once
+            auto read_bk = [&](int grp, R (&bf)[TN][VEC]) {  // [n][k] B panel, VEC steps at once
 #pragma unroll
                 for (int bn = 0; bn < TN; ++bn) {
                     const int n_loc = wn * WN + bn * MB + j;
@@ -397,7 +509,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     typename Vec<T, VEC>::type bv =
                         *reinterpret_cast<const typename Vec<T, VEC>::type *>(&Bs[n_loc * PITCH_B + place * VEC]);
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) bf[bn][e] = bv[e];
+                    for (int e = 0; e < VEC; ++e) bf[bn][e] = op_b(Vec<T, VEC>::get(bv, e));
                 }
             };
             if constexpr (A_KLAY) read_ak(0, ak[0]); else read_a(0, a[0]);
@@ -419,11 +531,14 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int bn = 0; bn < TN; ++bn) {
-                    const T bval = B_KLAY ? bk[(s / VEC) & 1][bn][s % VEC] : b[s & 1][bn];
+                    const R bval = B_KLAY ? bk[(s / VEC) & 1][bn][s % VEC] : b[s & 1][bn];
 #pragma unroll
                     for (int bm = 0; bm < TM; ++bm) {
-                        const T aval = A_KLAY ? ak[(s / VEC) & 1][bm][s % VEC] : a[s & 1][bm];
-                        acc[bn][bm] = M::run(bval, aval, acc[bn][bm]);
+#pragma unroll
+                        for (int pp = 0; pp < NP; ++pp) {
+                            const R aval = A_KLAY ? ak[(s / VEC) & 1][bm][s % VEC][pp] : a[s & 1][bm][pp];
+                            acc[bn][bm][pp] = M::run(bval, aval, acc[bn][bm][pp]);
+                        }
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -445,15 +560,20 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     if (SPLITK) {
         Cout = p.ws + (int64_t)blockIdx.y * p.ws_slice;
         ldc = p.ws_ld;
-        alpha = (T)1;
-        beta = (T)0;
+        alpha = el_one<T>();
+        beta = T();
     }
-    const bool read_c = !(beta == (T)0);
+    const bool read_c = !el_is_zero(beta);
+    auto acc_elem = [&](int bn, int bm, int v) -> T {
+        if constexpr (CPLX) return T{acc[bn][bm][0][v], acc[bn][bm][1][v]};
+        else return acc[bn][bm][0][v];
+    };
 
     // C is read in batches of CH accumulator rows per lane before any of them is written
     // back, so that the load latencies of a batch overlap instead of queueing behind each
     // store (loads and stores go to the same array, so the compiler keeps their order).
-    typedef typename Vec<T, VM>::utype UV;
+    typedef Vec<T, VM> VC;
+    typedef typename VC::utype UV;
     constexpr int CH = NACC < 8 ? NACC : 8;
 #pragma unroll
     for (int bn = 0; bn < TN; ++bn) {
@@ -482,29 +602,20 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     const int m = m0 + wm * WM + ga * (MB * VM) + j * VM;
                     if (m + VM <= p.M) {
-                        T r[VM];
+                        UV ov;
 #pragma unroll
                         for (int e = 0; e < VM; ++e) {
-                            r[e] = alpha * acc[bn][ga * VM + e][v];
-                            if (read_c) {
-                                T c_old;
-                                if constexpr (VM == 1) c_old = cold[dv][ga]; else c_old = cold[dv][ga][e];
-                                r[e] += beta * c_old;
-                            }
-                        }
-                        UV ov;
-                        if constexpr (VM == 1) ov = r[0];
-                        else {
-#pragma unroll
-                            for (int e = 0; e < VM; ++e) ov[e] = r[e];
+                            T r = el_scale(alpha, acc_elem(bn, ga * VM + e, v));
+                            if (read_c) r = el_axpy(beta, VC::get(cold[dv][ga], e), r);
+                            VC::set(ov, e, r);
                         }
                         *reinterpret_cast<UV *>(col + m) = ov;
                     } else {
 #pragma unroll
                         for (int e = 0; e < VM; ++e) {
                             if (m + e < p.M) {
-                                T r = alpha * acc[bn][ga * VM + e][v];
-                                if (read_c) r += beta * col[m + e];
+                                T r = el_scale(alpha, acc_elem(bn, ga * VM + e, v));
+                                if (read_c) r = el_axpy(beta, col[m + e], r);
                                 col[m + e] = r;
                             }
                         }
@@ -524,11 +635,11 @@ splitk_reduce_kernel(const T *ws, int64_t ws_ld, int64_t ws_slice, int splits, i
     const int m = (blockIdx.x % m_blocks) * 256 + threadIdx.x;
     const int n = blockIdx.x / m_blocks;
     if (m >= M || n >= N) return;
-    T s = (T)0;
-    for (int i = 0; i < splits; ++i) s += ws[(int64_t)i * ws_slice + (int64_t)n * ws_ld + m];
+    T s = T();
+    for (int i = 0; i < splits; ++i) s = el_add(s, ws[(int64_t)i * ws_slice + (int64_t)n * ws_ld + m]);
     T *c = C + (int64_t)n * ldc + m;
-    T r = alpha * s;
-    if (!(beta == (T)0)) r += beta * *c;
+    T r = el_scale(alpha, s);
+    if (!el_is_zero(beta)) r = el_axpy(beta, *c, r);
     *c = r;
 }
 
@@ -539,27 +650,27 @@ __global__ void __launch_bounds__(256) scale_c_kernel(int M, int N, int m_blocks
     const int n = blockIdx.x / m_blocks;
     if (m >= M || n >= N) return;
     T *c = C + (int64_t)n * ldc + m;
-    *c = (beta == (T)0) ? (T)0 : beta * *c;
+    *c = el_is_zero(beta) ? T() : el_scale(beta, *c);
 }
 
 // Plain kernel with 64-bit indexing for leading dimensions too large for the 32-bit
 // panel offsets of the MFMA kernel.  Same contract; one thread per C element.
 template <typename T>
 __global__ void __launch_bounds__(256)
-gemm_wide_ld_kernel(int transA, int transB, int M, int N, int K, int m_blocks, T alpha, const T *A, int64_t lda,
-                    const T *B, int64_t ldb, T beta, T *C, int64_t ldc) {
+gemm_wide_ld_kernel(int transA, int transB, int conjA, int conjB, int M, int N, int K, int m_blocks, T alpha,
+                    const T *A, int64_t lda, const T *B, int64_t ldb, T beta, T *C, int64_t ldc) {
     const int64_t m = (int64_t)(blockIdx.x % m_blocks) * 256 + threadIdx.x;
     const int64_t n = blockIdx.x / m_blocks;
     if (m >= M || n >= N) return;
-    T s = (T)0;
+    T s = T();
     for (int64_t k = 0; k < K; ++k) {
         T a = transA ? A[k + m * lda] : A[m + k * lda];
         T b = transB ? B[n + k * ldb] : B[k + n * ldb];
-        s = fma(a, b, s);
+        s = el_mad(a, conjA != 0, b, conjB != 0, s);
     }
     T *c = C + n * ldc + m;
-    T r = alpha * s;
-    if (!(beta == (T)0)) r += beta * *c;
+    T r = el_scale(alpha, s);
+    if (!el_is_zero(beta)) r = el_axpy(beta, *c, r);
     *c = r;
 }
 

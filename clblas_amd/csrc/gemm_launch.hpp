@@ -91,9 +91,9 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
 }
 
 template <typename T>
-static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, bool tB, int M, int N, int K,
-                                    T alpha, const T *A, int64_t lda, const T *B, int64_t ldb, T beta, T *C,
-                                    int64_t ldc, hipStream_t stream) {
+static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, bool tB, bool cA, bool cB, int M,
+                                    int N, int K, T alpha, const T *A, int64_t lda, const T *B, int64_t ldb,
+                                    T beta, T *C, int64_t ldc, hipStream_t stream) {
     if (K == 0) {
         int mb = (int)ceil_div64(M, 256);
         hipLaunchKernelGGL(scale_c_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
@@ -106,7 +106,8 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     if (lda > ld_limit || ldb > ld_limit) {
         int mb = (int)ceil_div64(M, 256);
         hipLaunchKernelGGL(gemm_wide_ld_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream,
-                           tA ? 1 : 0, tB ? 1 : 0, M, N, K, mb, alpha, A, lda, B, ldb, beta, C, ldc);
+                           tA ? 1 : 0, tB ? 1 : 0, cA ? 1 : 0, cB ? 1 : 0, M, N, K, mb, alpha, A, lda, B, ldb, beta, C,
+                           ldc);
         return hipGetLastError();
     }
 
@@ -121,6 +122,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     p.a_bytes = (tA ? ((int64_t)(M - 1) * lda + K) : ((int64_t)(K - 1) * lda + M)) * (int64_t)sizeof(T);
     p.b_bytes = (tB ? ((int64_t)(K - 1) * ldb + N) : ((int64_t)(N - 1) * ldb + K)) * (int64_t)sizeof(T);
     p.M = M; p.N = N; p.K = K;
+    p.conj_a = cA ? 1 : 0; p.conj_b = cB ? 1 : 0;
     p.alpha = alpha; p.beta = beta;
     p.tiles_m = (int)ceil_div64(M, e.bm);
     p.tiles_n = (int)ceil_div64(N, e.bn);

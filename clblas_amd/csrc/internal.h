@@ -8,6 +8,10 @@
 
 namespace cba {
 
+// Complex element, laid out as the reference's FloatComplex / DoubleComplex (cl_float2 /
+// cl_double2, src/clBLAS-complex.h:25-26: real part first).
+template <typename R> struct Cx { R re, im; };
+
 // Debug-only override of the GEMM tile choice: index into the per-type tile table taken
 // from the environment variable CLBLAS_AMD_GEMM_TILE, or -1.
 int forced_gemm_tile();
@@ -31,6 +35,14 @@ hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float a
 hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double alpha, const double *A,
                           int64_t lda, const double *B, int64_t ldb, double beta, double *C, int64_t ldc,
                           hipStream_t stream);
+
+// Complex variants: conjA / conjB conjugate the elements of op(A) / op(B) (clblasConjTrans).
+hipError_t cgemm_colmajor(bool transA, bool transB, bool conjA, bool conjB, int M, int N, int K, Cx<float> alpha,
+                          const Cx<float> *A, int64_t lda, const Cx<float> *B, int64_t ldb, Cx<float> beta,
+                          Cx<float> *C, int64_t ldc, hipStream_t stream);
+hipError_t zgemm_colmajor(bool transA, bool transB, bool conjA, bool conjB, int M, int N, int K, Cx<double> alpha,
+                          const Cx<double> *A, int64_t lda, const Cx<double> *B, int64_t ldb, Cx<double> beta,
+                          Cx<double> *C, int64_t ldc, hipStream_t stream);
 
 // Column-major TRSM drivers (same conventions).
 hipError_t strsm_colmajor(bool right, bool lower, bool trans, bool unit, int M, int N, float alpha, const float *A,

@@ -88,6 +88,12 @@ typedef enum clblasStatus_ {
     clblasInsufficientMemVecY = -1007
 } clblasStatus;
 
+/* Complex scalars and matrix elements: real part in s[0], imaginary part in s[1].
+ * Same size, alignment, element order and by-value calling convention as the reference's
+ * FloatComplex / DoubleComplex (src/clBLAS-complex.h:25-26: cl_float2 / cl_double2). */
+typedef struct FloatComplex_ { float s[2]; } __attribute__((aligned(8))) FloatComplex;
+typedef struct DoubleComplex_ { double s[2]; } __attribute__((aligned(16))) DoubleComplex;
+
 /* Replaces clblasGetVersion (src/clBLAS.h:176-177, src/library/blas/init.c:33-41).
  * Reports this library's own version. Always clblasSuccess. */
 clblasStatus clblasGetVersion(unsigned int *major, unsigned int *minor, unsigned int *patch);
@@ -118,6 +124,25 @@ clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          const double *A, size_t offA, size_t lda,
                          const double *B, size_t offB, size_t ldb, double beta,
                          double *C, size_t offC, size_t ldc, hipStream_t stream);
+
+/* Replaces clblasCgemm (src/clBLAS.h:7538-7561, src/library/blas/xgemm.cc:788-845).
+ *   C <- alpha * op(A) * op(B) + beta * C, complex fp32; clblasConjTrans is the conjugate
+ * transpose.  beta == 0+0i means C is not read.  Arithmetic follows the complex TYPE_MAD /
+ * TYPE_MAD_WRITE of AutoGemm/KernelOpenCL.py:106-165.  Validation as clblasSgemm.
+ * Matrices need only 4-byte alignment. */
+clblasStatus clblasCgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB,
+                         size_t M, size_t N, size_t K, FloatComplex alpha,
+                         const FloatComplex *A, size_t offA, size_t lda,
+                         const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta,
+                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream);
+
+/* Replaces clblasZgemm (src/clBLAS.h:7622-7645, src/library/blas/xgemm.cc:850-905).
+ * Matrices need only 8-byte alignment. */
+clblasStatus clblasZgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB,
+                         size_t M, size_t N, size_t K, DoubleComplex alpha,
+                         const DoubleComplex *A, size_t offA, size_t lda,
+                         const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
+                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream);
 
 /* Replaces clblasStrsm (src/clBLAS.h:7988-8008, src/library/blas/xtrsm.cc:1600-1661).
  *   side == Left : solve op(A) * X = alpha * B,  A is M x M

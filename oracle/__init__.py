@@ -48,6 +48,14 @@ def lib():
             f = getattr(L, name)
             f.restype = None
             f.argtypes = [_i, _i, _sz, real, _vp, _sz, _vp, _sz, real, _vp, _sz, _sz, _vp, _vp, _vp, _vp]
+        for name in ("oracle_cgemm", "oracle_zgemm"):
+            f = getattr(L, name)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _sz, _sz]
+        for name in ("oracle_cgemm_exact", "oracle_zgemm_exact"):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_i, _i, _i, _i, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _vp, _vp]
         for name, real in (("oracle_strsm_naive", ctypes.c_float), ("oracle_dtrsm_naive", ctypes.c_double),
                            ("oracle_strsm_blocked", ctypes.c_float), ("oracle_dtrsm_blocked", ctypes.c_double)):
             f = getattr(L, name)
@@ -87,6 +95,10 @@ def ref_lib():
             f = getattr(L, name)
             f.restype = None
             f.argtypes = [_i, _i, _i, _sz, _sz, _sz, real, _vp, _sz, _vp, _sz, real, _vp, _sz]
+        for name in ("ref_naive_cgemm", "ref_naive_zgemm"):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_i, _i, _i, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz]
         for name, real in (("ref_naive_strsm", ctypes.c_float), ("ref_naive_dtrsm", ctypes.c_double)):
             f = getattr(L, name)
             f.restype = None
@@ -107,9 +119,25 @@ def num_threads():
     return lib().oracle_num_threads()
 
 
+def _is_complex(a):
+    return a.dtype in (np.complex64, np.complex128)
+
+
+def _scalar(x, dtype):
+    """(re, im) of a Python complex as a 2-element real array matching complex `dtype`."""
+    z = complex(x)
+    return np.array([z.real, z.imag], dtype=np.float32 if dtype == np.complex64 else np.float64)
+
+
 def gemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
-    """In-place on C (1-D buffer). Returns the clblasStatus the reference would return."""
+    """In-place on C (1-D buffer). Returns the clblasStatus the reference would return.
+    complex64 / complex128 buffers select the complex routines (alpha, beta: Python complex)."""
     ref = C if C is not None else (A if A is not None else B)
+    if _is_complex(ref):
+        f = lib().oracle_cgemm if ref.dtype == np.complex64 else lib().oracle_zgemm
+        al, be = _scalar(alpha, ref.dtype), _scalar(beta, ref.dtype)
+        return f(int(order), int(transA), int(transB), M, N, K, _p(al), _p(A), offA, lda, _p(B), offB, ldb, _p(be),
+                 _p(C), offC, ldc)
     f = lib().oracle_sgemm if ref.dtype == np.float32 else lib().oracle_dgemm
     return f(int(order), int(transA), int(transB), M, N, K, alpha, _p(A), offA, lda, _p(B), offB, ldb, beta, _p(C),
              offC, ldc)
@@ -120,8 +148,16 @@ def gemm_exact(transA, transB, K, alpha, A, lda, B, ldb, beta, C, ldc, rows, col
     float64 for the listed elements: magnitude = |alpha| sum|a b| + |beta c|."""
     rows = np.ascontiguousarray(rows, dtype=np.int64)
     cols = np.ascontiguousarray(cols, dtype=np.int64)
-    exact = np.empty(rows.size, dtype=np.float64)
     mag = np.empty(rows.size, dtype=np.float64)
+    if _is_complex(A):
+        # transA / transB: 0 none, 1 transpose, 2 conjugate transpose; exact is complex128.
+        ex = np.empty(2 * rows.size, dtype=np.float64)
+        f = lib().oracle_cgemm_exact if A.dtype == np.complex64 else lib().oracle_zgemm_exact
+        al, be = _scalar(alpha, A.dtype), _scalar(beta, A.dtype)
+        f(int(transA != 0), int(transA == 2), int(transB != 0), int(transB == 2), K, _p(al), _p(A), lda, _p(B), ldb,
+          _p(be), _p(C), ldc, rows.size, _p(rows), _p(cols), _p(ex), _p(mag))
+        return ex.view(np.complex128), mag
+    exact = np.empty(rows.size, dtype=np.float64)
     f = lib().oracle_sgemm_exact if A.dtype == np.float32 else lib().oracle_dgemm_exact
     f(int(bool(transA)), int(bool(transB)), K, alpha, _p(A), lda, _p(B), ldb, beta, _p(C), ldc, rows.size, _p(rows),
       _p(cols), _p(exact), _p(mag))
@@ -155,6 +191,11 @@ def check_trsm(order, side, transA, M, N, haveA, offA, lda, memA, haveB, offB, l
 
 def ref_gemm(order, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc):
     """Reference naive gemm (no offsets: pass views that start at the first element)."""
+    if _is_complex(C):
+        f = ref_lib().ref_naive_cgemm if C.dtype == np.complex64 else ref_lib().ref_naive_zgemm
+        al, be = _scalar(alpha, C.dtype), _scalar(beta, C.dtype)
+        f(int(order), int(transA), int(transB), M, N, K, _p(al), _p(A), lda, _p(B), ldb, _p(be), _p(C), ldc)
+        return
     f = ref_lib().ref_naive_sgemm if C.dtype == np.float32 else ref_lib().ref_naive_dgemm
     f(int(order), int(transA), int(transB), M, N, K, alpha, _p(A), lda, _p(B), ldb, beta, _p(C), ldc)
 
@@ -167,6 +208,9 @@ def ref_trsm(order, side, uplo, transA, diag, M, N, alpha, A, lda, B, ldb):
 # ---- seeded generators -------------------------------------------------------------------
 
 def uniform(n, seed, dtype=np.float32):
+    if dtype in (np.complex64, np.complex128):  # re and im drawn as 2n reals
+        real = np.float32 if dtype == np.complex64 else np.float64
+        return uniform(2 * n, seed, real).view(dtype)
     x = np.empty(n, dtype=dtype)
     (lib().oracle_fill_uniform_f32 if dtype == np.float32 else lib().oracle_fill_uniform_f64)(_p(x), n, seed)
     return x
@@ -179,6 +223,9 @@ def normal(n, seed, dtype=np.float64):
 
 
 def integers(n, seed, limit, dtype=np.float32):
+    if dtype in (np.complex64, np.complex128):  # Gaussian integers
+        real = np.float32 if dtype == np.complex64 else np.float64
+        return integers(2 * n, seed, limit, real).view(dtype)
     x = np.empty(n, dtype=dtype)
     (lib().oracle_fill_int_f32 if dtype == np.float32 else lib().oracle_fill_int_f64)(_p(x), n, seed, limit)
     return x

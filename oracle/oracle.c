@@ -16,6 +16,11 @@
  *                             reference's own naive gemm compiled from
  *                             src/library/tools/ktest/naive/naive_blas.cpp (oracle/_ref).
  *   oracle_{s,d}gemm_exact  - same integer-exact inputs (must reproduce them exactly).
+ *   oracle_{c,z}gemm(_exact)- Gaussian-integer inputs against exact integer products for every
+ *                             order / transpose / conjugate combination; closed forms (i*i,
+ *                             identity, Hermitian products have real diagonals, alpha / beta
+ *                             rotations by i); conjugation identities; the reference's own
+ *                             naive complex gemm (oracle/_ref).
  *   oracle_{s,d}trsm_naive  - TRSM_extratest closed form (src/tests/correctness/corr-trsm.cpp:
  *                             240-452, X_r = r+1); src/samples/example_strsm.c:30-63 fixed
  *                             input; oracle/_ref naive trsm; residual identities.
@@ -227,6 +232,143 @@ GEMM_FRONT(oracle_dgemm, double, dgemm_colmajor)
 
 GEMM_EXACT(oracle_sgemm_exact, float, double, fabs)
 GEMM_EXACT(oracle_dgemm_exact, double, long double, fabsl)
+
+/* Complex GEMM (clblasCgemm / clblasZgemm, src/library/blas/xgemm.cc:788-905).  Elements are
+ * interleaved (re, im) pairs, as cl_float2 / cl_double2 (src/clBLAS-complex.h:25-26).
+ * Column-major kernel arithmetic, src/library/blas/AutoGemm/KernelOpenCL.py:
+ *   :106-141  TYPE_MAD, four mads per k in this order (x' = imaginary part negated when the
+ *             operand is conjugated; the four macro variants differ only in where the minus
+ *             signs sit, which is exact):
+ *                 s0 = mad( a0,  b0, s0);  s0 = mad(-a1', b1', s0);
+ *                 s1 = mad( a0, b1', s1);  s1 = mad( a1', b0,  s1);
+ *   :142-165  TYPE_MAD_WRITE: reg = alpha*reg as  r0 = reg0*al0; r0 = mad(-al1, reg1, r0);
+ *             r1 = reg1*al0; r1 = mad(al1, reg0, r1);  then (beta != 0 only)
+ *             r0 = mad(be0, c0, r0); r0 = mad(-be1, c1, r0); r1 = mad(be1, c0, r1);
+ *             r1 = mad(be0, c1, r1).
+ * beta == 0+0i never reads C (isZero<FloatComplex>, xgemm.cc:94-101). */
+#define CGEMM_COLMAJOR(NAME, R, FMA)                                                                         \
+    static void NAME(int tA, int cA, int tB, int cB, size_t M, size_t N, size_t K, const R *alpha,          \
+                     const R *A, size_t lda, const R *B, size_t ldb, const R *beta, R *C, size_t ldc) {     \
+        const size_t MBLK = 64;                                                                              \
+        ptrdiff_t nb;                                                                                        \
+        const ptrdiff_t n_mblk = (ptrdiff_t)((M + MBLK - 1) / MBLK);                                         \
+        const int beta_zero = beta[0] == (R)0 && beta[1] == (R)0;                                            \
+        _Pragma("omp parallel for schedule(dynamic, 1)")                                                     \
+        for (nb = 0; nb < n_mblk; ++nb) {                                                                    \
+            const size_t m0 = (size_t)nb * MBLK;                                                             \
+            const size_t mlen = (M - m0) < MBLK ? (M - m0) : MBLK;                                           \
+            R s0[64], s1[64], a0[64], a1[64];                                                                \
+            size_t n, k, i;                                                                                  \
+            for (n = 0; n < N; ++n) {                                                                        \
+                for (i = 0; i < mlen; ++i) s0[i] = s1[i] = (R)0;                                             \
+                for (k = 0; k < K; ++k) {                                                                    \
+                    const R *bp = tB ? B + 2 * (n + k * ldb) : B + 2 * (k + n * ldb);                        \
+                    const R b0 = bp[0], b1 = cB ? -bp[1] : bp[1];                                            \
+                    for (i = 0; i < mlen; ++i) {                                                             \
+                        const R *ap = tA ? A + 2 * (k + (m0 + i) * lda) : A + 2 * (m0 + i + k * lda);        \
+                        a0[i] = ap[0];                                                                       \
+                        a1[i] = cA ? -ap[1] : ap[1];                                                         \
+                    }                                                                                        \
+                    _Pragma("omp simd")                                                                      \
+                    for (i = 0; i < mlen; ++i) {                                                             \
+                        s0[i] = FMA(a0[i], b0, s0[i]);                                                       \
+                        s0[i] = FMA(-a1[i], b1, s0[i]);                                                      \
+                        s1[i] = FMA(a0[i], b1, s1[i]);                                                       \
+                        s1[i] = FMA(a1[i], b0, s1[i]);                                                       \
+                    }                                                                                        \
+                }                                                                                            \
+                for (i = 0; i < mlen; ++i) {                                                                 \
+                    R *cp = C + 2 * (m0 + i + n * ldc);                                                      \
+                    R r0 = s0[i] * alpha[0], r1;                                                             \
+                    r0 = FMA(-alpha[1], s1[i], r0);                                                          \
+                    r1 = s1[i] * alpha[0];                                                                   \
+                    r1 = FMA(alpha[1], s0[i], r1);                                                           \
+                    if (!beta_zero) {                                                                        \
+                        const R c0 = cp[0], c1 = cp[1];                                                      \
+                        r0 = FMA(beta[0], c0, r0);                                                           \
+                        r0 = FMA(-beta[1], c1, r0);                                                          \
+                        r1 = FMA(beta[1], c0, r1);                                                           \
+                        r1 = FMA(beta[0], c1, r1);                                                           \
+                    }                                                                                        \
+                    cp[0] = r0;                                                                              \
+                    cp[1] = r1;                                                                              \
+                }                                                                                            \
+            }                                                                                                \
+        }                                                                                                    \
+    }
+
+CGEMM_COLMAJOR(cgemm_colmajor, float, fmaf)
+CGEMM_COLMAJOR(zgemm_colmajor, double, fma)
+
+/* Front end: checks as for the real types (xgemm.cc:807-829), ConjTrans kept
+ * (correctTranspose is the identity for complex types, xgemm.cc:334-335), row-major folded
+ * by swapping the operands together with their transpose flags (xgemm.cc:40-61).
+ * alpha / beta point at (re, im); A, B, C at interleaved elements; offsets and leading
+ * dimensions count complex elements. */
+#define CGEMM_FRONT(NAME, R, CORE)                                                                           \
+    int NAME(int order, int transA, int transB, size_t M, size_t N, size_t K, const R *alpha, const R *A,   \
+             size_t offA, size_t lda, const R *B, size_t offB, size_t ldb, const R *beta, R *C, size_t offC, \
+             size_t ldc) {                                                                                   \
+        int st = oracle_check_gemm(order, transA, transB, M, N, K, A != NULL, offA, lda, 0, B != NULL, offB, \
+                                   ldb, 0, C != NULL, offC, ldc, 0);                                         \
+        int tA, tB, cA, cB;                                                                                  \
+        if (st) return st;                                                                                   \
+        tA = transA != NO_TRANS;                                                                             \
+        tB = transB != NO_TRANS;                                                                             \
+        cA = transA == CONJ_TRANS;                                                                           \
+        cB = transB == CONJ_TRANS;                                                                           \
+        if (order == ROW_MAJOR)                                                                              \
+            CORE(tB, cB, tA, cA, N, M, K, alpha, B + 2 * offB, ldb, A + 2 * offA, lda, beta, C + 2 * offC,   \
+                 ldc);                                                                                       \
+        else                                                                                                 \
+            CORE(tA, cA, tB, cB, M, N, K, alpha, A + 2 * offA, lda, B + 2 * offB, ldb, beta, C + 2 * offC,   \
+                 ldc);                                                                                       \
+        return ST_SUCCESS;                                                                                   \
+    }
+
+CGEMM_FRONT(oracle_cgemm, float, cgemm_colmajor)
+CGEMM_FRONT(oracle_zgemm, double, zgemm_colmajor)
+
+/* Complex counterpart of the high-precision yardstick above.  exact[2i], exact[2i+1]: real
+ * and imaginary part; mag[i] bounds the magnitude of everything summed into either part:
+ *   (|al0|+|al1|) * sum_k (|a0|+|a1|)(|b0|+|b1|) + (|be0|+|be1|)(|c0|+|c1|). */
+#define CGEMM_EXACT(NAME, R, W, ABSW)                                                                        \
+    void NAME(int tA, int cA, int tB, int cB, size_t K, const R *alpha, const R *A, size_t lda, const R *B, \
+              size_t ldb, const R *beta, const R *C, size_t ldc, size_t count, const int64_t *rows,          \
+              const int64_t *cols, double *exact, double *mag) {                                             \
+        ptrdiff_t i;                                                                                         \
+        const int beta_zero = beta[0] == (R)0 && beta[1] == (R)0;                                            \
+        _Pragma("omp parallel for schedule(static)")                                                         \
+        for (i = 0; i < (ptrdiff_t)count; ++i) {                                                             \
+            const size_t m = (size_t)rows[i], n = (size_t)cols[i];                                           \
+            W s0 = 0, s1 = 0, sa = 0, r0, r1, g;                                                             \
+            size_t k;                                                                                        \
+            for (k = 0; k < K; ++k) {                                                                        \
+                const R *ap = tA ? A + 2 * (k + m * lda) : A + 2 * (m + k * lda);                            \
+                const R *bp = tB ? B + 2 * (n + k * ldb) : B + 2 * (k + n * ldb);                            \
+                const W a0 = ap[0], a1 = cA ? -(W)ap[1] : (W)ap[1];                                          \
+                const W b0 = bp[0], b1 = cB ? -(W)bp[1] : (W)bp[1];                                          \
+                s0 += a0 * b0 - a1 * b1;                                                                     \
+                s1 += a0 * b1 + a1 * b0;                                                                     \
+                sa += (ABSW(a0) + ABSW(a1)) * (ABSW(b0) + ABSW(b1));                                         \
+            }                                                                                                \
+            r0 = (W)alpha[0] * s0 - (W)alpha[1] * s1;                                                        \
+            r1 = (W)alpha[0] * s1 + (W)alpha[1] * s0;                                                        \
+            g = (ABSW((W)alpha[0]) + ABSW((W)alpha[1])) * sa;                                                \
+            if (!beta_zero) {                                                                                \
+                const W c0 = C[2 * (m + n * ldc)], c1 = C[2 * (m + n * ldc) + 1];                            \
+                r0 += (W)beta[0] * c0 - (W)beta[1] * c1;                                                     \
+                r1 += (W)beta[0] * c1 + (W)beta[1] * c0;                                                     \
+                g += (ABSW((W)beta[0]) + ABSW((W)beta[1])) * (ABSW(c0) + ABSW(c1));                          \
+            }                                                                                                \
+            exact[2 * i] = (double)r0;                                                                       \
+            exact[2 * i + 1] = (double)r1;                                                                   \
+            mag[i] = (double)g;                                                                              \
+        }                                                                                                    \
+    }
+
+CGEMM_EXACT(oracle_cgemm_exact, float, double, fabs)
+CGEMM_EXACT(oracle_zgemm_exact, double, long double, fabsl)
 
 /* ------------------------------------------------------------------------------------ */
 /* TRSM                                                                                  */

@@ -31,6 +31,29 @@ void ref_naive_dgemm(int order, int transA, int transB, size_t M, size_t N, size
                             (NaiveBlas::clblasTranspose)transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
 }
 
+// Complex: alpha / beta are passed by address (re, im); matrices are interleaved pairs with
+// the layout of FloatComplex / DoubleComplex.
+void ref_naive_cgemm(int order, int transA, int transB, size_t M, size_t N, size_t K, const float *alpha,
+                     const void *A, size_t lda, const void *B, size_t ldb, const float *beta, void *C, size_t ldc) {
+    NaiveBlas::FloatComplex al, be;
+    al.s[0] = alpha[0]; al.s[1] = alpha[1];
+    be.s[0] = beta[0]; be.s[1] = beta[1];
+    NaiveBlas::gemm<NaiveBlas::FloatComplex>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasTranspose)transA,
+                                  (NaiveBlas::clblasTranspose)transB, M, N, K, al, (const NaiveBlas::FloatComplex *)A, lda,
+                                  (const NaiveBlas::FloatComplex *)B, ldb, be, (NaiveBlas::FloatComplex *)C, ldc);
+}
+
+void ref_naive_zgemm(int order, int transA, int transB, size_t M, size_t N, size_t K, const double *alpha,
+                     const void *A, size_t lda, const void *B, size_t ldb, const double *beta, void *C,
+                     size_t ldc) {
+    NaiveBlas::DoubleComplex al, be;
+    al.s[0] = alpha[0]; al.s[1] = alpha[1];
+    be.s[0] = beta[0]; be.s[1] = beta[1];
+    NaiveBlas::gemm<NaiveBlas::DoubleComplex>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasTranspose)transA,
+                                   (NaiveBlas::clblasTranspose)transB, M, N, K, al, (const NaiveBlas::DoubleComplex *)A, lda,
+                                   (const NaiveBlas::DoubleComplex *)B, ldb, be, (NaiveBlas::DoubleComplex *)C, ldc);
+}
+
 void ref_naive_strsm(int order, int side, int uplo, int transA, int diag, size_t M, size_t N, float alpha,
                      const float *A, size_t lda, float *B, size_t ldb) {
     NaiveBlas::trsm<float>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasSide)side, (NaiveBlas::clblasUplo)uplo,

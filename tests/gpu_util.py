@@ -13,7 +13,8 @@ def _dev(x):
 
 
 def gemm(order, tA, tB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, tile=None):
-    fn = clblas_amd.sgemm if C.dtype == np.float32 else clblas_amd.dgemm
+    fn = {np.dtype(np.float32): clblas_amd.sgemm, np.dtype(np.float64): clblas_amd.dgemm,
+          np.dtype(np.complex64): clblas_amd.cgemm, np.dtype(np.complex128): clblas_amd.zgemm}[C.dtype]
     dA, dB, dC = _dev(A), _dev(B), _dev(C)
     if tile is not None:
         os.environ["CLBLAS_AMD_GEMM_TILE"] = str(tile)

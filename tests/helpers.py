@@ -61,10 +61,19 @@ def exact_int_limits(K, alpha, beta, dtype):
     return max(2, min(ab, 1 << 10)), max(2, min(c, 1 << 10))
 
 
-EPS = {np.dtype(np.float32): 2.0 ** -24, np.dtype(np.float64): 2.0 ** -53}
+EPS = {np.dtype(np.float32): 2.0 ** -24, np.dtype(np.float64): 2.0 ** -53,
+       np.dtype(np.complex64): 2.0 ** -24, np.dtype(np.complex128): 2.0 ** -53}
 
 
 def gemm_bound(K, mag, dtype, c=2.0):
     """|C - C_exact| <= c * (K+2) * eps * (|alpha| |A||B| + |beta||C|): the parity bound of the
     task with the unit roundoff; c=2 leaves room for both our result and the reference's."""
     return c * (K + 2) * EPS[np.dtype(dtype)] * mag + np.finfo(dtype).tiny
+
+
+def cgemm_bound(K, mag, dtype, c=2.0):
+    """Complex counterpart, applied to the real and to the imaginary part separately: each is a
+    sum of 2K products (plus 2 + 2 in the epilogue), every term bounded in magnitude through
+    mag = (|al.re|+|al.im|) (|A.re|+|A.im|)(|B.re|+|B.im|) + (|be.re|+|be.im|)(|C.re|+|C.im|)."""
+    real = np.float32 if np.dtype(dtype) == np.dtype(np.complex64) else np.float64
+    return c * (2 * K + 6) * EPS[np.dtype(dtype)] * mag + np.finfo(real).tiny
