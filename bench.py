@@ -1,13 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
 HBM).  Prints ONE JSON line.  `value` is SGEMM TFLOP/s using the reference's own flop
 count 2*M*N*K (src/client/clfunc_xgemm.hpp:95-107); DGEMM (config 4) and DTRSM (config 5,
-M*(M+1)*N flops, src/client/clfunc_xtrsm.hpp:70-92) are reported in `extra`.
+M*(M+1)*N flops, src/client/clfunc_xtrsm.hpp:70-92) are reported in `extra`, and so are CGEMM /
+ZGEMM at the same size (8*M*N*K flops, clfunc_xgemm.hpp:95-107).
 `cpu_baseline` times the CPU oracle (a port of the reference arithmetic, OpenMP over the
 host cores) on a bounded sample of the same workload; it is a reported baseline only.
 """
@@ -65,7 +66,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, or copy (profiling; copy = a plain "
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm or copy (profiling; copy = a plain "
                     "1 GiB device copy used to scale the HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -174,6 +175,28 @@ def main():
         if d_tflops:
             extra["dtrsm"]["pct_of_dgemm_rate"] = round(100 * t_tflops / d_tflops, 2)
         del A, B, B0
+
+    # ---- CGEMM / ZGEMM at the same size (no BASELINE configuration; the neighbours of the path) ----
+    for name, dt, fn, peak in (("cgemm", torch.complex64, clblas_amd.cgemm, PEAK_FP32_MATRIX),
+                               ("zgemm", torch.complex128, clblas_amd.zgemm, PEAK_FP64_MATRIX)):
+        if args.only not in ("", name):
+            continue
+        rdt = torch.float32 if dt == torch.complex64 else torch.float64
+        A, B, C = (torch.view_as_complex(torch.rand(n * n, 2, device="cuda", dtype=rdt, generator=gen) * 2 - 1)
+                   for _ in range(3))
+
+        def cgemm():
+            st = fn(COL, NOTRANS, NOTRANS, n, n, n, 1.0 + 0.5j, A, 0, n, B, 0, n, 0.5 - 0.25j, C, 0, n)
+            if st != 0:
+                raise RuntimeError("clblas%s returned %d" % (name, st))
+
+        csteps = max(3, steps // 2)
+        wall, ev_ms = timed_calls(torch, cgemm, csteps, 2)
+        c_tflops = 8.0 * n * n * n / (ev_ms * 1e-3) / 1e12
+        extra[name] = {"workload": "%s column-major NN %d^3, alpha=1+0.5i, beta=0.5-0.25i, uniform[-1,1)" % (name.upper(), n),
+                       "tflops": round(c_tflops, 3), "launch_ms": round(ev_ms, 4),
+                       "pct_of_matrix_peak": round(100 * c_tflops / peak, 2)}
+        del A, B, C
 
     # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
     cpu = None

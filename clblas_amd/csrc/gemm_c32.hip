@@ -5,13 +5,13 @@ namespace cba {
 
 // Ordered from the largest tile to the smallest.  A complex element carries four times the
 // flops of a real one for twice the bytes, so these tiles match the real 256x128 / 128x128
-// ones in arithmetic intensity at half the panel depth.
-//   0: 128x128x8, wave 64x64 (2 workgroups of 4 waves per CU)
+// ones in arithmetic intensity.
+//   0: 128x128x16, wave 64x64 (2 workgroups of 4 waves per CU)
 //   1:  64x64x8,  wave 32x32, split-K capable
 static const TileEntry<Cx<float>> *c32_tiles(int *n) {
     static const TileEntry<Cx<float>> tab[] = {
-        make_tile_entry<Cx<float>, 128, 128, 8, 64, 64, 2, false>(0.88),
-        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true>(0.78),
+        make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, false>(0.92),
+        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true>(0.80),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

@@ -29,12 +29,11 @@
 //     interleaved between blocks so that one 16-byte LDS read feeds VM blocks and one
 //     16-byte global store writes VM consecutive rows of C.
 //   * Complex types (interleaved re/im, src/library/blas/AutoGemm/KernelOpenCL.py:106-165)
-//     run on the same real MFMAs: the lane groups that a real MFMA spreads over consecutive
-//     k carry the real and the imaginary part of ONE k instead, so with the B-side operand
-//     (br | bi) a block of Re C accumulates from the A-side operand (ar | -ai) and the block
-//     of Im C from (ai | ar): two MFMAs per complex k and block, every MFMA flop useful.
-//     Lanes pick their part out of the (re, im) pair they read from LDS; conjugation is a
-//     sign flip of the imaginary lanes.
+//     run on the same real MFMAs with the same lane <-> k mapping: a lane reads whole
+//     (re, im) elements and every block of C keeps two accumulators,
+//         Re += ar*br,  Re += ai*(-bi),  Im += ar*bi,  Im += ai*br
+//     - four MFMAs per block and step, all of their flops useful, the only extra work one
+//     sign flip per B element.  Conjugation moves that flip to br and/or negates Im at the end.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -288,8 +287,7 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     typedef Mma<typename Elem<T>::Real> M;
     static constexpr bool CPLX = Elem<T>::CPLX;
     static constexpr int VEC = 16 / (int)sizeof(T);
-    // Complex: two lane groups (re, im) per k, so an MFMA covers half as many k.
-    static constexpr int MB = M::MB, KS = CPLX ? M::KS / 2 : M::KS, NACC = M::NACC;
+    static constexpr int MB = M::MB, KS = M::KS, NACC = M::NACC;
     static constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN;
     static constexpr int NT = 64 * WAVES_M * WAVES_N;
     static constexpr int TM = WM / MB, TN = WN / MB;
@@ -340,30 +338,19 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     const int wave = tid >> 6;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);  // same value, known to be wave-uniform
     const int wm = wave % Cfg::WAVES_M, wn = wave / Cfg::WAVES_M;
-    const int j = lane % MB;                            // position along the block edge
-    const int g = CPLX ? lane / (2 * MB) : lane / MB;  // k sub-step supplied by this lane
-    const int part = CPLX ? (lane / MB) & 1 : 0;        // complex: 0 = lane carries re, 1 = im
-    // Sign flips (on the sign bit) that turn the part a lane picked into its MFMA operand:
-    //   B side (br | bi'), A side for Re C (ar | -ai'), for Im C (ai' | ar), x' = conjugated.
-    const uint32_t sgn_b = (CPLX && part && p.conj_b) ? 0x80000000u : 0u;
-    const uint32_t sgn_an = (CPLX && part && !p.conj_a) ? 0x80000000u : 0u;
-    const uint32_t sgn_as = (CPLX && !part && p.conj_a) ? 0x80000000u : 0u;
+    const int j = lane % MB;  // position along the block edge
+    const int g = lane / MB;  // k sub-step supplied by this lane
+    // Complex product with sA, sB = -1 where op(A), op(B) are conjugated, t = sA*sB:
+    //   Re  = sum ar*br + ai*(-t*bi)
+    //   Im' = sum ar*bi + ai*( t*br),   Im = sB * Im'
+    // so exactly one of bi, br is sign-flipped per B element (masks below; the other mask
+    // is zero) and Im' is negated in the epilogue when B is conjugated.
+    const bool t_pos = CPLX && (p.conj_a == p.conj_b);
+    const uint32_t sgn_bi = (CPLX && t_pos) ? 0x80000000u : 0u;
+    const uint32_t sgn_br = (CPLX && !t_pos) ? 0x80000000u : 0u;
     auto flip = [](R x, uint32_t m) -> R {
         if constexpr (sizeof(R) == 4) return __builtin_bit_cast(R, __builtin_bit_cast(uint32_t, x) ^ m);
         else return __builtin_bit_cast(R, __builtin_bit_cast(uint64_t, x) ^ ((uint64_t)m << 32));
-    };
-    // Element read from LDS -> MFMA operand(s) of this lane.
-    auto ops_a = [&](T x, R (&o)[NP]) {
-        if constexpr (CPLX) {
-            o[0] = flip(part ? x.im : x.re, sgn_an);
-            o[1] = flip(part ? x.re : x.im, sgn_as);
-        } else {
-            o[0] = x;
-        }
-    };
-    auto op_b = [&](T x) -> R {
-        if constexpr (CPLX) return flip(part ? x.im : x.re, sgn_b);
-        else return x;
     };
 
     // ---- tile assignment: contiguous chunk of the tile list per XCD, then walk
@@ -468,29 +455,29 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             // i.e. VEC consecutive steps walk VEC consecutive k: a k-major panel row is read
             // per step, a [x][k] panel is read as one 16-byte vector per VEC steps.
             // Fragments are read one step (one VEC-step group for [x][k]) ahead of their use.
-            R a[2][TM][NP], b[2][TN], ak[2][TM][VEC][NP], bk[2][TN][VEC];
+            T a[2][TM], b[2][TN], ak[2][TM][VEC], bk[2][TN][VEC];
             auto kmap = [&](int s) { return (s / VEC) * (VEC * NG) + g * VEC + (s % VEC); };
-            auto read_a = [&](int s, R (&af)[TM][NP]) {  // k-major A panel
+            auto read_a = [&](int s, T (&af)[TM]) {  // k-major A panel
                 const int krow = kmap(s);
 #pragma unroll
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     typename Vec<T, VM>::type av =
                         *reinterpret_cast<const typename Vec<T, VM>::type *>(&As[LA::lds_at(krow, a_frag + ga * MB * VM)]);
 #pragma unroll
-                    for (int e = 0; e < VM; ++e) ops_a(Vec<T, VM>::get(av, e), af[ga * VM + e]);
+                    for (int e = 0; e < VM; ++e) af[ga * VM + e] = Vec<T, VM>::get(av, e);
                 }
             };
-            auto read_b = [&](int s, R (&bf)[TN]) {  // k-major B panel
+            auto read_b = [&](int s, T (&bf)[TN]) {  // k-major B panel
                 const int krow = kmap(s);
 #pragma unroll
                 for (int gb = 0; gb < TN / VN; ++gb) {
                     typename Vec<T, VN>::type bv =
                         *reinterpret_cast<const typename Vec<T, VN>::type *>(&Bs[LB::lds_at(krow, b_frag + gb * MB * VN)]);
 #pragma unroll
-                    for (int e = 0; e < VN; ++e) bf[gb * VN + e] = op_b(Vec<T, VN>::get(bv, e));
+                    for (int e = 0; e < VN; ++e) bf[gb * VN + e] = Vec<T, VN>::get(bv, e);
                 }
             };
-            auto read_ak = [&](int grp, R (&af)[TM][VEC][NP]) {  // [m'][k] A panel, VEC steps at once
+            auto read_ak = [&](int grp, T (&af)[TM][VEC]) {  // [m'][k] A panel, VEC steps at once
 #pragma unroll
                 for (int bm = 0; bm < TM; ++bm) {
                     const int m_img = wm * WM + bm * MB + j;  // image row of block bm, lane j
@@ -498,10 +485,10 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     typename Vec<T, VEC>::type av =
                         *reinterpret_cast<const typename Vec<T, VEC>::type *>(&As[m_img * PITCH_A + place * VEC]);
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) ops_a(Vec<T, VEC>::get(av, e), af[bm][e]);
+                    for (int e = 0; e < VEC; ++e) af[bm][e] = Vec<T, VEC>::get(av, e);
                 }
             };
-            auto read_bk = [&](int grp, R (&bf)[TN][VEC]) {  // [n][k] B panel, VEC steps at once
+            auto read_bk = [&](int grp, T (&bf)[TN][VEC]) {  // [n][k] B panel, VEC steps at once
 #pragma unroll
                 for (int bn = 0; bn < TN; ++bn) {
                     const int n_loc = wn * WN + bn * MB + j;
@@ -509,7 +496,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     typename Vec<T, VEC>::type bv =
                         *reinterpret_cast<const typename Vec<T, VEC>::type *>(&Bs[n_loc * PITCH_B + place * VEC]);
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) bf[bn][e] = op_b(Vec<T, VEC>::get(bv, e));
+                    for (int e = 0; e < VEC; ++e) bf[bn][e] = Vec<T, VEC>::get(bv, e);
                 }
             };
             if constexpr (A_KLAY) read_ak(0, ak[0]); else read_a(0, a[0]);
@@ -529,17 +516,41 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
+                auto a_of = [&](int bm) -> T { return A_KLAY ? ak[(s / VEC) & 1][bm][s % VEC] : a[s & 1][bm]; };
+                auto b_of = [&](int bn) -> T { return B_KLAY ? bk[(s / VEC) & 1][bn][s % VEC] : b[s & 1][bn]; };
+                if constexpr (!CPLX) {
 #pragma unroll
-                for (int bn = 0; bn < TN; ++bn) {
-                    const R bval = B_KLAY ? bk[(s / VEC) & 1][bn][s % VEC] : b[s & 1][bn];
+                    for (int bn = 0; bn < TN; ++bn)
 #pragma unroll
-                    for (int bm = 0; bm < TM; ++bm) {
+                        for (int bm = 0; bm < TM; ++bm) acc[bn][bm][0] = M::run(b_of(bn), a_of(bm), acc[bn][bm][0]);
+                } else {
+                    // Four sweeps over the blocks, so that the two MFMAs into one accumulator
+                    // are TM*TN*2 instructions apart.
+                    R bre[TN], bim[TN], bre_x[TN], bim_x[TN];
 #pragma unroll
-                        for (int pp = 0; pp < NP; ++pp) {
-                            const R aval = A_KLAY ? ak[(s / VEC) & 1][bm][s % VEC][pp] : a[s & 1][bm][pp];
-                            acc[bn][bm][pp] = M::run(bval, aval, acc[bn][bm][pp]);
-                        }
+                    for (int bn = 0; bn < TN; ++bn) {
+                        const T bv = b_of(bn);
+                        bre[bn] = bv.re;
+                        bim[bn] = bv.im;
+                        bim_x[bn] = flip(bv.im, sgn_bi);  // -t*bi up to the zero mask
+                        bre_x[bn] = flip(bv.re, sgn_br);  //  t*br
                     }
+#pragma unroll
+                    for (int bn = 0; bn < TN; ++bn)
+#pragma unroll
+                        for (int bm = 0; bm < TM; ++bm) acc[bn][bm][0] = M::run(bre[bn], a_of(bm).re, acc[bn][bm][0]);
+#pragma unroll
+                    for (int bn = 0; bn < TN; ++bn)
+#pragma unroll
+                        for (int bm = 0; bm < TM; ++bm) acc[bn][bm][1] = M::run(bim[bn], a_of(bm).re, acc[bn][bm][1]);
+#pragma unroll
+                    for (int bn = 0; bn < TN; ++bn)
+#pragma unroll
+                        for (int bm = 0; bm < TM; ++bm) acc[bn][bm][0] = M::run(bim_x[bn], a_of(bm).im, acc[bn][bm][0]);
+#pragma unroll
+                    for (int bn = 0; bn < TN; ++bn)
+#pragma unroll
+                        for (int bm = 0; bm < TM; ++bm) acc[bn][bm][1] = M::run(bre_x[bn], a_of(bm).im, acc[bn][bm][1]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -564,8 +575,9 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         beta = T();
     }
     const bool read_c = !el_is_zero(beta);
+    const bool neg_im = CPLX && p.conj_b;  // Im = sB * Im'
     auto acc_elem = [&](int bn, int bm, int v) -> T {
-        if constexpr (CPLX) return T{acc[bn][bm][0][v], acc[bn][bm][1][v]};
+        if constexpr (CPLX) return T{acc[bn][bm][0][v], neg_im ? -acc[bn][bm][1][v] : acc[bn][bm][1][v]};
         else return acc[bn][bm][0][v];
     };
 
