@@ -73,7 +73,7 @@ EXPORTED_SYMBOLS = (
     "clblasZgemm",
     "clblasStrsm",
     "clblasDtrsm",
-)
+) + tuple("clblas%s%s" % (t, f) for f in ("syrk", "trmm", "symm") for t in "SDCZ")
 
 _lib = None
 
@@ -102,6 +102,17 @@ def _declare(lib):
         fn = getattr(lib, name)
         fn.restype = i
         fn.argtypes = [i, i, i, i, i, sz, sz, real, vp, sz, sz, vp, sz, sz, vp]
+    scalars = {"S": ctypes.c_float, "D": ctypes.c_double, "C": FloatComplex, "Z": DoubleComplex}
+    for t, sc in scalars.items():
+        fn = getattr(lib, "clblas%ssyrk" % t)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, sc, vp, sz, sz, sc, vp, sz, sz, vp]
+        fn = getattr(lib, "clblas%strmm" % t)
+        fn.restype = i
+        fn.argtypes = [i, i, i, i, i, sz, sz, sc, vp, sz, sz, vp, sz, sz, vp]
+        fn = getattr(lib, "clblas%ssymm" % t)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, sc, vp, sz, sz, vp, sz, sz, sc, vp, sz, sz, vp]
     lib.clblasSetup.restype = i
     lib.clblasSetup.argtypes = []
     lib.clblasTeardown.restype = None
@@ -192,3 +203,35 @@ def strsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, l
 def dtrsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):
     return load_library().clblasDtrsm(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha,
                                       _ptr(A), offA, lda, _ptr(B), offB, ldb, _stream(stream))
+
+
+def _scalar(prefix, x):
+    """Python number -> the by-value scalar type of the S/D/C/Z routine family."""
+    if prefix == "C":
+        z = complex(x)
+        return FloatComplex(z.real, z.imag)
+    if prefix == "Z":
+        z = complex(x)
+        return DoubleComplex(z.real, z.imag)
+    return float(x)
+
+
+def syrk(prefix, order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, stream=None):
+    """clblas{prefix}syrk, prefix in "SDCZ" (src/clBLAS.h:8278-8503)."""
+    fn = getattr(load_library(), "clblas%ssyrk" % prefix)
+    return fn(int(order), int(uplo), int(transA), N, K, _scalar(prefix, alpha), _ptr(A), offA, lda,
+              _scalar(prefix, beta), _ptr(C), offC, ldc, _stream(stream))
+
+
+def trmm(prefix, order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):
+    """clblas{prefix}trmm, prefix in "SDCZ" (src/clBLAS.h:7696-7928)."""
+    fn = getattr(load_library(), "clblas%strmm" % prefix)
+    return fn(int(order), int(side), int(uplo), int(transA), int(diag), M, N, _scalar(prefix, alpha), _ptr(A), offA,
+              lda, _ptr(B), offB, ldb, _stream(stream))
+
+
+def symm(prefix, order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    """clblas{prefix}symm, prefix in "SDCZ" (src/clBLAS.h:8897-9145)."""
+    fn = getattr(load_library(), "clblas%ssymm" % prefix)
+    return fn(int(order), int(side), int(uplo), M, N, _scalar(prefix, alpha), _ptr(A), offA, lda, _ptr(B), offB, ldb,
+              _scalar(prefix, beta), _ptr(C), offC, ldc, _stream(stream))

@@ -4,6 +4,7 @@
 //   src/library/blas/xgemm.cc:667-905  (clblasSgemm / clblasDgemm / clblasCgemm / clblasZgemm),
 //   src/library/blas/xgemm.cc:341-383  (clblasGemm<T>: ConjTrans and row-major folding),
 //   src/library/blas/xtrsm.cc:1600-1785 (clblasStrsm / clblasDtrsm),
+//   src/library/blas/xsyrk.c:27-233, xtrmm.c:27-245, xsymm.c:33-429 (SYRK / TRMM / SYMM),
 //   src/library/blas/functor/functor_xtrsm.cc:57-75 (doTrsm validation),
 //   src/library/blas/generic/common.c:585-688 (checkMatrixSizes),
 //   src/library/blas/init.c:33-263 (GetVersion / Setup / Teardown).
@@ -38,17 +39,17 @@ struct WsSlot {
     size_t bytes = 0;
 };
 std::mutex g_ws_mutex;
-std::map<std::pair<int, hipStream_t>, WsSlot> g_ws;  // (device, stream) -> current buffer
+std::map<std::pair<std::pair<int, int>, hipStream_t>, WsSlot> g_ws;  // ((device, kind), stream) -> current buffer
 std::vector<std::pair<int, void *>> g_ws_retired;    // outgrown buffers, freed at teardown
 std::mutex g_lds_mutex;
 std::map<std::pair<int, const void *>, size_t> g_lds_limit;
 }  // namespace
 
-void *workspace_get(hipStream_t stream, size_t bytes) {
+void *workspace_get(hipStream_t stream, size_t bytes, int kind) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    WsSlot &slot = g_ws[std::make_pair(dev, stream)];
+    WsSlot &slot = g_ws[std::make_pair(std::make_pair(dev, kind), stream)];
     if (slot.bytes >= bytes && slot.ptr) return slot.ptr;
     size_t want = bytes < (size_t)(1 << 20) ? (size_t)(1 << 20) : bytes;
     void *p = nullptr;
@@ -68,7 +69,7 @@ void workspace_release_all() {
     (void)hipGetDevice(&cur);
     for (auto &kv : g_ws) {
         if (kv.second.ptr) {
-            (void)hipSetDevice(kv.first.first);
+            (void)hipSetDevice(kv.first.first.first);
             (void)hipFree(kv.second.ptr);
         }
     }
@@ -125,13 +126,14 @@ clblasStatus map_hip_error(hipError_t e) {
     (void)hipGetLastError();
     if (e == hipErrorOutOfMemory) return clblasOutOfResources;
     if (e == hipErrorInvalidValue) return clblasInvalidValue;
+    if (e == hipErrorNotSupported) return clblasNotImplemented;
     return clblasOutOfResources;
 }
 
 const size_t kMaxDim = 0x7fffffff;  // kernels index tiles with 32-bit ints (reference: cl_uint, xgemm.cc:362-372)
 
-template <typename T, typename Fn>
-clblasStatus gemm_front(Fn launch, clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M,
+template <typename T>
+clblasStatus gemm_front(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M,
                         size_t N, size_t K, T alpha, const T *A, size_t offA, size_t lda, const T *B, size_t offB,
                         size_t ldb, T beta, T *C, size_t offC, size_t ldc, hipStream_t stream) {
     // Order of checks follows xgemm.cc:685-706: objects A, B, C; then (K != 0) sizes of A,
@@ -161,17 +163,93 @@ clblasStatus gemm_front(Fn launch, clblasOrder order, clblasTranspose transA, cl
         std::swap(lda, ldb);
         std::swap(pa, pb);
     }
-    return map_hip_error(launch(tA, tB, cA, cB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb, (int64_t)ldb,
-                                beta, C + offC, (int64_t)ldc, stream));
+    return map_hip_error(cba::launch_gemm<T>(tA, tB, cA, cB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb,
+                                             (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
 }
 
-hipError_t sgemm_real(bool tA, bool tB, bool, bool, int M, int N, int K, float alpha, const float *A, int64_t lda,
-                      const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream) {
-    return cba::sgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+template <typename T> struct IsComplex { static const bool value = false; };
+template <typename R> struct IsComplex<cba::Cx<R>> { static const bool value = true; };
+
+// SYRK front end.  Checks as doSyrk (src/library/blas/xsyrk.c:56-72): objects A, C; ConjTrans
+// is invalid for complex types; A is N x K, C is N x N.  Row major: the same memory read
+// column-major holds A^T and C^T, so flip the transpose flag and the triangle.
+template <typename T>
+clblasStatus syrk_front(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, T alpha,
+                        const T *A, size_t offA, size_t lda, T beta, T *C, size_t offC, size_t ldc,
+                        hipStream_t stream) {
+    if (!A) return clblasInvalidMatA;
+    if (!C) return clblasInvalidMatC;
+    if (!valid_order(order) || !valid_trans(transA) || (uplo != clblasUpper && uplo != clblasLower))
+        return clblasInvalidValue;
+    if (IsComplex<T>::value && transA == clblasConjTrans) return clblasInvalidValue;
+    clblasStatus st;
+    if ((st = check_matrix_sizes(order, transA, N, K, lda, MAT_A)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if (N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
+    bool lower = uplo == clblasLower, trans = transA != clblasNoTrans;
+    if (order == clblasRowMajor) {
+        lower = !lower;
+        trans = !trans;
+    }
+    return map_hip_error(cba::syrk_colmajor<T>(lower, trans, (int)N, (int)K, alpha, A + offA, (int64_t)lda, beta,
+                                               C + offC, (int64_t)ldc, stream));
 }
-hipError_t dgemm_real(bool tA, bool tB, bool, bool, int M, int N, int K, double alpha, const double *A, int64_t lda,
-                      const double *B, int64_t ldb, double beta, double *C, int64_t ldc, hipStream_t stream) {
-    return cba::dgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+
+// TRMM front end.  Checks as doTrmm (src/library/blas/xtrmm.c:47-64), the same as TRSM's;
+// row-major folding as for TRSM.
+template <typename T>
+clblasStatus trmm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                        clblasDiag diag, size_t M, size_t N, T alpha, const T *A, size_t offA, size_t lda, T *B,
+                        size_t offB, size_t ldb, hipStream_t stream) {
+    if (!A) return clblasInvalidMatA;
+    if (!B) return clblasInvalidMatB;
+    if (!valid_order(order) || !valid_trans(transA) || (side != clblasLeft && side != clblasRight) ||
+        (uplo != clblasUpper && uplo != clblasLower) || (diag != clblasUnit && diag != clblasNonUnit))
+        return clblasInvalidValue;
+    const size_t msize = side == clblasLeft ? M : N;
+    clblasStatus st;
+    if ((st = check_matrix_sizes(order, transA, msize, msize, lda, MAT_A)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B)) != clblasSuccess) return st;
+    if (M > kMaxDim || N > kMaxDim) return clblasNotImplemented;
+    bool right = side == clblasRight, lower = uplo == clblasLower;
+    if (order == clblasRowMajor) {
+        std::swap(M, N);
+        right = !right;
+        lower = !lower;
+    }
+    return map_hip_error(cba::trmm_colmajor<T>(right, lower, transA != clblasNoTrans,
+                                               IsComplex<T>::value && transA == clblasConjTrans, diag == clblasUnit,
+                                               (int)M, (int)N, alpha, A + offA, (int64_t)lda, B + offB, (int64_t)ldb,
+                                               stream));
+}
+
+// SYMM front end.  Checks as doSymm (src/library/blas/xsymm.c:50-71): objects A, B, C; A is
+// M x M (left) or N x N (right); B and C are M x N.  Row major swaps M and N and flips side
+// and triangle (xsymm.c:104-124).
+template <typename T>
+clblasStatus symm_front(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, T alpha, const T *A,
+                        size_t offA, size_t lda, const T *B, size_t offB, size_t ldb, T beta, T *C, size_t offC,
+                        size_t ldc, hipStream_t stream) {
+    if (!A) return clblasInvalidMatA;
+    if (!B) return clblasInvalidMatB;
+    if (!C) return clblasInvalidMatC;
+    if (!valid_order(order) || (side != clblasLeft && side != clblasRight) ||
+        (uplo != clblasUpper && uplo != clblasLower))
+        return clblasInvalidValue;
+    const size_t msize = side == clblasLeft ? M : N;
+    clblasStatus st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, msize, msize, lda, MAT_A)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if (M > kMaxDim || N > kMaxDim) return clblasNotImplemented;
+    bool right = side == clblasRight, lower = uplo == clblasLower;
+    if (order == clblasRowMajor) {
+        std::swap(M, N);
+        right = !right;
+        lower = !lower;
+    }
+    return map_hip_error(cba::symm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda, B + offB,
+                                               (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
 }
 
 static_assert(sizeof(FloatComplex) == sizeof(cba::Cx<float>) && sizeof(DoubleComplex) == sizeof(cba::Cx<double>),
@@ -244,7 +322,7 @@ clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B,
                          size_t offB, size_t ldb, float beta, float *C, size_t offC, size_t ldc,
                          hipStream_t stream) {
-    return gemm_front<float>(sgemm_real, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb,
+    return gemm_front<float>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb,
                              beta, C, offC, ldc, stream);
 }
 
@@ -252,7 +330,7 @@ clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          size_t K, double alpha, const double *A, size_t offA, size_t lda, const double *B,
                          size_t offB, size_t ldb, double beta, double *C, size_t offC, size_t ldc,
                          hipStream_t stream) {
-    return gemm_front<double>(dgemm_real, order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB,
+    return gemm_front<double>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB,
                               ldb, beta, C, offC, ldc, stream);
 }
 
@@ -261,7 +339,7 @@ clblasStatus clblasCgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta, FloatComplex *C,
                          size_t offC, size_t ldc, hipStream_t stream) {
     typedef cba::Cx<float> E;
-    return gemm_front<E>(cba::cgemm_colmajor, order, transA, transB, M, N, K, cx(alpha),
+    return gemm_front<E>(order, transA, transB, M, N, K, cx(alpha),
                          reinterpret_cast<const E *>(A), offA, lda, reinterpret_cast<const E *>(B), offB, ldb,
                          cx(beta), reinterpret_cast<E *>(C), offC, ldc, stream);
 }
@@ -271,7 +349,7 @@ clblasStatus clblasZgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta, DoubleComplex *C,
                          size_t offC, size_t ldc, hipStream_t stream) {
     typedef cba::Cx<double> E;
-    return gemm_front<E>(cba::zgemm_colmajor, order, transA, transB, M, N, K, cx(alpha),
+    return gemm_front<E>(order, transA, transB, M, N, K, cx(alpha),
                          reinterpret_cast<const E *>(A), offA, lda, reinterpret_cast<const E *>(B), offB, ldb,
                          cx(beta), reinterpret_cast<E *>(C), offC, ldc, stream);
 }
@@ -288,6 +366,78 @@ clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, cl
                          size_t lda, double *B, size_t offB, size_t ldb, hipStream_t stream) {
     return trsm_front<double>(cba::dtrsm_colmajor, order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
                               offB, ldb, stream);
+}
+
+clblasStatus clblasSsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         float alpha, const float *A, size_t offA, size_t lda, float beta, float *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return syrk_front<float>(order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasStrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, float alpha, const float *A, size_t offA, size_t lda, float *B,
+                         size_t offB, size_t ldb, hipStream_t stream) {
+    return trmm_front<float>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream);
+}
+
+clblasStatus clblasSsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, float alpha,
+                         const float *A, size_t offA, size_t lda, const float *B, size_t offB, size_t ldb, float beta, float *C,
+                         size_t offC, size_t ldc, hipStream_t stream) {
+    return symm_front<float>(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasDsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         double alpha, const double *A, size_t offA, size_t lda, double beta, double *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return syrk_front<double>(order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasDtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, double alpha, const double *A, size_t offA, size_t lda, double *B,
+                         size_t offB, size_t ldb, hipStream_t stream) {
+    return trmm_front<double>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream);
+}
+
+clblasStatus clblasDsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, double alpha,
+                         const double *A, size_t offA, size_t lda, const double *B, size_t offB, size_t ldb, double beta, double *C,
+                         size_t offC, size_t ldc, hipStream_t stream) {
+    return symm_front<double>(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasCsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, FloatComplex beta, FloatComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return syrk_front<cba::Cx<float>>(order, uplo, transA, N, K, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, cx(beta), reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasCtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, FloatComplex *B,
+                         size_t offB, size_t ldb, hipStream_t stream) {
+    return trmm_front<cba::Cx<float>>(order, side, uplo, transA, diag, M, N, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<cba::Cx<float> *>(B), offB, ldb, stream);
+}
+
+clblasStatus clblasCsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, FloatComplex alpha,
+                         const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta, FloatComplex *C,
+                         size_t offC, size_t ldc, hipStream_t stream) {
+    return symm_front<cba::Cx<float>>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasZsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, DoubleComplex beta, DoubleComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return syrk_front<cba::Cx<double>>(order, uplo, transA, N, K, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, cx(beta), reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasZtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, DoubleComplex *B,
+                         size_t offB, size_t ldb, hipStream_t stream) {
+    return trmm_front<cba::Cx<double>>(order, side, uplo, transA, diag, M, N, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<cba::Cx<double> *>(B), offB, ldb, stream);
+}
+
+clblasStatus clblasZsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, DoubleComplex alpha,
+                         const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta, DoubleComplex *C,
+                         size_t offC, size_t ldc, hipStream_t stream) {
+    return symm_front<cba::Cx<double>>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
 }
 
 }  // extern "C"

@@ -10,8 +10,8 @@ namespace cba {
 //   1:  64x64x8,  wave 32x32, split-K capable
 static const TileEntry<Cx<float>> *c32_tiles(int *n) {
     static const TileEntry<Cx<float>> tab[] = {
-        make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, false>(0.92),
-        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true>(0.80),
+        make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, false, true>(0.92),
+        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true, true>(0.80),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;
@@ -19,11 +19,11 @@ static const TileEntry<Cx<float>> *c32_tiles(int *n) {
 
 hipError_t cgemm_colmajor(bool transA, bool transB, bool conjA, bool conjB, int M, int N, int K, Cx<float> alpha,
                           const Cx<float> *A, int64_t lda, const Cx<float> *B, int64_t ldb, Cx<float> beta,
-                          Cx<float> *C, int64_t ldc, hipStream_t stream) {
+                          Cx<float> *C, int64_t ldc, hipStream_t stream, const GemmTri *tri) {
     int n;
     const TileEntry<Cx<float>> *tab = c32_tiles(&n);
     return run_gemm_colmajor<Cx<float>>(tab, n, transA, transB, conjA, conjB, M, N, K, alpha, A, lda, B, ldb, beta,
-                                        C, ldc, stream);
+                                        C, ldc, stream, tri);
 }
 
 }  // namespace cba

@@ -8,8 +8,8 @@ namespace cba {
 //   1:  64x64x8, wave 32x32, split-K capable
 static const TileEntry<Cx<double>> *c64_tiles(int *n) {
     static const TileEntry<Cx<double>> tab[] = {
-        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, false>(0.92),
-        make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true>(0.84),
+        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, false, true>(0.92),
+        make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true>(0.84),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;
@@ -17,11 +17,11 @@ static const TileEntry<Cx<double>> *c64_tiles(int *n) {
 
 hipError_t zgemm_colmajor(bool transA, bool transB, bool conjA, bool conjB, int M, int N, int K, Cx<double> alpha,
                           const Cx<double> *A, int64_t lda, const Cx<double> *B, int64_t ldb, Cx<double> beta,
-                          Cx<double> *C, int64_t ldc, hipStream_t stream) {
+                          Cx<double> *C, int64_t ldc, hipStream_t stream, const GemmTri *tri) {
     int n;
     const TileEntry<Cx<double>> *tab = c64_tiles(&n);
     return run_gemm_colmajor<Cx<double>>(tab, n, transA, transB, conjA, conjB, M, N, K, alpha, A, lda, B, ldb, beta,
-                                         C, ldc, stream);
+                                         C, ldc, stream, tri);
 }
 
 }  // namespace cba

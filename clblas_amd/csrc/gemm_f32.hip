@@ -9,19 +9,19 @@ namespace cba {
 //   2:  64x64x16,  wave 32x32, split-K capable (small / deep-K problems)
 static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
-        make_tile_entry<float, 256, 128, 16, 128, 64, 2, false>(0.885),
-        make_tile_entry<float, 128, 128, 16, 64, 64, 2, false>(0.86),
-        make_tile_entry<float, 64, 64, 16, 32, 32, 2, true>(0.78),
+        make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.885),
+        make_tile_entry<float, 128, 128, 16, 64, 64, 2, false, true>(0.86),
+        make_tile_entry<float, 64, 64, 16, 32, 32, 2, true, true>(0.78),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;
 }
 
 hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float alpha, const float *A, int64_t lda,
-                          const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream) {
+                          const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream, const GemmTri *tri) {
     int n;
     const TileEntry<float> *tab = f32_tiles(&n);
-    return run_gemm_colmajor<float>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+    return run_gemm_colmajor<float>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, tri);
 }
 
 }  // namespace cba

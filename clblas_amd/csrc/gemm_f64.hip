@@ -8,8 +8,8 @@ namespace cba {
 //   1:  64x64x16,  wave 32x32, split-K capable
 static const TileEntry<double> *f64_tiles(int *n) {
     static const TileEntry<double> tab[] = {
-        make_tile_entry<double, 128, 128, 16, 64, 64, 2, false>(0.86),
-        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true>(0.82),
+        make_tile_entry<double, 128, 128, 16, 64, 64, 2, false, true>(0.86),
+        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true>(0.82),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;
@@ -17,10 +17,10 @@ static const TileEntry<double> *f64_tiles(int *n) {
 
 hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double alpha, const double *A,
                           int64_t lda, const double *B, int64_t ldb, double beta, double *C, int64_t ldc,
-                          hipStream_t stream) {
+                          hipStream_t stream, const GemmTri *tri) {
     int n;
     const TileEntry<double> *tab = f64_tiles(&n);
-    return run_gemm_colmajor<double>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+    return run_gemm_colmajor<double>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, tri);
 }
 
 }  // namespace cba

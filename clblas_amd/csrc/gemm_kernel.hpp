@@ -183,6 +183,15 @@ template <typename T> struct GemmParams {
     int k_per_split;  // multiple of BK; >= K when the K loop is not split
     T *ws;            // split-K partial sums: ws[split * ws_slice + n * ws_ld + m]
     int64_t ws_ld, ws_slice;
+    // Triangular structure (kernels built with TRI only; all zero otherwise).
+    //   tri_c: store only the lower (1: m >= n) or upper (2: m <= n) triangle of C; tiles
+    //          wholly outside it are not enumerated at all (grid = number of active tiles).
+    //   tri_a / tri_b: op(A)(m,k) / op(B)(k,n) is triangular: elements with k > x (1) or
+    //          k < x (2), x = m resp. n, count as zero whatever memory holds; unit_* = 1: the
+    //          diagonal k == x counts as one, 2: as zero.  Panels outside the triangle are
+    //          skipped.
+    //   rev_m / rev_n: walk the tile rows / columns from the far end (longest tiles first).
+    int tri_c, tri_a, tri_b, unit_a, unit_b, rev_m, rev_n;
 };
 
 static __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, int64_t bytes_left) {
@@ -267,6 +276,35 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
                                                      (int)voff[i], 0, 0, 0);
     }
 
+    // Triangular operand: in the 16 bytes each of this thread's loads delivered, zeroes the
+    // elements outside the triangle (mode 1 keeps k <= x, mode 2 keeps k >= x; x0, k0: global
+    // coordinates of the panel's first element); unit == 1 sets the diagonal to one, 2 to zero.
+    // Call after waiting for the thread's own loads.
+    __device__ __forceinline__ void mask_tri(T *lds, int tid, int x0, int k0, int mode, int unit) const {
+        const int lane = tid & 63, wave = tid >> 6;
+        auto fix = [&](T &v, int xg, int kg) {
+            const bool keep = mode == 1 ? kg <= xg : kg >= xg;
+            if (!keep || (unit == 2 && kg == xg)) v = T();
+            else if (unit == 1 && kg == xg) v = el_one<T>();
+        };
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            if (MODE == LM_DMA_X) {
+                const int e0 = (wave + i * NW) * CHUNK + lane * VEC;
+                const int k = e0 / BX, x = e0 % BX;
+                T *q = lds + (wave + i * NW) * CHUNK_PITCH + lane * VEC;
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) fix(q[e], x0 + x + e, k0 + k);
+            } else {
+                const int ximg = (wave + i * NW) * (64 / S) + lane / S;
+                const int place = lane % S, slot = place ^ swz(ximg);
+                const int xg = x0 + perm(ximg);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) fix(lds[ximg * BK + place * VEC + e], xg, k0 + slot * VEC + e);
+            }
+        }
+    }
+
     // LM_DMA_K: clears the elements past K of a partial panel, each thread in the 16 bytes
     // its own loads delivered (call after waiting for those loads).
     __device__ __forceinline__ void clear_k_tail(T *lds, int tid, int k_valid) const {
@@ -315,9 +353,11 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static constexpr size_t SMEM = (size_t)NSTAGE * STAGE * sizeof(T);
 };
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, bool SPLITK, int MINW>
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, bool SPLITK, int MINW,
+          bool TRI = false>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64, MINW)
 gemm_mfma_kernel(const GemmParams<T> p) {
+    static_assert(!(SPLITK && TRI), "triangular variants do not split K");
     typedef GemmCfg<T, BM, BN, BK, WM, WN, A_KC, B_KC> Cfg;
     typedef typename Elem<T>::Real R;
     typedef Mma<R> M;
@@ -358,14 +398,31 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     //      XCD share A and B panels in that XCD's L2. ----
     int tile;
     {
-        const int nwg = p.tiles_m * p.tiles_n;
+        const int nwg = gridDim.x;
         const int id = blockIdx.x;
         const int xcd = id & 7, q = id >> 3;
         const int per = nwg >> 3, rem = nwg & 7;
         tile = p.xcd_remap ? xcd * per + (xcd < rem ? xcd : rem) + q : id;
     }
     int tm, tn;
-    {
+    if (TRI && p.tri_c) {
+        // Only tiles that touch the stored triangle exist: row tm holds the columns
+        // [0, last] (lower) or [first, tiles_n) (upper); walk the rows until `tile` fits.
+        tm = 0;
+        tn = 0;
+        for (int r = 0; r < p.tiles_m; ++r) {
+            int first = 0, count;
+            if (p.tri_c == 1) {
+                const int last = (r * BM + BM - 1) / BN;
+                count = last + 1 < p.tiles_n ? last + 1 : p.tiles_n;
+            } else {
+                first = (r * BM) / BN;
+                count = first < p.tiles_n ? p.tiles_n - first : 0;
+            }
+            if (tile < count) { tm = r; tn = first + tile; break; }
+            tile -= count;
+        }
+    } else {
         const int per_group = p.group_m * p.tiles_n;
         const int grp = tile / per_group;
         const int first_m = grp * p.group_m;
@@ -373,6 +430,8 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         const int r = tile - grp * per_group;
         tm = first_m + r % gm;
         tn = r / gm;
+        if (TRI && p.rev_m) tm = p.tiles_m - 1 - tm;
+        if (TRI && p.rev_n) tn = p.tiles_n - 1 - tn;
     }
     const int m0 = tm * BM, n0 = tn * BN;
 
@@ -382,7 +441,14 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         k_begin = blockIdx.y * p.k_per_split;
         k_end = k_begin + p.k_per_split < p.K ? k_begin + p.k_per_split : p.K;
     }
-    const int n_panels = (k_end - k_begin + BK - 1) / BK;
+    if (TRI) {
+        // Panels that lie wholly in the zero part of a triangular operand are skipped.
+        if (p.tri_a == 1 && m0 + BM < k_end) k_end = m0 + BM;
+        if (p.tri_b == 1 && n0 + BN < k_end) k_end = n0 + BN;
+        if (p.tri_a == 2 && (m0 / BK) * BK > k_begin) k_begin = (m0 / BK) * BK;
+        if (p.tri_b == 2 && (n0 / BK) * BK > k_begin) k_begin = (n0 / BK) * BK;
+    }
+    const int n_panels = k_end > k_begin ? (k_end - k_begin + BK - 1) / BK : 0;
 
     typename Cfg::LoaderA la;
     typename Cfg::LoaderB lb;
@@ -432,6 +498,14 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             if (k_valid < BK) {
                 la.clear_k_tail(dst, tid, k_valid);
                 lb.clear_k_tail(dst + A_ELEMS, tid, k_valid);
+            }
+            if (TRI) {
+                // Only the panels that meet the diagonal (or the zero side of it) need the fix-up.
+                const int k0 = k_begin + kp * BK;
+                if ((p.tri_a == 1 && k0 + BK > m0) || (p.tri_a == 2 && k0 < m0 + BM))
+                    la.mask_tri(dst, tid, m0, k0, p.tri_a, p.unit_a);
+                if ((p.tri_b == 1 && k0 + BK > n0) || (p.tri_b == 2 && k0 < n0 + BN))
+                    lb.mask_tri(dst + A_ELEMS, tid, n0, k0, p.tri_b, p.unit_b);
             }
             __syncthreads();
         };
@@ -613,7 +687,12 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 #pragma unroll
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     const int m = m0 + wm * WM + ga * (MB * VM) + j * VM;
-                    if (m + VM <= p.M) {
+                    bool whole = true;  // all VM rows of this vector are stored
+                    if (TRI && p.tri_c) {
+                        if (p.tri_c == 1 ? m + VM - 1 < n : m > n) continue;  // none of them is
+                        whole = p.tri_c == 1 ? m >= n : m + VM - 1 <= n;
+                    }
+                    if (m + VM <= p.M && whole) {
                         UV ov;
 #pragma unroll
                         for (int e = 0; e < VM; ++e) {
@@ -625,7 +704,8 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     } else {
 #pragma unroll
                         for (int e = 0; e < VM; ++e) {
-                            if (m + e < p.M) {
+                            const bool kept = !(TRI && p.tri_c) || (p.tri_c == 1 ? m + e >= n : m + e <= n);
+                            if (m + e < p.M && kept) {
                                 T r = el_scale(alpha, acc_elem(bn, ga * VM + e, v));
                                 if (read_c) r = el_axpy(beta, col[m + e], r);
                                 col[m + e] = r;

@@ -20,9 +20,11 @@ template <typename T> struct TileEntry {
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
     void (*plain[4])(const GemmParams<T>);
     void (*splitk[4])(const GemmParams<T>);
+    void (*tri[4])(const GemmParams<T>);  // variants that honour the triangular fields (or null)
 };
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK>
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false>
 TileEntry<T> make_tile_entry(double eff) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
@@ -47,6 +49,14 @@ TileEntry<T> make_tile_entry(double eff) {
     } else {
         for (int i = 0; i < 4; ++i) e.splitk[i] = nullptr;
     }
+    if constexpr (WITH_TRI) {
+        e.tri[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, false, MINW, true>;
+        e.tri[1] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, false, false, MINW, true>;
+        e.tri[2] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, true, false, MINW, true>;
+        e.tri[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, false, MINW, true>;
+    } else {
+        for (int i = 0; i < 4; ++i) e.tri[i] = nullptr;
+    }
     return e;
 }
 
@@ -61,22 +71,24 @@ static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b;
 // paid for automatically because whole tiles are counted).  The smallest tile adds a K
 // split when even it cannot give every CU a workgroup.
 template <typename T>
-static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, int *tile_out,
-                        int *splits_out) {
+static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, bool need_tri,
+                        int *tile_out, int *splits_out) {
     const int64_t kCUs = 256;
     int pick = ntab - 1;  // table is ordered large -> small
-    if (force >= 0 && force < ntab) {
+    if (force >= 0 && force < ntab && (!need_tri || tab[force].tri[0])) {
         pick = force;
     } else {
         double best = 0;
+        bool have = false;
         for (int i = 0; i < ntab; ++i) {
+            if (need_tri && !tab[i].tri[0]) continue;
             const int64_t t = ceil_div64(M, tab[i].bm) * ceil_div64(N, tab[i].bn);
             const double cost = (double)ceil_div64(t, kCUs) * tab[i].bm * tab[i].bn / tab[i].eff;
-            if (i == 0 || cost < best) { best = cost; pick = i; }
+            if (!have || cost < best) { best = cost; pick = i; have = true; }
         }
     }
     int splits = 1;
-    if (tab[pick].has_splitk) {
+    if (tab[pick].has_splitk && !need_tri) {
         int64_t t = ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn);
         if (t < kCUs && K >= 8 * tab[pick].bk) {
             int64_t want = (2 * kCUs) / t;              // aim for ~2 workgroups per CU
@@ -93,7 +105,9 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
 template <typename T>
 static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, bool tB, bool cA, bool cB, int M,
                                     int N, int K, T alpha, const T *A, int64_t lda, const T *B, int64_t ldb,
-                                    T beta, T *C, int64_t ldc, hipStream_t stream) {
+                                    T beta, T *C, int64_t ldc, hipStream_t stream, const GemmTri *tri = nullptr) {
+    const bool need_tri = tri && tri->any();
+    if (need_tri && K == 0) return hipErrorInvalidValue;  // callers reject empty products earlier
     if (K == 0) {
         int mb = (int)ceil_div64(M, 256);
         hipLaunchKernelGGL(scale_c_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
@@ -104,6 +118,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     const int64_t max_edge = 256;
     const int64_t ld_limit = (int64_t)0x7fffffff / (max_edge * (int64_t)sizeof(T)) - 8;
     if (lda > ld_limit || ldb > ld_limit) {
+        if (need_tri) return hipErrorNotSupported;
         int mb = (int)ceil_div64(M, 256);
         hipLaunchKernelGGL(gemm_wide_ld_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream,
                            tA ? 1 : 0, tB ? 1 : 0, cA ? 1 : 0, cB ? 1 : 0, M, N, K, mb, alpha, A, lda, B, ldb, beta, C,
@@ -112,7 +127,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     }
 
     int tile, splits;
-    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), &tile, &splits);
+    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, &tile, &splits);
     const TileEntry<T> &e = tab[tile];
 
     GemmParams<T> p;
@@ -132,11 +147,38 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     p.xcd_remap = debug_env_int("CLBLAS_AMD_GEMM_XCD", 1);
     p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
     p.k_per_split = K;
+    p.tri_c = p.tri_a = p.tri_b = p.unit_a = p.unit_b = p.rev_m = p.rev_n = 0;
     const int idx = (tA ? 2 : 0) | (tB ? 1 : 0);
-    const int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n;
+    int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return hipErrorInvalidValue;
 
     auto fn = e.plain[idx];
+    if (need_tri) {
+        if (!e.tri[idx]) return hipErrorNotSupported;
+        fn = e.tri[idx];
+        p.tri_c = tri->tri_c; p.tri_a = tri->tri_a; p.tri_b = tri->tri_b;
+        p.unit_a = tri->unit_a; p.unit_b = tri->unit_b;
+        if (p.tri_c) {
+            // same enumeration as the kernel's: tiles that touch the stored triangle
+            ntiles = 0;
+            for (int r = 0; r < p.tiles_m; ++r) {
+                if (p.tri_c == 1) {
+                    const int64_t last = ((int64_t)r * e.bm + e.bm - 1) / e.bn;
+                    ntiles += last + 1 < p.tiles_n ? last + 1 : p.tiles_n;
+                } else {
+                    const int64_t first = ((int64_t)r * e.bm) / e.bn;
+                    ntiles += first < p.tiles_n ? p.tiles_n - first : 0;
+                }
+            }
+        }
+        if (p.tri_a || p.tri_b) {
+            // Tiles differ in depth: start the deepest first and deal consecutive tiles to
+            // different XCDs so that every XCD gets the same mix.
+            p.rev_m = p.tri_a == 1;
+            p.rev_n = p.tri_b == 1;
+            p.xcd_remap = 0;
+        }
+    }
     if (splits > 1) {
         int64_t kps = ceil_div64(ceil_div64(K, splits), e.bk) * e.bk;
         splits = (int)ceil_div64(K, kps);

@@ -1,0 +1,124 @@
+// SYRK, TRMM and SYMM as GEMM-shaped calls on the MFMA GEMM core.
+//
+// The reference runs these through its generated solver kernels (src/library/blas/xsyrk.c,
+// xtrmm.c, xsymm.c; xsymm.c:150-330 already composes SYMM from GEMM passes).  Here each is
+// one or two launches of the GEMM kernel's triangular variant:
+//   SYRK  one launch; only the tiles that touch the stored triangle of C exist, tiles on
+//         the diagonal store element-wise.
+//   TRMM  B is copied to a workspace W, then B <- alpha op(A) W (or alpha W op(A)) with the
+//         triangular operand masked in LDS and the panels in its zero half skipped.
+//   SYMM  A = T + S^T with T the stored triangle and S its strict part:
+//         C <- alpha T B + beta C, then C <- alpha S^T B + C (two half-depth launches, no
+//         workspace).
+#include "gemm_kernel.hpp"
+#include "internal.h"
+
+namespace cba {
+
+template <> hipError_t launch_gemm<float>(bool tA, bool tB, bool, bool, int M, int N, int K, float alpha,
+                                          const float *A, int64_t lda, const float *B, int64_t ldb, float beta,
+                                          float *C, int64_t ldc, hipStream_t s, const GemmTri *tri) {
+    return sgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s, tri);
+}
+template <> hipError_t launch_gemm<double>(bool tA, bool tB, bool, bool, int M, int N, int K, double alpha,
+                                           const double *A, int64_t lda, const double *B, int64_t ldb, double beta,
+                                           double *C, int64_t ldc, hipStream_t s, const GemmTri *tri) {
+    return dgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s, tri);
+}
+template <> hipError_t launch_gemm<Cx<float>>(bool tA, bool tB, bool cA, bool cB, int M, int N, int K,
+                                              Cx<float> alpha, const Cx<float> *A, int64_t lda, const Cx<float> *B,
+                                              int64_t ldb, Cx<float> beta, Cx<float> *C, int64_t ldc, hipStream_t s,
+                                              const GemmTri *tri) {
+    return cgemm_colmajor(tA, tB, cA, cB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s, tri);
+}
+template <> hipError_t launch_gemm<Cx<double>>(bool tA, bool tB, bool cA, bool cB, int M, int N, int K,
+                                               Cx<double> alpha, const Cx<double> *A, int64_t lda,
+                                               const Cx<double> *B, int64_t ldb, Cx<double> beta, Cx<double> *C,
+                                               int64_t ldc, hipStream_t s, const GemmTri *tri) {
+    return zgemm_colmajor(tA, tB, cA, cB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s, tri);
+}
+
+// dst(m, n) = src(m, n) for an M x N column-major matrix; block b covers rows
+// [256 * (b % m_blocks), +256) of column b / m_blocks.
+template <typename T>
+__global__ void __launch_bounds__(256)
+copy_matrix_kernel(int M, int N, int m_blocks, const T *src, int64_t lds_, T *dst, int64_t ldd) {
+    const int m = (blockIdx.x % m_blocks) * 256 + threadIdx.x;
+    const int n = blockIdx.x / m_blocks;
+    if (m < M && n < N) dst[(int64_t)n * ldd + m] = src[(int64_t)n * lds_ + m];
+}
+
+template <typename T>
+hipError_t syrk_colmajor(bool lower, bool trans, int N, int K, T alpha, const T *A, int64_t lda, T beta, T *C,
+                         int64_t ldc, hipStream_t stream) {
+    GemmTri tri;
+    tri.tri_c = lower ? 1 : 2;
+    // op(A) op(A)^T: the second operand is the same matrix with the opposite transpose flag.
+    return launch_gemm<T>(trans, !trans, false, false, N, N, K, alpha, A, lda, A, lda, beta, C, ldc, stream, &tri);
+}
+
+template <typename T>
+hipError_t trmm_colmajor(bool right, bool lower, bool trans, bool conj, bool unit, int M, int N, T alpha, const T *A,
+                         int64_t lda, T *B, int64_t ldb, hipStream_t stream) {
+    const int64_t ldw = ((int64_t)M + 63) / 64 * 64;
+    T *W = (T *)workspace_get(stream, (size_t)ldw * N * sizeof(T), 1);
+    if (!W) return hipErrorOutOfMemory;
+    const int mb = (M + 255) / 256;
+    if ((int64_t)mb * N > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(copy_matrix_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
+                       (const T *)B, ldb, W, ldw);
+    hipError_t err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    GemmTri tri;
+    const bool op_lower = lower != trans;  // op(A) is lower triangular
+    if (!right) {
+        // op(A)(m,k): lower keeps k <= m
+        tri.tri_a = op_lower ? 1 : 2;
+        tri.unit_a = unit ? 1 : 0;
+        return launch_gemm<T>(trans, false, conj, false, M, N, M, alpha, A, lda, W, ldw, T(), B, ldb, stream, &tri);
+    }
+    // op(A)(k,n): lower keeps k >= n
+    tri.tri_b = op_lower ? 2 : 1;
+    tri.unit_b = unit ? 1 : 0;
+    return launch_gemm<T>(false, trans, false, conj, M, N, N, alpha, W, ldw, A, lda, T(), B, ldb, stream, &tri);
+}
+
+template <typename T>
+hipError_t symm_colmajor(bool right, bool lower, int M, int N, T alpha, const T *A, int64_t lda, const T *B,
+                         int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream) {
+    GemmTri stored, mirrored;
+    hipError_t err;
+    if (!right) {
+        // stored triangle as it lies: lower keeps k <= m; its strict part read transposed
+        // fills the other side: op(A)(m,k) = A(k,m), stored for k > m (lower) / k < m (upper).
+        stored.tri_a = lower ? 1 : 2;
+        mirrored.tri_a = lower ? 2 : 1;
+        mirrored.unit_a = 2;
+        err = launch_gemm<T>(false, false, false, false, M, N, M, alpha, A, lda, B, ldb, beta, C, ldc, stream, &stored);
+        if (err != hipSuccess) return err;
+        return launch_gemm<T>(true, false, false, false, M, N, M, alpha, A, lda, B, ldb, el_one<T>(), C, ldc, stream,
+                              &mirrored);
+    }
+    // A is the second operand, op(A)(k,n): lower keeps k >= n.
+    stored.tri_b = lower ? 2 : 1;
+    mirrored.tri_b = lower ? 1 : 2;
+    mirrored.unit_b = 2;
+    err = launch_gemm<T>(false, false, false, false, M, N, N, alpha, B, ldb, A, lda, beta, C, ldc, stream, &stored);
+    if (err != hipSuccess) return err;
+    return launch_gemm<T>(false, true, false, false, M, N, N, alpha, B, ldb, A, lda, el_one<T>(), C, ldc, stream,
+                          &mirrored);
+}
+
+#define CBA_INSTANTIATE(T)                                                                                         \
+    template hipError_t syrk_colmajor<T>(bool, bool, int, int, T, const T *, int64_t, T, T *, int64_t, hipStream_t); \
+    template hipError_t trmm_colmajor<T>(bool, bool, bool, bool, bool, int, int, T, const T *, int64_t, T *, int64_t, \
+                                         hipStream_t);                                                             \
+    template hipError_t symm_colmajor<T>(bool, bool, int, int, T, const T *, int64_t, const T *, int64_t, T, T *,   \
+                                         int64_t, hipStream_t);
+CBA_INSTANTIATE(float)
+CBA_INSTANTIATE(double)
+CBA_INSTANTIATE(Cx<float>)
+CBA_INSTANTIATE(Cx<double>)
+#undef CBA_INSTANTIATE
+
+}  // namespace cba

@@ -162,6 +162,70 @@ clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo,
                          double alpha, const double *A, size_t offA, size_t lda,
                          double *B, size_t offB, size_t ldb, hipStream_t stream);
 
+/* ---- GEMM-shaped neighbours on the same MFMA core: SYRK, TRMM, SYMM (all four types) ---- */
+
+/* Replace clblas{S,D,C,Z}syrk (src/clBLAS.h:8278-8503, src/library/blas/xsyrk.c:27-233).
+ *   C <- alpha * op(A) * op(A)^T + beta * C, C is N x N and only its `uplo` triangle is read
+ * or written; op(A) is N x K (transA == NoTrans: A is N x K, else K x N).  Validation follows
+ * doSyrk (xsyrk.c:56-72): null A/C -> clblasInvalidMat{A,C}; clblasConjTrans with a complex
+ * type -> clblasInvalidValue; sizes of A, then C (K == 0 -> clblasInvalidDim). */
+clblasStatus clblasSsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         float alpha, const float *A, size_t offA, size_t lda, float beta,
+                         float *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8278-8297 */
+clblasStatus clblasDsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         double alpha, const double *A, size_t offA, size_t lda, double beta,
+                         double *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8350-8369 */
+clblasStatus clblasCsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, FloatComplex beta,
+                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8416-8435 */
+clblasStatus clblasZsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, DoubleComplex beta,
+                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8484-8503 */
+
+/* Replace clblas{S,D,C,Z}trmm (src/clBLAS.h:7696-7928, src/library/blas/xtrmm.c:27-245).
+ *   side == Left : B <- alpha * op(A) * B,  A is M x M
+ *   side == Right: B <- alpha * B * op(A),  A is N x N
+ * A triangular; only its `uplo` triangle is read and, with diag == Unit, not its diagonal.
+ * Validation as clblas?trsm (xtrmm.c:47-64).  Uses a library-owned M x N device workspace. */
+clblasStatus clblasStrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, float alpha,
+                         const float *A, size_t offA, size_t lda,
+                         float *B, size_t offB, size_t ldb, hipStream_t stream); /* src/clBLAS.h:7696-7716 */
+clblasStatus clblasDtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, double alpha,
+                         const double *A, size_t offA, size_t lda,
+                         double *B, size_t offB, size_t ldb, hipStream_t stream); /* src/clBLAS.h:7771-7791 */
+clblasStatus clblasCtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, FloatComplex alpha,
+                         const FloatComplex *A, size_t offA, size_t lda,
+                         FloatComplex *B, size_t offB, size_t ldb, hipStream_t stream); /* src/clBLAS.h:7838-7858 */
+clblasStatus clblasZtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, DoubleComplex alpha,
+                         const DoubleComplex *A, size_t offA, size_t lda,
+                         DoubleComplex *B, size_t offB, size_t ldb, hipStream_t stream); /* src/clBLAS.h:7908-7928 */
+
+/* Replace clblas{S,D,C,Z}symm (src/clBLAS.h:8897-9145, src/library/blas/xsymm.c:33-429).
+ *   side == Left : C <- alpha * A * B + beta * C,  A is M x M
+ *   side == Right: C <- alpha * B * A + beta * C,  A is N x N
+ * A symmetric (not Hermitian), only its `uplo` triangle is read; B and C are M x N.
+ * Validation follows doSymm (xsymm.c:50-71): null A/B/C, sizes of A, B, C in that order. */
+clblasStatus clblasSsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N,
+                         float alpha, const float *A, size_t offA, size_t lda,
+                         const float *B, size_t offB, size_t ldb, float beta,
+                         float *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8897-8919 */
+clblasStatus clblasDsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N,
+                         double alpha, const double *A, size_t offA, size_t lda,
+                         const double *B, size_t offB, size_t ldb, double beta,
+                         double *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8978-9000 */
+clblasStatus clblasCsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N,
+                         FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                         const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta,
+                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9051-9073 */
+clblasStatus clblasZsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N,
+                         DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                         const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
+                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9123-9145 */
+
 #ifdef __cplusplus
 }
 #endif

@@ -61,6 +61,16 @@ def lib():
             f = getattr(L, name)
             f.restype = _i
             f.argtypes = [_i, _i, _i, _i, _i, _sz, _sz, real, _vp, _sz, _sz, _vp, _sz, _sz]
+        for t in "sdcz":
+            f = getattr(L, "oracle_%ssyrk" % t)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz]
+            f = getattr(L, "oracle_%strmm" % t)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz]
+            f = getattr(L, "oracle_%ssymm" % t)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _sz, _sz]
         L.oracle_check_gemm.restype = _i
         L.oracle_check_gemm.argtypes = [_i, _i, _i, _sz, _sz, _sz, _i, _sz, _sz, _sz, _i, _sz, _sz, _sz, _i, _sz,
                                         _sz, _sz]
@@ -99,6 +109,10 @@ def ref_lib():
             f = getattr(L, name)
             f.restype = None
             f.argtypes = [_i, _i, _i, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz]
+        L.ref_naive_syrk.restype = None
+        L.ref_naive_syrk.argtypes = [_i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _vp, _sz]
+        L.ref_naive_trmm.restype = None
+        L.ref_naive_trmm.argtypes = [_i, _i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _sz]
         for name, real in (("ref_naive_strsm", ctypes.c_float), ("ref_naive_dtrsm", ctypes.c_double)):
             f = getattr(L, name)
             f.restype = None
@@ -176,6 +190,57 @@ def trsm_blocked(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, 
     f = lib().oracle_strsm_blocked if ref.dtype == np.float32 else lib().oracle_dtrsm_blocked
     return f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha, _p(A), offA, lda, _p(B), offB,
              ldb)
+
+
+_PREFIX = {np.dtype(np.float32): "s", np.dtype(np.float64): "d", np.dtype(np.complex64): "c",
+           np.dtype(np.complex128): "z"}
+
+
+def prefix(a):
+    """Routine-family letter (s, d, c, z) of a buffer's dtype."""
+    return _PREFIX[a.dtype]
+
+
+def _sc(x, ref):
+    """alpha / beta as the array the level-3 routines take by address."""
+    if _is_complex(ref):
+        return _scalar(x, ref.dtype)
+    return np.array([x], dtype=ref.dtype)
+
+
+def syrk(order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc):
+    ref = C if C is not None else A
+    al, be = _sc(alpha, ref), _sc(beta, ref)
+    return getattr(lib(), "oracle_%ssyrk" % prefix(ref))(int(order), int(uplo), int(transA), N, K, _p(al), _p(A), offA,
+                                                         lda, _p(be), _p(C), offC, ldc)
+
+
+def trmm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
+    ref = B if B is not None else A
+    al = _sc(alpha, ref)
+    return getattr(lib(), "oracle_%strmm" % prefix(ref))(int(order), int(side), int(uplo), int(transA), int(diag), M, N,
+                                                         _p(al), _p(A), offA, lda, _p(B), offB, ldb)
+
+
+def symm(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    ref = C if C is not None else (A if A is not None else B)
+    al, be = _sc(alpha, ref), _sc(beta, ref)
+    return getattr(lib(), "oracle_%ssymm" % prefix(ref))(int(order), int(side), int(uplo), M, N, _p(al), _p(A), offA,
+                                                         lda, _p(B), offB, ldb, _p(be), _p(C), offC, ldc)
+
+
+def ref_syrk(order, uplo, transA, N, K, alpha, A, lda, beta, C, ldc):
+    """Reference naive syrk (no offsets)."""
+    al, be = _sc(alpha, C), _sc(beta, C)
+    ref_lib().ref_naive_syrk("sdcz".index(prefix(C)), int(order), int(uplo), int(transA), N, K, _p(al), _p(A), lda,
+                             _p(be), _p(C), ldc)
+
+
+def ref_trmm(order, side, uplo, transA, diag, M, N, alpha, A, lda, B, ldb):
+    """Reference naive trmm (no offsets)."""
+    al = _sc(alpha, B)
+    ref_lib().ref_naive_trmm("sdcz".index(prefix(B)), int(order), int(side), int(uplo), int(transA), int(diag), M, N,
+                             _p(al), _p(A), lda, _p(B), ldb)
 
 
 def check_gemm(order, transA, transB, M, N, K, haveA, offA, lda, memA, haveB, offB, ldb, memB, haveC, offC, ldc,

@@ -27,6 +27,13 @@
  *   oracle_{s,d}trsm_blocked- the same, plus agreement with the naive solver within the
  *                             reference's own per-element bound (trsm-delta.h:44-240 style),
  *                             NaN-poisoned unused triangle, zero-diagonal -> 1 behaviour.
+ *   oracle_{s,d,c,z}{syrk,trmm,symm} (level3.inc)
+ *                           - exact-integer inputs against exact integer products for every
+ *                             order / side / triangle / transpose / diagonal combination with
+ *                             the unused triangle NaN-poisoned; the reference's own naive syrk
+ *                             and trmm (oracle/_ref); SYMM, which has no naive statement in the
+ *                             reference, against oracle GEMM on the explicitly symmetrised
+ *                             matrix; TRMM followed by TRSM returns the input.
  *   oracle_check_*          - expectations of src/tests/functional/func-error.cpp:58-104 and
  *                             the branch table of generic/common.c:585-688.
  *   Bit-for-bit output of the OpenCL kernels (implementation-defined `mad` contraction,
@@ -51,6 +58,7 @@ enum { UNIT = 0, NON_UNIT = 1 };
 enum { LEFT = 0, RIGHT = 1 };
 enum {
     ST_SUCCESS = 0,
+    ST_INVALID_VALUE = -30,
     ST_NOT_IMPLEMENTED = -1024,
     ST_INVALID_MAT_A = -1022,
     ST_INVALID_MAT_B = -1021,
@@ -369,6 +377,38 @@ CGEMM_FRONT(oracle_zgemm, double, zgemm_colmajor)
 
 CGEMM_EXACT(oracle_cgemm_exact, float, double, fabs)
 CGEMM_EXACT(oracle_zgemm_exact, double, long double, fabsl)
+
+/* ------------------------------------------------------------------------------------ */
+/* SYRK / TRMM / SYMM (the GEMM-shaped neighbours), all four types: level3.inc            */
+/* ------------------------------------------------------------------------------------ */
+#define P s
+#define R float
+#define NC 1
+#include "level3.inc"
+#undef P
+#undef R
+#undef NC
+#define P d
+#define R double
+#define NC 1
+#include "level3.inc"
+#undef P
+#undef R
+#undef NC
+#define P c
+#define R float
+#define NC 2
+#include "level3.inc"
+#undef P
+#undef R
+#undef NC
+#define P z
+#define R double
+#define NC 2
+#include "level3.inc"
+#undef P
+#undef R
+#undef NC
 
 /* ------------------------------------------------------------------------------------ */
 /* TRSM                                                                                  */

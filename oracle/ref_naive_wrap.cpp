@@ -16,6 +16,14 @@ using std::isnan;
 
 #include REF_NAIVE_BLAS_CPP
 
+// Scalar of type T (a real, or a complex made of two R) read from its address.
+template <typename T, typename R> static T ref_scalar(const void *p) {
+    T z;
+    *(R *)&z = ((const R *)p)[0];
+    if (sizeof(T) == 2 * sizeof(R)) ((R *)&z)[1] = ((const R *)p)[1];
+    return z;
+}
+
 extern "C" {
 
 void ref_naive_sgemm(int order, int transA, int transB, size_t M, size_t N, size_t K, float alpha, const float *A,
@@ -66,6 +74,31 @@ void ref_naive_dtrsm(int order, int side, int uplo, int transA, int diag, size_t
     NaiveBlas::trsm<double>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasSide)side,
                             (NaiveBlas::clblasUplo)uplo, (NaiveBlas::clblasTranspose)transA,
                             (NaiveBlas::clblasDiag)diag, M, N, alpha, A, lda, B, ldb);
+}
+
+// SYRK and TRMM of the reference's naive BLAS; scalars by address, T selected by `type`
+// (0 float, 1 double, 2 FloatComplex, 3 DoubleComplex).
+#define REF_DISPATCH(CALL)                                                            \
+    switch (type) {                                                                   \
+    case 0: { typedef float T; typedef float R; CALL; break; }                        \
+    case 1: { typedef double T; typedef double R; CALL; break; }                      \
+    case 2: { typedef NaiveBlas::FloatComplex T; typedef float R; CALL; break; }      \
+    default: { typedef NaiveBlas::DoubleComplex T; typedef double R; CALL; break; }   \
+    }
+
+void ref_naive_syrk(int type, int order, int uplo, int trans, size_t N, size_t K, const void *alpha, const void *A,
+                    size_t lda, const void *beta, void *C, size_t ldc) {
+    REF_DISPATCH((NaiveBlas::syrk<T>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasUplo)uplo,
+                                     (NaiveBlas::clblasTranspose)trans, N, K, ref_scalar<T, R>(alpha), (const T *)A,
+                                     lda, ref_scalar<T, R>(beta), (T *)C, ldc)))
+}
+
+void ref_naive_trmm(int type, int order, int side, int uplo, int trans, int diag, size_t M, size_t N,
+                    const void *alpha, const void *A, size_t lda, void *B, size_t ldb) {
+    REF_DISPATCH((NaiveBlas::trmm<T>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasSide)side,
+                                     (NaiveBlas::clblasUplo)uplo, (NaiveBlas::clblasTranspose)trans,
+                                     (NaiveBlas::clblasDiag)diag, M, N, ref_scalar<T, R>(alpha), (const T *)A, lda,
+                                     (T *)B, ldb)))
 }
 
 }  // extern "C"

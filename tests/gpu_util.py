@@ -32,3 +32,43 @@ def trsm(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
     st = fn(order, side, uplo, tA, diag, M, N, alpha, dA, offA, lda, dB, offB, ldb)
     torch.cuda.synchronize()
     return st, dB.cpu().numpy()
+
+
+def _forced_tile(tile):
+    class _Ctx:
+        def __enter__(self):
+            if tile is not None:
+                os.environ["CLBLAS_AMD_GEMM_TILE"] = str(tile)
+
+        def __exit__(self, *a):
+            os.environ.pop("CLBLAS_AMD_GEMM_TILE", None)
+    return _Ctx()
+
+
+_PREFIX = {np.dtype(np.float32): "S", np.dtype(np.float64): "D", np.dtype(np.complex64): "C",
+           np.dtype(np.complex128): "Z"}
+
+
+def syrk(order, uplo, tA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, tile=None):
+    dA, dC = _dev(A), _dev(C)
+    with _forced_tile(tile):
+        st = clblas_amd.syrk(_PREFIX[C.dtype], order, uplo, tA, N, K, alpha, dA, offA, lda, beta, dC, offC, ldc)
+        torch.cuda.synchronize()
+    return st, dC.cpu().numpy()
+
+
+def trmm(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, tile=None):
+    dA, dB = _dev(A), _dev(B)
+    with _forced_tile(tile):
+        st = clblas_amd.trmm(_PREFIX[B.dtype], order, side, uplo, tA, diag, M, N, alpha, dA, offA, lda, dB, offB, ldb)
+        torch.cuda.synchronize()
+    return st, dB.cpu().numpy()
+
+
+def symm(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, tile=None):
+    dA, dB, dC = _dev(A), _dev(B), _dev(C)
+    with _forced_tile(tile):
+        st = clblas_amd.symm(_PREFIX[C.dtype], order, side, uplo, M, N, alpha, dA, offA, lda, dB, offB, ldb, beta, dC,
+                             offC, ldc)
+        torch.cuda.synchronize()
+    return st, dC.cpu().numpy()

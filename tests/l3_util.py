@@ -1,0 +1,88 @@
+"""Input builders and exact expectations shared by the SYRK / TRMM / SYMM tests (CPU oracle
+pinning and GPU parity)."""
+import numpy as np
+
+import oracle
+from helpers import COL, ROW, NOTRANS, TRANS, CONJ, UPPER, LOWER, UNIT, NONUNIT, LEFT, RIGHT, logical_view, mem_dims
+
+REAL = [np.float32, np.float64]
+CPLX = [np.complex64, np.complex128]
+ALL = REAL + CPLX
+
+
+def is_cplx(dtype):
+    return np.dtype(dtype).kind == "c"
+
+
+def nan_of(dtype):
+    return dtype(complex(np.nan, np.nan)) if is_cplx(dtype) else dtype(np.nan)
+
+
+def scalars(dtype):
+    """Exactly representable alpha, beta (Gaussian integers for the complex types)."""
+    return ((2 - 1j), (-1 + 2j)) if is_cplx(dtype) else (2.0, -3.0)
+
+
+def real_scalars(dtype):
+    return ((0.7 - 0.3j), (-1.3 + 0.5j)) if is_cplx(dtype) else (0.7, -1.3)
+
+
+def matrix(order, rows, cols, off, pad, seed, dtype, integer, limit=8):
+    """1-D buffer (+ld) holding a rows x cols matrix in `order` with `pad` extra leading
+    elements per stride and `off` leading elements."""
+    inner, outer = mem_dims(order, NOTRANS, rows, cols)
+    ld = inner + pad
+    n = off + outer * ld
+    buf = oracle.integers(n, seed, limit, dtype) if integer else oracle.uniform(n, seed, dtype)
+    return buf, ld
+
+
+def tri_mask(n, lower):
+    i, j = np.indices((n, n))
+    return i >= j if lower else i <= j
+
+
+def poison_triangle(buf, order, n, off, ld, uplo, unit=False):
+    """NaN everywhere in the n x n square except the `uplo` triangle (and, with unit, NaN on the
+    diagonal too): anything that reads the wrong element shows up as NaN."""
+    v = logical_view(buf, order, NOTRANS, n, n, off, ld)
+    keep = tri_mask(n, uplo == LOWER)
+    if unit:
+        keep = keep & ~np.eye(n, dtype=bool)
+    v[~keep] = nan_of(buf.dtype.type)
+
+
+def tri_dense(buf, order, n, off, ld, uplo, unit):
+    """The triangular matrix the routines see: zeros outside the triangle, ones on a unit diagonal."""
+    v = logical_view(buf, order, NOTRANS, n, n, off, ld)
+    t = np.where(tri_mask(n, uplo == LOWER), v, 0).astype(np.complex128 if is_cplx(buf.dtype) else np.float64)
+    if unit:
+        np.fill_diagonal(t, 1)
+    return t
+
+
+def sym_dense(buf, order, n, off, ld, uplo):
+    v = logical_view(buf, order, NOTRANS, n, n, off, ld)
+    wide = np.complex128 if is_cplx(buf.dtype) else np.float64
+    t = np.where(tri_mask(n, uplo == LOWER), v, 0).astype(wide)
+    return t + t.T - np.diag(np.diag(t))
+
+
+def op(x, trans):
+    return x if trans == NOTRANS else (x.T if trans == TRANS else x.conj().T)
+
+
+def abs1(x):
+    """|re| + |im| (plain |x| for real data)."""
+    return np.abs(x.real) + np.abs(x.imag) if np.iscomplexobj(x) else np.abs(x)
+
+
+def bound(K, mag, dtype, c=2.0):
+    """c (2K+6) u mag for complex, c (K+2) u mag for real data (see helpers.gemm_bound)."""
+    from helpers import cgemm_bound, gemm_bound
+    return cgemm_bound(K, mag, dtype, c) if is_cplx(dtype) else gemm_bound(K, mag, dtype, c)
+
+
+def err(got, want):
+    d = got - want
+    return np.maximum(np.abs(d.real), np.abs(d.imag)) if np.iscomplexobj(d) else np.abs(d)
