@@ -10,8 +10,8 @@ namespace cba {
 //   1:  64x64x8,  wave 32x32, split-K capable
 static const TileEntry<Cx<float>> *c32_tiles(int *n) {
     static const TileEntry<Cx<float>> tab[] = {
-        make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, false, true>(0.92),
-        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true, true>(0.80),
+        make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, false, true>(0.93),
+        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true, true>(0.84),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

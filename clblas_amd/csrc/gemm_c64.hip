@@ -8,8 +8,8 @@ namespace cba {
 //   1:  64x64x8, wave 32x32, split-K capable
 static const TileEntry<Cx<double>> *c64_tiles(int *n) {
     static const TileEntry<Cx<double>> tab[] = {
-        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, false, true>(0.92),
-        make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true>(0.84),
+        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, false, true>(0.93),
+        make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true>(0.86),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

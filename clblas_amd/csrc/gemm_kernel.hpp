@@ -406,21 +406,40 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     }
     int tm, tn;
     if (TRI && p.tri_c) {
-        // Only tiles that touch the stored triangle exist: row tm holds the columns
-        // [0, last] (lower) or [first, tiles_n) (upper); walk the rows until `tile` fits.
+        // Only tiles that touch the stored triangle exist: row r holds the columns [0, last]
+        // (lower) or [first, tiles_n) (upper).  They are walked like the full grid - groups of
+        // `group_m` rows, column by column inside a group - so that neighbours in the list
+        // share panels; the walk is replayed here until `tile` is reached.
         tm = 0;
         tn = 0;
-        for (int r = 0; r < p.tiles_m; ++r) {
-            int first = 0, count;
-            if (p.tri_c == 1) {
-                const int last = (r * BM + BM - 1) / BN;
-                count = last + 1 < p.tiles_n ? last + 1 : p.tiles_n;
-            } else {
-                first = (r * BM) / BN;
-                count = first < p.tiles_n ? p.tiles_n - first : 0;
+        bool found = false;
+        for (int r0 = 0; r0 < p.tiles_m && !found; r0 += p.group_m) {
+            const int r1 = r0 + p.group_m < p.tiles_m ? r0 + p.group_m : p.tiles_m;
+            int in_group = 0;
+            for (int r = r0; r < r1; ++r) {
+                if (p.tri_c == 1) {
+                    const int last = (r * BM + BM - 1) / BN;
+                    in_group += last + 1 < p.tiles_n ? last + 1 : p.tiles_n;
+                } else {
+                    const int first = (r * BM) / BN;
+                    in_group += first < p.tiles_n ? p.tiles_n - first : 0;
+                }
             }
-            if (tile < count) { tm = r; tn = first + tile; break; }
-            tile -= count;
+            if (tile >= in_group) { tile -= in_group; continue; }
+            for (int c = 0; c < p.tiles_n; ++c) {
+                int lo = r0, hi = r1;  // rows [lo, hi) of the group hold column c
+                if (p.tri_c == 1) {
+                    const int need = c * BN - BM + 1;  // first row index that reaches column c
+                    const int rmin = need <= 0 ? 0 : (need + BM - 1) / BM;
+                    lo = rmin > r0 ? rmin : r0;
+                } else {
+                    const int rmax = (c * BN + BN - 1) / BM;
+                    hi = rmax + 1 < r1 ? rmax + 1 : r1;
+                }
+                const int cnt = hi > lo ? hi - lo : 0;
+                if (tile < cnt) { tm = lo + tile; tn = c; found = true; break; }
+                tile -= cnt;
+            }
         }
     } else {
         const int per_group = p.group_m * p.tiles_n;

@@ -68,10 +68,29 @@ static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b;
 // its MFMA pipes, so time is quantised per CU, not per resident workgroup:
 //     time ~ ceil(tiles / 256) * BM * BN / eff
 // with eff the measured MFMA efficiency of that tile shape on large problems (padding is
-// paid for automatically because whole tiles are counted).  The smallest tile adds a K
+// paid for automatically because whole tiles are counted; for SYRK only the tiles of the
+// stored triangle count).  The smallest tile adds a K
 // split when even it cannot give every CU a workgroup.
+// Number of bm x bn tiles of an M x N matrix that touch its lower (tri_c == 1) or upper (2)
+// triangle; all of them for tri_c == 0.  Row r holds the columns [0, last] resp. [first, end).
+static inline int64_t active_tiles(int M, int N, int bm, int bn, int tri_c) {
+    const int64_t tiles_m = ceil_div64(M, bm), tiles_n = ceil_div64(N, bn);
+    if (!tri_c) return tiles_m * tiles_n;
+    int64_t total = 0;
+    for (int64_t r = 0; r < tiles_m; ++r) {
+        if (tri_c == 1) {
+            const int64_t last = (r * bm + bm - 1) / bn;
+            total += last + 1 < tiles_n ? last + 1 : tiles_n;
+        } else {
+            const int64_t first = (r * bm) / bn;
+            total += first < tiles_n ? tiles_n - first : 0;
+        }
+    }
+    return total;
+}
+
 template <typename T>
-static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, bool need_tri,
+static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, bool need_tri, int tri_c,
                         int *tile_out, int *splits_out) {
     const int64_t kCUs = 256;
     int pick = ntab - 1;  // table is ordered large -> small
@@ -82,8 +101,9 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         bool have = false;
         for (int i = 0; i < ntab; ++i) {
             if (need_tri && !tab[i].tri[0]) continue;
-            const int64_t t = ceil_div64(M, tab[i].bm) * ceil_div64(N, tab[i].bn);
-            const double cost = (double)ceil_div64(t, kCUs) * tab[i].bm * tab[i].bn / tab[i].eff;
+            const int64_t t = active_tiles(M, N, tab[i].bm, tab[i].bn, tri_c);
+            double cost = (double)ceil_div64(t, kCUs) * tab[i].bm * tab[i].bn / tab[i].eff;
+            if (t <= kCUs) cost /= 0.85;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             if (!have || cost < best) { best = cost; pick = i; have = true; }
         }
     }
@@ -127,7 +147,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     }
 
     int tile, splits;
-    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, &tile, &splits);
+    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, need_tri ? tri->tri_c : 0, &tile, &splits);
     const TileEntry<T> &e = tab[tile];
 
     GemmParams<T> p;
@@ -158,24 +178,14 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         fn = e.tri[idx];
         p.tri_c = tri->tri_c; p.tri_a = tri->tri_a; p.tri_b = tri->tri_b;
         p.unit_a = tri->unit_a; p.unit_b = tri->unit_b;
-        if (p.tri_c) {
-            // same enumeration as the kernel's: tiles that touch the stored triangle
-            ntiles = 0;
-            for (int r = 0; r < p.tiles_m; ++r) {
-                if (p.tri_c == 1) {
-                    const int64_t last = ((int64_t)r * e.bm + e.bm - 1) / e.bn;
-                    ntiles += last + 1 < p.tiles_n ? last + 1 : p.tiles_n;
-                } else {
-                    const int64_t first = ((int64_t)r * e.bm) / e.bn;
-                    ntiles += first < p.tiles_n ? p.tiles_n - first : 0;
-                }
-            }
-        }
+        if (p.tri_c) ntiles = active_tiles(M, N, e.bm, e.bn, p.tri_c);  // the kernel enumerates the same set
         if (p.tri_a || p.tri_b) {
-            // Tiles differ in depth: start the deepest first and deal consecutive tiles to
-            // different XCDs so that every XCD gets the same mix.
+            // Tiles differ in depth (by tile row for a triangular A, by tile column for B):
+            // start them strictly deepest first - row by row resp. column by column - and deal
+            // consecutive tiles to different XCDs so that every XCD gets the same mix.
             p.rev_m = p.tri_a == 1;
             p.rev_n = p.tri_b == 1;
+            p.group_m = p.tri_a ? 1 : p.tiles_m;
             p.xcd_remap = 0;
         }
     }
