@@ -1,8 +1,8 @@
 // clblas_amd-client: benchmark command line for libclblas_amd.so.
 //
 // Takes the place of the reference's clBLAS-client (src/client/client.cpp:80-112 for the
-// option names, src/client/clfunc_xgemm.hpp:95-107 and clfunc_xtrsm.hpp:70-92 for the
-// GFLOP/s formulas) for the two function families this library implements, and prints the
+// option names, src/client/clfunc_x{gemm,trsm,trmm,syrk,symm}.hpp for the GFLOP/s formulas)
+// for the function families this library implements, and prints the
 // CSV schema of the reference's published benchmark files (doc/performance/**.csv):
 //   m,n,k,lda,ldb,ldc,offa,offb,offc,alpha,beta,order,transa,transb,side,uplo,diag,
 //   function,device,library,numQueues,label,GFLOPS
@@ -44,7 +44,7 @@ void usage() {
         "  -o/--order 0|1                                0 = row major, 1 = column major\n"
         "  --transposeA 0|1|2  --transposeB 0|1|2\n"
         "  --side 0|1  --uplo 0|1  --diag 0|1            0 = left/upper/unit\n"
-        "  -f/--function gemm|trsm   -r/--precision s|d\n"
+        "  -f/--function gemm|trsm|trmm|syrk|symm   -r/--precision s|d|c|z (trsm: s|d)\n"
         "  -p/--profile N                                timed samples (default 20)\n"
         "  --apiCallCount N                              calls per sample (default 10)\n"
         "  --label TEXT  --noheader");
@@ -96,30 +96,95 @@ size_t footprint(int order, int trans, size_t rows, size_t cols, size_t off, siz
     return off + (outer - 1) * ld + inner;
 }
 
-template <typename T> void fill(std::vector<T> &v, uint64_t seed, double scale, double shift) {
+// Fills `count` reals (matrix elements, or re/im pairs of them) with uniform values.
+template <typename R> void fill(std::vector<R> &v, uint64_t seed, double scale) {
     uint64_t s = seed * 0x9e3779b97f4a7c15ULL + 1;
     for (auto &x : v) {
         s = s * 6364136223846793005ULL + 1442695040888963407ULL;
-        x = (T)(((double)(s >> 40) / (double)(1 << 24) * 2.0 - 1.0) * scale + shift);
+        x = (R)(((double)(s >> 40) / (double)(1 << 24) * 2.0 - 1.0) * scale);
     }
 }
 
-template <typename T> double run_case(const Options &o, size_t m, size_t n, size_t k, bool &ok) {
-    const bool gemm = o.function == "gemm";
-    const size_t an = o.side == 0 ? m : n;  // order of the triangular matrix
+// One set of overloads per element type, so that run_case can be written once.
+template <typename T> struct Type;
+template <> struct Type<float> { typedef float Real; static const int NC = 1; static float scalar(double x) { return (float)x; } };
+template <> struct Type<double> { typedef double Real; static const int NC = 1; static double scalar(double x) { return x; } };
+template <> struct Type<FloatComplex> {
+    typedef float Real; static const int NC = 2;
+    static FloatComplex scalar(double x) { FloatComplex z; z.s[0] = (float)x; z.s[1] = 0.f; return z; }
+};
+template <> struct Type<DoubleComplex> {
+    typedef double Real; static const int NC = 2;
+    static DoubleComplex scalar(double x) { DoubleComplex z; z.s[0] = x; z.s[1] = 0.0; return z; }
+};
+
+#define CLIENT_OVERLOADS(T, L)                                                                                       \
+    clblasStatus gemm(clblasOrder o, clblasTranspose ta, clblasTranspose tb, size_t m, size_t n, size_t k, T al,     \
+                      const T *a, size_t oa, size_t lda, const T *b, size_t ob, size_t ldb, T be, T *c, size_t oc,   \
+                      size_t ldc, hipStream_t s) {                                                                   \
+        return clblas##L##gemm(o, ta, tb, m, n, k, al, a, oa, lda, b, ob, ldb, be, c, oc, ldc, s);                   \
+    }                                                                                                                \
+    clblasStatus syrk(clblasOrder o, clblasUplo u, clblasTranspose ta, size_t n, size_t k, T al, const T *a,         \
+                      size_t oa, size_t lda, T be, T *c, size_t oc, size_t ldc, hipStream_t s) {                     \
+        return clblas##L##syrk(o, u, ta, n, k, al, a, oa, lda, be, c, oc, ldc, s);                                   \
+    }                                                                                                                \
+    clblasStatus trmm(clblasOrder o, clblasSide sd, clblasUplo u, clblasTranspose ta, clblasDiag d, size_t m,        \
+                      size_t n, T al, const T *a, size_t oa, size_t lda, T *b, size_t ob, size_t ldb,                \
+                      hipStream_t s) {                                                                               \
+        return clblas##L##trmm(o, sd, u, ta, d, m, n, al, a, oa, lda, b, ob, ldb, s);                                \
+    }                                                                                                                \
+    clblasStatus symm(clblasOrder o, clblasSide sd, clblasUplo u, size_t m, size_t n, T al, const T *a, size_t oa,   \
+                      size_t lda, const T *b, size_t ob, size_t ldb, T be, T *c, size_t oc, size_t ldc,              \
+                      hipStream_t s) {                                                                               \
+        return clblas##L##symm(o, sd, u, m, n, al, a, oa, lda, b, ob, ldb, be, c, oc, ldc, s);                       \
+    }
+CLIENT_OVERLOADS(float, S)
+CLIENT_OVERLOADS(double, D)
+CLIENT_OVERLOADS(FloatComplex, C)
+CLIENT_OVERLOADS(DoubleComplex, Z)
+#undef CLIENT_OVERLOADS
+clblasStatus trsm(clblasOrder o, clblasSide sd, clblasUplo u, clblasTranspose ta, clblasDiag d, size_t m, size_t n,
+                  float al, const float *a, size_t oa, size_t lda, float *b, size_t ob, size_t ldb, hipStream_t s) {
+    return clblasStrsm(o, sd, u, ta, d, m, n, al, a, oa, lda, b, ob, ldb, s);
+}
+clblasStatus trsm(clblasOrder o, clblasSide sd, clblasUplo u, clblasTranspose ta, clblasDiag d, size_t m, size_t n,
+                  double al, const double *a, size_t oa, size_t lda, double *b, size_t ob, size_t ldb, hipStream_t s) {
+    return clblasDtrsm(o, sd, u, ta, d, m, n, al, a, oa, lda, b, ob, ldb, s);
+}
+template <typename T>
+clblasStatus trsm(clblasOrder, clblasSide, clblasUplo, clblasTranspose, clblasDiag, size_t, size_t, T, const T *, size_t,
+                  size_t, T *, size_t, size_t, hipStream_t) {
+    return clblasNotImplemented;  // complex TRSM is not part of this library
+}
+
+enum Fn { FN_GEMM, FN_TRSM, FN_TRMM, FN_SYRK, FN_SYMM };
+
+template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t n, size_t k, bool &ok) {
+    typedef typename Type<T>::Real R;
+    const int NC = Type<T>::NC;
+    const bool tri = fn == FN_TRSM || fn == FN_TRMM;    // A triangular, B in place
+    const size_t an = o.side == 0 ? m : n;                // order of the triangular / symmetric matrix
     auto tight = [&](int trans, size_t rows, size_t cols) { return ((o.order == 1) == (trans == 0)) ? rows : cols; };
-    const size_t lda = o.lda ? o.lda : (gemm ? tight(o.transA, m, k) : an);
-    const size_t ldb = o.ldb ? o.ldb : (gemm ? tight(o.transB, k, n) : tight(0, m, n));
-    const size_t ldc = o.ldc ? o.ldc : tight(0, m, n);
-    const size_t na = gemm ? footprint(o.order, o.transA, m, k, o.offA, lda) : footprint(o.order, 0, an, an, o.offA, lda);
-    const size_t nb = gemm ? footprint(o.order, o.transB, k, n, o.offBX, ldb) : footprint(o.order, 0, m, n, o.offBX, ldb);
-    const size_t nc = gemm ? footprint(o.order, 0, m, n, o.offCY, ldc) : 1;
-    std::vector<T> ha(na), hb(nb), hc(nc);
-    fill(ha, 1, gemm ? 1.0 : 1.0 / (double)an, 0.0);
-    fill(hb, 2, 1.0, 0.0);
-    fill(hc, 3, 1.0, 0.0);
-    if (!gemm)  // well-conditioned triangle: diagonal in [1,2)
-        for (size_t i = 0; i < an; ++i) ha[o.offA + i * lda + i] = (T)(1.0 + std::fabs((double)ha[o.offA + i * lda + i]) * (double)an);
+    // shapes of A, B, C as the routine sees them
+    size_t ar = m, ac = k, br = k, bc = n, cr = m, cc = n;
+    int ta = o.transA, tb = o.transB;
+    if (tri || fn == FN_SYMM) { ar = ac = an; ta = 0; br = m; bc = n; tb = 0; }
+    if (fn == FN_SYRK) { ar = n; ac = k; cr = cc = n; }
+    const size_t lda = o.lda ? o.lda : tight(ta, ar, ac);
+    const size_t ldb = o.ldb ? o.ldb : tight(tb, br, bc);
+    const size_t ldc = o.ldc ? o.ldc : tight(0, cr, cc);
+    const size_t na = footprint(o.order, ta, ar, ac, o.offA, lda);
+    const size_t nb = fn == FN_SYRK ? 1 : footprint(o.order, tb, br, bc, o.offBX, ldb);
+    const size_t nc = (tri) ? 1 : footprint(o.order, 0, cr, cc, o.offCY, ldc);
+    std::vector<R> ha(na * NC), hb(nb * NC), hc(nc * NC);
+    fill(ha, 1, tri ? 1.0 / (double)an : 1.0);
+    fill(hb, 2, 1.0);
+    fill(hc, 3, 1.0);
+    if (tri)  // well-conditioned triangle: diagonal in [1,2)
+        for (size_t i = 0; i < an; ++i) {
+            R &d = ha[(o.offA + i * lda + i) * NC];
+            d = (R)(1.0 + std::fabs((double)d) * (double)an);
+        }
     T *da, *db, *dc;
     HIP_OK(hipMalloc((void **)&da, na * sizeof(T)));
     HIP_OK(hipMalloc((void **)&db, nb * sizeof(T)));
@@ -133,23 +198,20 @@ template <typename T> double run_case(const Options &o, size_t m, size_t n, size
     HIP_OK(hipEventCreate(&e0));
     HIP_OK(hipEventCreate(&e1));
 
+    const T alpha = Type<T>::scalar(o.alpha), beta = Type<T>::scalar(o.beta);
+    const clblasOrder ord = (clblasOrder)o.order;
+    const clblasTranspose tA = (clblasTranspose)o.transA, tB = (clblasTranspose)o.transB;
+    const clblasSide side = (clblasSide)o.side;
+    const clblasUplo uplo = (clblasUplo)o.uplo;
+    const clblasDiag diag = (clblasDiag)o.diag;
     auto call = [&]() -> clblasStatus {
-        if (gemm) {
-            if (sizeof(T) == 4)
-                return clblasSgemm((clblasOrder)o.order, (clblasTranspose)o.transA, (clblasTranspose)o.transB, m, n, k,
-                                   (float)o.alpha, (const float *)da, o.offA, lda, (const float *)db, o.offBX, ldb,
-                                   (float)o.beta, (float *)dc, o.offCY, ldc, stream);
-            return clblasDgemm((clblasOrder)o.order, (clblasTranspose)o.transA, (clblasTranspose)o.transB, m, n, k,
-                               o.alpha, (const double *)da, o.offA, lda, (const double *)db, o.offBX, ldb, o.beta,
-                               (double *)dc, o.offCY, ldc, stream);
+        switch (fn) {
+        case FN_GEMM: return gemm(ord, tA, tB, m, n, k, alpha, da, o.offA, lda, db, o.offBX, ldb, beta, dc, o.offCY, ldc, stream);
+        case FN_TRSM: return trsm(ord, side, uplo, tA, diag, m, n, alpha, (const T *)da, o.offA, lda, db, o.offBX, ldb, stream);
+        case FN_TRMM: return trmm(ord, side, uplo, tA, diag, m, n, alpha, da, o.offA, lda, db, o.offBX, ldb, stream);
+        case FN_SYRK: return syrk(ord, uplo, tA, n, k, alpha, da, o.offA, lda, beta, dc, o.offCY, ldc, stream);
+        default: return symm(ord, side, uplo, m, n, alpha, da, o.offA, lda, db, o.offBX, ldb, beta, dc, o.offCY, ldc, stream);
         }
-        if (sizeof(T) == 4)
-            return clblasStrsm((clblasOrder)o.order, (clblasSide)o.side, (clblasUplo)o.uplo, (clblasTranspose)o.transA,
-                               (clblasDiag)o.diag, m, n, (float)o.alpha, (const float *)da, o.offA, lda, (float *)db,
-                               o.offBX, ldb, stream);
-        return clblasDtrsm((clblasOrder)o.order, (clblasSide)o.side, (clblasUplo)o.uplo, (clblasTranspose)o.transA,
-                           (clblasDiag)o.diag, m, n, o.alpha, (const double *)da, o.offA, lda, (double *)db, o.offBX,
-                           ldb, stream);
     };
 
     ok = true;
@@ -158,7 +220,7 @@ template <typename T> double run_case(const Options &o, size_t m, size_t n, size
     HIP_OK(hipStreamSynchronize(stream));
     std::vector<double> samples;
     for (unsigned p = 0; ok && p < std::max(1u, o.profile); ++p) {
-        if (!gemm) HIP_OK(hipMemcpyAsync(db, hb.data(), nb * sizeof(T), hipMemcpyHostToDevice, stream));  // fresh right-hand sides
+        if (tri) HIP_OK(hipMemcpyAsync(db, hb.data(), nb * sizeof(T), hipMemcpyHostToDevice, stream));  // fresh B
         HIP_OK(hipEventRecord(e0, stream));
         for (unsigned c = 0; c < std::max(1u, o.apiCallCount); ++c) call();
         HIP_OK(hipEventRecord(e1, stream));
@@ -171,7 +233,17 @@ template <typename T> double run_case(const Options &o, size_t m, size_t n, size
     if (ok) {
         std::sort(samples.begin(), samples.end());
         const double ns = samples[samples.size() / 2];
-        const double flop = gemm ? 2.0 * m * n * k : (o.side == 0 ? (double)m * (m + 1) * n : (double)m * (n + 1) * n);
+        // flop counts of the reference client: clfunc_xgemm.hpp:95-107,1199-1210, clfunc_xtrsm.hpp:70-92,
+        // clfunc_xtrmm.hpp:85-95,757-784, clfunc_xsyrk.hpp:65-68,588-649, clfunc_xsymm.hpp:63-69,628-645
+        const double cplx = NC == 2 ? 4.0 : 1.0, M = (double)m, N = (double)n, K = (double)k;
+        double flop = 0;
+        switch (fn) {
+        case FN_GEMM: flop = 2.0 * cplx * M * N * K; break;
+        case FN_TRSM:
+        case FN_TRMM: flop = cplx * (o.side == 0 ? M * (M + 1) * N : M * (N + 1) * N); break;
+        case FN_SYRK: flop = cplx * N * (N + 1) * K; break;
+        default: flop = 2.0 * cplx * (o.side == 0 ? M * M * N : N * N * M); break;
+        }
         gflops = flop / ns;
     }
     HIP_OK(hipEventDestroy(e0));
@@ -190,8 +262,13 @@ const char *trans_name(int t) { return t == 0 ? "none" : (t == 1 ? "transpose" :
 int main(int argc, char **argv) {
     Options o;
     if (!parse(argc, argv, o)) { usage(); return 2; }
-    if ((o.function != "gemm" && o.function != "trsm") || (o.precision != "s" && o.precision != "d")) {
-        std::fprintf(stderr, "this library implements -f gemm|trsm with -r s|d\n");
+    const char *fnames[] = {"gemm", "trsm", "trmm", "syrk", "symm"};
+    int fn = -1;
+    for (int i = 0; i < 5; ++i)
+        if (o.function == fnames[i]) fn = i;
+    const bool real = o.precision == "s" || o.precision == "d", cplx = o.precision == "c" || o.precision == "z";
+    if (fn < 0 || !(real || cplx) || (fn == FN_TRSM && !real)) {
+        std::fprintf(stderr, "this library implements -f gemm|trmm|syrk|symm with -r s|d|c|z and -f trsm with -r s|d\n");
         return 2;
     }
     if (clblasSetup() != clblasSuccess) { std::fprintf(stderr, "clblasSetup failed (needs a gfx950 device)\n"); return 1; }
@@ -209,7 +286,11 @@ int main(int argc, char **argv) {
     for (size_t i = 0; i < count; ++i) {
         const size_t m = sizes.empty() ? o.m : sizes[i], n = sizes.empty() ? o.n : sizes[i], k = sizes.empty() ? o.k : sizes[i];
         bool ok = true;
-        const double g = o.precision == "s" ? run_case<float>(o, m, n, k, ok) : run_case<double>(o, m, n, k, ok);
+        double g;
+        if (o.precision == "s") g = run_case<float>(o, (Fn)fn, m, n, k, ok);
+        else if (o.precision == "d") g = run_case<double>(o, (Fn)fn, m, n, k, ok);
+        else if (o.precision == "c") g = run_case<FloatComplex>(o, (Fn)fn, m, n, k, ok);
+        else g = run_case<DoubleComplex>(o, (Fn)fn, m, n, k, ok);
         if (!ok) { rc = 1; continue; }
         std::printf("%zu,%zu,%zu,%zu,%zu,%zu,%zu,%zu,%zu,%g,%g,%s,%s,%s,%s,%s,%s,%s%s,gpu,clblas_amd,1,%s,%g\n", m, n, k,
                     o.lda, o.ldb, o.ldc, o.offA, o.offBX, o.offCY, o.alpha, o.beta, o.order ? "column" : "row",
