@@ -1,14 +1,14 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
 HBM).  Prints ONE JSON line.  `value` is SGEMM TFLOP/s using the reference's own flop
 count 2*M*N*K (src/client/clfunc_xgemm.hpp:95-107); DGEMM (config 4) and DTRSM (config 5,
 M*(M+1)*N flops, src/client/clfunc_xtrsm.hpp:70-92) are reported in `extra`, and so are CGEMM /
-ZGEMM at the same size (8*M*N*K flops, clfunc_xgemm.hpp:95-107).
+ZGEMM at the same size (8*M*N*K flops, clfunc_xgemm.hpp:95-107) and S/D SYRK, TRMM, SYMM.
 `cpu_baseline` times the CPU oracle (a port of the reference arithmetic, OpenMP over the
 host cores) on a bounded sample of the same workload; it is a reported baseline only.
 """
@@ -121,7 +121,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MATRIX,
                          "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MATRIX, 4),
                          "traffic": SGEMM_8192_TRAFFIC_BYTES if n == 8192 else None,
-                         "kernel": "gemm_mfma_kernel<float,256,128,16,...> (one launch per call)",
+                         "kernel": "gemm_mfma_kernel<float,128,128,16,...> (one launch per call)",
                          "launch_ms": round(ev_ms, 4)},
         }
         extra["sgemm_pct_of_fp32_matrix_peak"] = round(100 * tflops / PEAK_FP32_MATRIX, 2)
@@ -197,6 +197,35 @@ def main():
                        "tflops": round(c_tflops, 3), "launch_ms": round(ev_ms, 4),
                        "pct_of_matrix_peak": round(100 * c_tflops / peak, 2)}
         del A, B, C
+
+    # ---- SYRK / TRMM / SYMM at the same size (useful flops only: the reference client's counts) ----
+    if args.only in ("", "level3"):
+        lv = {}
+        for pre, dt, peak in (("S", torch.float32, PEAK_FP32_MATRIX), ("D", torch.float64, PEAK_FP64_MATRIX)):
+            A = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            B0 = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            B = B0.clone()
+            C = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            cases = (
+                ("syrk", float(n) * (n + 1) * n, None,
+                 lambda: clblas_amd.syrk(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, 1.0, C, 0, n)),
+                ("trmm", float(n) * (n + 1) * n, lambda: B.copy_(B0),
+                 lambda: clblas_amd.trmm(pre, COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, A, 0, n, B, 0, n)),
+                ("symm", 2.0 * n * n * n, None,
+                 lambda: clblas_amd.symm(pre, COL, LEFT, LOWER, n, n, 1.0, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+            )
+            for name, fl, before, fn in cases:
+                def call(fn=fn, name=name):
+                    st = fn()
+                    if st != 0:
+                        raise RuntimeError("clblas%s%s returned %d" % (pre, name, st))
+                wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 1, before_each=before)
+                tf = fl / (ev_ms * 1e-3) / 1e12
+                lv[pre.lower() + name] = {"tflops": round(tf, 2), "ms_per_call": round(ev_ms, 4),
+                                          "pct_of_matrix_peak": round(100 * tf / peak, 1)}
+            del A, B, B0, C
+        lv["workload"] = "column-major, lower, left, no transpose, N=M=K=%d, alpha=beta=1" % n
+        extra["level3"] = lv
 
     # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
     cpu = None
