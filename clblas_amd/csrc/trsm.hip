@@ -5,15 +5,15 @@
 // for STRSM, the legacy block solver (src/library/blas/gens/trsm.c:1213-1456).  The
 // reference inverts every 128x128 diagonal block (trtri kernels) and then alternates
 // "X_i = inv(A_ii) B_i" with a trailing DGEMM update, using an M x N temporary.  Here the
-// diagonal blocks (128 x 128) are solved directly by substitution inside one kernel (eight
-// wavefronts, one lane per right-hand side, the block's triangle broadcast from LDS), the
-// sweep is recursive so that almost all flops land in large-K GEMM updates, and B is solved
-// in place without a temporary.
+// diagonal blocks (256 x 256) are solved inside one kernel by block substitution over their
+// 16 x 16 sub-blocks on the MFMA units (only the 16 x 16 diagonal sub-triangles are inverted,
+// by substitution, in a packing pass), the sweep is recursive so that almost all flops land
+// in large-K GEMM updates, and B is solved in place without a temporary.
 // The block sweep directions are those of xtrsm.cc:1226-1477; alpha is applied exactly once
 // to every element of B (xtrsm.cc:1236-1240).
 //
-// A zero on a non-unit diagonal gives Inf/NaN (1/0), as in the textbook algorithm; the
-// reference's inversion kernel substitutes 1 instead (trtri/diag_dtrtri_lower_128_16.cpp:93-96).
+// A zero on a non-unit diagonal gives Inf/NaN (1/0); the reference's inversion kernel
+// substitutes 1 instead (trtri/diag_dtrtri_lower_128_16.cpp:93-96).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -21,122 +21,188 @@
 
 namespace cba {
 
-// Solves one diagonal block (up to 128 x 128) against 64 right-hand sides per workgroup.
-//
-// The block is the nb x nb (nb <= NB) triangle at A(i0,i0).  "Equation order" P = 0..nb-1
-// walks the block forward (index P) or backward (index nb-1-P) so that equation P only
-// involves unknowns Q < P.  coef(P,Q) is the factor of unknown Q in equation P:
-//   left :  op(A)(iP, iQ)        right:  op(A)(iQ, iP)
-// so with teff = trans XOR right it is A[iP + iQ*lda] (teff false) or A[iQ + iP*lda].
-// Right-hand side j is a column of B for side=left (element r at B[r + j*ldb]) and a row
-// of B for side=right (element r at B[j + r*ldb]).
-//
-// Work split: 8 wavefronts, wavefront w owns equations [16w, 16w+16) and keeps them in
-// registers, one lane per right-hand side.  Step s: wavefront s finishes its 16 unknowns
-// by substitution (each new unknown is folded into the remaining equations at once, so
-// the FMAs of one step are independent) and publishes them through LDS; after the
-// barrier every later wavefront subtracts the 16 x 16 coupling block times those unknowns.
-// The triangle sits in LDS as 36 blocks of 16 x 16, read as wave-uniform broadcasts one
-// column ahead of the FMAs that use them.
-// Only the referenced triangle of A is read (never the other one, nor a unit diagonal).
-// For side=left a right-hand side is a column of B, so giving each lane "its" column
-// directly would make every load touch 64 different columns; the panel is instead moved
-// between HBM and registers through an LDS staging area with lanes running along the
-// contiguous direction (the area reuses the triangle's LDS before and after the solve).
-template <typename T> struct TrsmLeaf {
-    static constexpr int NB = 128, IB = 16, NBLK = NB / IB, CW = 64, THREADS = 64 * NBLK;
-    static constexpr int EP = IB + 16 / (int)sizeof(T);   // column pitch of an E block: columns stay 16-byte aligned
-    static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;  // blocks (bi,bj), bi >= bj, at bi*(bi+1)/2 + bj
-    static constexpr int E_ELEMS = N_EBLK * IB * EP;
-    static constexpr int X_ELEMS = 2 * IB * CW;
-    static constexpr int SP = NB + 2;                     // pitch of the right-hand-side staging area
-    static constexpr int S_ELEMS = CW * SP;               // shares LDS with E (used before and after it)
-    static_assert(S_ELEMS <= E_ELEMS + X_ELEMS, "staging area must fit in the E/X region");
-    static constexpr size_t SMEM = (size_t)(E_ELEMS + X_ELEMS + NB) * sizeof(T);
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef double f64x4_t __attribute__((ext_vector_type(4)));
+
+// 16 x 16 x 4 MFMA: D[i][j] += sum_k A[i][k] B[k][j]; lane l supplies A[l%16][l/16] and
+// B[l/16][l%16] and holds D[krow(l/16, v)][l%16] in accumulator element v (layouts checked
+// on the device).
+template <typename T> struct Mma16;
+template <> struct Mma16<double> {
+    typedef f64x4_t Acc;
+    static __device__ __forceinline__ Acc run(double a, double b, Acc c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    static __host__ __device__ __forceinline__ int krow(int g, int v) { return g + 4 * v; }
+};
+template <> struct Mma16<float> {
+    typedef f32x4_t Acc;
+    static __device__ __forceinline__ Acc run(float a, float b, Acc c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+    }
+    static __host__ __device__ __forceinline__ int krow(int g, int v) { return 4 * g + v; }
 };
 
-// IB values of one E-block column (16-byte LDS reads; the address is wave-uniform).
-template <typename T, int IB> static __device__ __forceinline__ void load_e_column(const T *src, T (&dst)[IB]) {
-    constexpr int V = 16 / (int)sizeof(T);
-    typedef T VT __attribute__((ext_vector_type(V)));
+// Diagonal blocks (up to 256 x 256) are solved in 16 x 16 sub-blocks on the MFMA units.
+//
+// "Equation order" P = 0..nb-1 walks a diagonal block forward (index P) or backward (index
+// nb-1-P) so that equation P only involves unknowns Q <= P.  coef(P,Q) is the factor of
+// unknown Q in equation P:   left: op(A)(iP, iQ)   right: op(A)(iQ, iP),
+// so with teff = trans XOR right it is A[iP + iQ*lda] (teff false) or A[iQ + iP*lda].
+// In that order every diagonal block is lower triangular, L = (L_ws), 16 x 16 sub-blocks of
+// 16 x 16, and the solve is the block substitution
+//     X_s = inv(L_ss) Y_s ;   Y_w -= L_ws X_s  (w > s)        s = 0..15.
+// A packing pass (trsm_pack_kernel, once per call, all diagonal blocks at once) reads the
+// referenced triangle of A - never the other one, nor a unit diagonal - inverts the sixteen
+// small triangles L_ss by substitution and writes, per diagonal block, the 136 sub-blocks
+// inv(L_ss) and -L_ws in the order the MFMA "A" operand wants them: entry [lane][c] is
+// element (p = lane%16, q = krow(lane/16, c)), so a lane fetches its four values of a
+// sub-block with one or two 16-byte loads and nothing is broadcast.  Row w's sub-blocks
+// (w,0..w) are consecutive, so each wavefront streams its own row straight from memory
+// (L2), two steps ahead of their use.
+// (The reference inverts whole 128 x 128 blocks, trtri/*.cpp; inverting only the 16 x 16
+// ones keeps the result much closer to plain substitution.)
+//
+// Leaf kernel: one workgroup = one diagonal block x CW = 32 right-hand sides, 16 wavefronts;
+// wavefront w owns equations [16w, 16w+16) as two 16 x 16 accumulator blocks (lane l:
+// right-hand side l%16 of each block, equations krow(l/16, v)).  Accumulator layout and
+// MFMA "B" operand layout coincide, so Y_s feeds the MFMAs as it is and X_s goes to the
+// other wavefronts through LDS in the same per-lane order.  Step s: wavefront s computes
+// X_s (8 MFMAs), publishes it, barrier, wavefronts w > s subtract L_ws X_s (8 MFMAs each).
+// For side=left a right-hand side is a column of B; the panel moves between HBM and the
+// accumulator layout through an LDS staging area so that global accesses run along columns.
+template <typename T> struct TrsmLeaf {
+    static constexpr int NB = 256, IB = 16, NBLK = NB / IB, CW = 32, NBK = CW / 16, THREADS = 64 * NBLK;
+    static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;  // sub-blocks (bi,bj), bi >= bj, at bi*(bi+1)/2 + bj
+    static constexpr int PACK_ELEMS = N_EBLK * IB * IB;   // per diagonal block
+    static constexpr int X_ELEMS = 2 * NBK * 64 * 4;      // two buffers of X_s in per-lane order
+    static constexpr int SP = NB + 2;                     // pitch of the right-hand-side staging area
+    static constexpr int S_ELEMS = CW * SP;
+    static constexpr size_t SMEM = (size_t)(X_ELEMS + S_ELEMS) * sizeof(T);
+};
+
+// Packs all diagonal blocks of the n x n triangle (see above).  Workgroup (bi, b) of 256
+// threads packs sub-block row bi of diagonal block b (rows/columns [256 b, 256 b + nb)).
+template <typename T, bool FORWARD>
+__global__ void __launch_bounds__(256)
+trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool unit, T *__restrict__ pack) {
+    typedef TrsmLeaf<T> L;
+    typedef Mma16<T> M;
+    constexpr int IB = L::IB;
+    __shared__ T Ld[IB][IB + 1];  // the diagonal sub-triangle, then its inverse
+    const int tid = threadIdx.x;
+    const int bi = blockIdx.x;
+    const int i0 = blockIdx.y * L::NB;
+    const int nb = n - i0 < L::NB ? n - i0 : L::NB;
+    const T *Ablk = A + i0 + (int64_t)i0 * lda;
+    T *out = pack + (int64_t)blockIdx.y * L::PACK_ELEMS + (int64_t)(bi * (bi + 1) / 2) * (IB * IB);
+    auto coef = [&](int P, int Q) -> T {  // Q < P < nb
+        const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
+        return teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
+    };
+    // off-diagonal sub-blocks (bi, 0..bi-1), negated; rows past nb are zero
+    for (int e = tid; e < bi * IB * IB; e += 256) {
+        const int bj = e / (IB * IB), w = e % (IB * IB);
+        const int lane = w / 4, c = w % 4;
+        const int P = bi * IB + lane % 16, Q = bj * IB + M::krow(lane / 16, c);
+        out[e] = (P < nb) ? -coef(P, Q) : (T)0;  // Q < P always holds here; Q < nb follows from P < nb
+    }
+    // diagonal sub-triangle into LDS (identity where the block is short)
+    {
+        const int p = tid / IB, q = tid % IB;
+        const int P = bi * IB + p, Q = bi * IB + q;
+        T v = (T)0;
+        if (p == q) {
+            v = (T)1;
+            if (!unit && P < nb) {
+                const int ip = FORWARD ? P : nb - 1 - P;
+                v = Ablk[ip + (int64_t)ip * lda];
+            }
+        } else if (q < p && P < nb) {
+            v = coef(P, Q);
+        }
+        Ld[p][q] = v;
+    }
+    __syncthreads();
+    // invert: thread zc < 16 solves L z = e_zc by substitution
+    T z[IB];
+    const int zc = tid;
+    if (tid < IB) {
 #pragma unroll
-    for (int p = 0; p < IB; p += V) {
-        VT v = *reinterpret_cast<const VT *>(src + p);
+        for (int p = 0; p < IB; ++p) {
+            T acc = (p == zc) ? (T)1 : (T)0;
 #pragma unroll
-        for (int e = 0; e < V; ++e) dst[p + e] = v[e];
+            for (int q = 0; q < IB; ++q)
+                if (q < p) acc -= Ld[p][q] * z[q];
+            z[p] = (p < zc) ? (T)0 : acc / Ld[p][p];
+        }
+    }
+    __syncthreads();
+    if (tid < IB) {
+#pragma unroll
+        for (int p = 0; p < IB; ++p) Ld[p][zc] = z[p];
+    }
+    __syncthreads();
+    {
+        const int lane = tid / 4, c = tid % 4;
+        out[bi * (IB * IB) + tid] = Ld[lane % 16][M::krow(lane / 16, c)];
     }
 }
 
 template <typename T, bool RIGHT, bool FORWARD>
 __global__ void __launch_bounds__(TrsmLeaf<T>::THREADS)
-trsm_diag_kernel(const T *__restrict__ Ablk, int64_t lda, bool teff, bool unit, int nb, T alpha,
-                 T *__restrict__ Bblk, int64_t ldb, int nrhs) {
+trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk, int64_t ldb, int nrhs) {
     typedef TrsmLeaf<T> L;
-    constexpr int IB = L::IB, CW = L::CW, EP = L::EP, NT = L::THREADS;
+    typedef Mma16<T> M;
+    typedef typename M::Acc Acc;
+    constexpr int IB = L::IB, CW = L::CW, NBK = L::NBK, NT = L::THREADS, NBLK = L::NBLK;
+    constexpr int V = 16 / (int)sizeof(T);  // elements per 16 bytes
+    typedef T VT __attribute__((ext_vector_type(V)));
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    T *E = reinterpret_cast<T *>(smem_raw);
-    T *X = E + L::E_ELEMS;
-    T *Dinv = X + L::X_ELEMS;
+    T *X = reinterpret_cast<T *>(smem_raw);
+    T *S = X + L::X_ELEMS;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
-
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, jj = lane & 15;
     const int64_t j0 = (int64_t)blockIdx.x * CW;
-    const int64_t j = j0 + lane;
-    const bool col_ok = j < nrhs;
-    T y[IB];
+    const int nsteps = (nb + IB - 1) / IB;  // sub-block rows that exist
 
-    // ---- triangle: issue its loads first so that they overlap the right-hand-side traffic.
-    //      Element e of the (block, q, p) enumeration; only the referenced triangle is read. ----
-    constexpr int E_ITERS = L::N_EBLK * IB * IB / NT;
-    static_assert(L::N_EBLK * IB * IB % NT == 0, "triangle fill must divide over the workgroup");
-    auto e_coords = [&](int u, int &blk, int &p, int &q) {
-        const int e = tid + u * NT;
-        blk = e / (IB * IB);
-        const int w = e % (IB * IB);
-        // Let the index that is contiguous in memory vary fastest across lanes.
-        if (teff) { q = w % IB; p = w / IB; } else { p = w % IB; q = w / IB; }
-    };
-    auto e_slot = [&](int u) {
-        int blk, p, q;
-        e_coords(u, blk, p, q);
-        return blk * (IB * EP) + q * EP + p;
-    };
-    T eval[E_ITERS];
+    // A lane's four values of sub-block (wave, s): MFMA "A" operand, chunk c = element c.
+    const T *erow = packed + (int64_t)(wave * (wave + 1) / 2) * (IB * IB) + lane * 4;
+    auto load_e = [&](int s, T (&a)[4]) {
+        const T *src = erow + s * (IB * IB);
 #pragma unroll
-    for (int u = 0; u < E_ITERS; ++u) {
-        int blk, p, q;
-        e_coords(u, blk, p, q);
-        int bi = 0;
-        while ((bi + 1) * (bi + 2) / 2 <= blk) ++bi;
-        const int bj = blk - bi * (bi + 1) / 2;
-        const int P = bi * IB + p, Q = bj * IB + q;
-        eval[u] = (T)0;
-        if (Q < P && P < nb) {
-            const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
-            eval[u] = teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
+        for (int c = 0; c < 4; c += V) {
+            VT t = *reinterpret_cast<const VT *>(src + c);
+#pragma unroll
+            for (int e = 0; e < V && c + e < 4; ++e) a[c + e] = t[e];
         }
-    }
-    T dval = (T)1;
-    if (tid < L::NB && !unit && tid < nb) {
-        const int ip = FORWARD ? tid : nb - 1 - tid;
-        dval = Ablk[ip + (int64_t)ip * lda];
-    }
+    };
+    constexpr int RING = 3;  // sub-blocks in flight: this step's and the next two
+    T ea[RING][4];
+#pragma unroll
+    for (int s = 0; s < RING - 1; ++s)
+        if (s <= wave && wave < nsteps) load_e(s, ea[s]);
 
-    // ---- this wavefront's 16 equations of right-hand side j into registers ----
+    // ---- right-hand sides into the accumulator layout: y[k][v] = alpha * b(equation krow(g,v) of
+    //      this wavefront, right-hand side j0 + 16k + jj) ----
+    Acc y[NBK];
+    auto mem_row = [&](int P) { return FORWARD ? P : nb - 1 - P; };
     if (RIGHT) {
 #pragma unroll
-        for (int p = 0; p < IB; ++p) {
-            const int P = wave * IB + p;
-            const int r = FORWARD ? P : nb - 1 - P;
-            T v = (T)0;
-            if (P < nb && col_ok) v = Bblk[j + (int64_t)r * ldb];
-            y[p] = alpha * v;
+        for (int k = 0; k < NBK; ++k) {
+            const int64_t j = j0 + 16 * k + jj;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int P = wave * IB + M::krow(g, v);
+                T b = (T)0;
+                if (P < nb && j < nrhs) b = Bblk[j + (int64_t)mem_row(P) * ldb];
+                y[k][v] = alpha * b;
+            }
         }
     } else {
-        T *S = E;  // staging area, overwritten by the triangle afterwards
-        // All loads are issued before the first LDS write so that their latencies overlap.
         constexpr int NLD = CW * (L::NB / 2) / NT;
         T v0[NLD], v1[NLD];
 #pragma unroll
@@ -160,93 +226,65 @@ trsm_diag_kernel(const T *__restrict__ Ablk, int64_t lda, bool teff, bool unit, 
         }
         __syncthreads();
 #pragma unroll
-        for (int p = 0; p < IB; ++p) {
-            const int P = wave * IB + p;
-            const int r = FORWARD ? P : (nb - 1 - P < 0 ? 0 : nb - 1 - P);
-            y[p] = (P < nb) ? alpha * S[lane * L::SP + r] : (T)0;
-        }
-        __syncthreads();
+        for (int k = 0; k < NBK; ++k)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int P = wave * IB + M::krow(g, v);
+                y[k][v] = (P < nb) ? alpha * S[(16 * k + jj) * L::SP + mem_row(P)] : (T)0;
+            }
     }
 
-    // ---- triangle into LDS (its loads were issued first, see above) ----
 #pragma unroll
-    for (int u = 0; u < E_ITERS; ++u) E[e_slot(u)] = eval[u];
-    if (tid < L::NB) Dinv[tid] = (T)1 / dval;
-    __syncthreads();
-
-#pragma unroll 1
-    for (int s = 0; s < L::NBLK; ++s) {
-        T *Xs = X + (s & 1) * (IB * CW);
-        if (wave == s) {
-            const T *Ed = E + (s * (s + 1) / 2 + s) * (IB * EP);
-            T dinv[IB];
-            load_e_column<T, IB>(Dinv + s * IB, dinv);
-            T ea[IB], eb[IB];
-            load_e_column<T, IB>(Ed, ea);
+    for (int s = 0; s < NBLK; ++s) {
+        if (s < nsteps) {  // uniform over the workgroup
+            T *Xs = X + (s & 1) * (NBK * 64 * 4);
+            if (s + RING - 1 <= wave && wave < nsteps) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
+            if (wave == s) {
+                Acc x[NBK];
 #pragma unroll
-            for (int q = 0; q < IB; q += 2) {
-                load_e_column<T, IB>(Ed + (q + 1) * EP, eb);
-                __builtin_amdgcn_sched_barrier(0);
-                {
-                    const T x = y[q] * dinv[q];
-                    y[q] = x;
-                    Xs[q * CW + lane] = x;
+                for (int k = 0; k < NBK; ++k) x[k] = Acc{0, 0, 0, 0};
 #pragma unroll
-                    for (int p = q + 1; p < IB; ++p) y[p] = fma(-ea[p], x, y[p]);
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int k = 0; k < NBK; ++k) x[k] = M::run(ea[s % RING][c], y[k][c], x[k]);
+#pragma unroll
+                for (int k = 0; k < NBK; ++k) {
+                    y[k] = x[k];
+                    *reinterpret_cast<Acc *>(Xs + (k * 64 + lane) * 4) = x[k];
                 }
-                __builtin_amdgcn_sched_barrier(0);
-                if (q + 2 < IB) load_e_column<T, IB>(Ed + (q + 2) * EP, ea);
-                __builtin_amdgcn_sched_barrier(0);
-                {
-                    const T x = y[q + 1] * dinv[q + 1];
-                    y[q + 1] = x;
-                    Xs[(q + 1) * CW + lane] = x;
-#pragma unroll
-                    for (int p = q + 2; p < IB; ++p) y[p] = fma(-eb[p], x, y[p]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
             }
-        }
-        __syncthreads();
-        if (wave > s && wave * IB < nb) {
-            const T *Eo = E + (wave * (wave + 1) / 2 + s) * (IB * EP);
-            T xs[IB];
+            __syncthreads();
+            if (wave > s && wave < nsteps) {
+                Acc xb[NBK];
 #pragma unroll
-            for (int q = 0; q < IB; ++q) xs[q] = Xs[q * CW + lane];
-            T ea[IB], eb[IB];
-            load_e_column<T, IB>(Eo, ea);
+                for (int k = 0; k < NBK; ++k) xb[k] = *reinterpret_cast<const Acc *>(Xs + (k * 64 + lane) * 4);
 #pragma unroll
-            for (int q = 0; q < IB; q += 2) {
-                load_e_column<T, IB>(Eo + (q + 1) * EP, eb);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int c = 0; c < 4; ++c)
 #pragma unroll
-                for (int p = 0; p < IB; ++p) y[p] = fma(-ea[p], xs[q], y[p]);
-                __builtin_amdgcn_sched_barrier(0);
-                if (q + 2 < IB) load_e_column<T, IB>(Eo + (q + 2) * EP, ea);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int p = 0; p < IB; ++p) y[p] = fma(-eb[p], xs[q + 1], y[p]);
-                __builtin_amdgcn_sched_barrier(0);
+                    for (int k = 0; k < NBK; ++k) y[k] = M::run(ea[s % RING][c], xb[k][c], y[k]);
             }
         }
     }
 
     if (RIGHT) {
 #pragma unroll
-        for (int p = 0; p < IB; ++p) {
-            const int P = wave * IB + p;
-            const int r = FORWARD ? P : nb - 1 - P;
-            if (P < nb && col_ok) Bblk[j + (int64_t)r * ldb] = y[p];
+        for (int k = 0; k < NBK; ++k) {
+            const int64_t j = j0 + 16 * k + jj;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int P = wave * IB + M::krow(g, v);
+                if (P < nb && j < nrhs) Bblk[j + (int64_t)mem_row(P) * ldb] = y[k][v];
+            }
         }
     } else {
-        T *S = E;
-        __syncthreads();  // every wavefront is done with the triangle
+        // The staging area was last read before the first step's barrier.
 #pragma unroll
-        for (int p = 0; p < IB; ++p) {
-            const int P = wave * IB + p;
-            const int r = FORWARD ? P : (nb - 1 - P < 0 ? 0 : nb - 1 - P);
-            if (P < nb) S[lane * L::SP + r] = y[p];
-        }
+        for (int k = 0; k < NBK; ++k)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int P = wave * IB + M::krow(g, v);
+                if (P < nb) S[(16 * k + jj) * L::SP + mem_row(P)] = y[k][v];
+            }
         __syncthreads();
         constexpr int NLD = CW * (L::NB / 2) / NT;
 #pragma unroll
@@ -285,13 +323,29 @@ template <typename T> struct TrsmDriver {
     T *B;
     int64_t ldb;
     hipStream_t stream;
+    const T *pack;  // packed diagonal blocks, TrsmLeaf<T>::PACK_ELEMS each
+
+    // Packs every diagonal block of the triangle (one launch per call).
+    hipError_t prepare() {
+        typedef TrsmLeaf<T> L;
+        const int n = right ? N : M;
+        const int nblk = (n + NBL - 1) / NBL;
+        T *w = (T *)workspace_get(stream, (size_t)nblk * L::PACK_ELEMS * sizeof(T), 2);
+        if (!w) return hipErrorOutOfMemory;
+        pack = w;
+        if (forward)
+            hipLaunchKernelGGL((trsm_pack_kernel<T, true>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff, unit, w);
+        else
+            hipLaunchKernelGGL((trsm_pack_kernel<T, false>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff, unit, w);
+        return hipGetLastError();
+    }
 
     hipError_t leaf(int i0, int nb, T alpha) {
-        const T *Ablk = A + i0 + (int64_t)i0 * lda;
         const int nrhs = right ? M : N;
         T *Bblk = right ? B + (int64_t)i0 * ldb : B + i0;
         typedef TrsmLeaf<T> L;
-        void (*fn)(const T *, int64_t, bool, bool, int, T, T *, int64_t, int);
+        const T *packed = pack + (int64_t)(i0 / NBL) * L::PACK_ELEMS;
+        void (*fn)(const T *, int, T, T *, int64_t, int);
         if (right) fn = forward ? trsm_diag_kernel<T, true, true> : trsm_diag_kernel<T, true, false>;
         else fn = forward ? trsm_diag_kernel<T, false, true> : trsm_diag_kernel<T, false, false>;
         if (L::SMEM > 64 * 1024) {
@@ -299,7 +353,7 @@ template <typename T> struct TrsmDriver {
             if (e != hipSuccess) return e;
         }
         dim3 grid((unsigned)((nrhs + L::CW - 1) / L::CW)), block(L::THREADS);
-        hipLaunchKernelGGL(fn, grid, block, L::SMEM, stream, Ablk, lda, teff, unit, nb, alpha, Bblk, ldb, nrhs);
+        hipLaunchKernelGGL(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs);
         return hipGetLastError();
     }
 
@@ -346,6 +400,8 @@ static hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool unit, i
     d.forward = right ? (lower == trans) : (lower != trans);
     d.teff = trans != right;
     d.M = M; d.N = N; d.A = A; d.lda = lda; d.B = B; d.ldb = ldb; d.stream = stream;
+    hipError_t e = d.prepare();
+    if (e != hipSuccess) return e;
     return d.solve(0, right ? N : M, alpha);
 }
 
