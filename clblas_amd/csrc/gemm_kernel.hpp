@@ -192,7 +192,67 @@ template <typename T> struct GemmParams {
     //          skipped.
     //   rev_m / rev_n: walk the tile rows / columns from the far end (longest tiles first).
     int tri_c, tri_a, tri_b, unit_a, unit_b, rev_m, rev_n;
+    // Sliced tail (TRI kernels only): the last tiles of the list - those of the final, partly
+    // filled round of 256 CUs - are each cut into `tail_slices` K ranges of `tail_kps`, so that
+    // the round lasts 1/tail_slices as long.  Workgroup ids from `tail_first` on are slices
+    // (tile tail_first + u / tail_slices, slice u % tail_slices); slice u stores its partial
+    // tile to ws + u * BM * BN (tile-local, pitch BM) and tail_reduce_kernel finishes C.
+    int tail_first, tail_slices, tail_kps;
 };
+
+// Tile row / column of entry `tile` of the tile list (bm x bn tiles).  Full grid: groups of
+// `group_m` tile rows, column by column inside a group, so that concurrently running
+// workgroups of one XCD share A and B panels in that XCD's L2.  With tri_c only the tiles that
+// touch the stored triangle exist: row r holds the columns [0, last] (lower) or
+// [first, tiles_n) (upper); they are walked the same way and the walk is replayed here until
+// `tile` is reached.
+template <typename T>
+static __device__ __forceinline__ void tile_coords(const GemmParams<T> &p, bool tri, int bm, int bn, int tile, int &tm,
+                                                   int &tn) {
+    if (tri && p.tri_c) {
+        tm = 0;
+        tn = 0;
+        bool found = false;
+        for (int r0 = 0; r0 < p.tiles_m && !found; r0 += p.group_m) {
+            const int r1 = r0 + p.group_m < p.tiles_m ? r0 + p.group_m : p.tiles_m;
+            int in_group = 0;
+            for (int r = r0; r < r1; ++r) {
+                if (p.tri_c == 1) {
+                    const int last = (r * bm + bm - 1) / bn;
+                    in_group += last + 1 < p.tiles_n ? last + 1 : p.tiles_n;
+                } else {
+                    const int first = (r * bm) / bn;
+                    in_group += first < p.tiles_n ? p.tiles_n - first : 0;
+                }
+            }
+            if (tile >= in_group) { tile -= in_group; continue; }
+            for (int c = 0; c < p.tiles_n; ++c) {
+                int lo = r0, hi = r1;  // rows [lo, hi) of the group hold column c
+                if (p.tri_c == 1) {
+                    const int need = c * bn - bm + 1;  // first row index that reaches column c
+                    const int rmin = need <= 0 ? 0 : (need + bm - 1) / bm;
+                    lo = rmin > r0 ? rmin : r0;
+                } else {
+                    const int rmax = (c * bn + bn - 1) / bm;
+                    hi = rmax + 1 < r1 ? rmax + 1 : r1;
+                }
+                const int cnt = hi > lo ? hi - lo : 0;
+                if (tile < cnt) { tm = lo + tile; tn = c; found = true; break; }
+                tile -= cnt;
+            }
+        }
+    } else {
+        const int per_group = p.group_m * p.tiles_n;
+        const int grp = tile / per_group;
+        const int first_m = grp * p.group_m;
+        const int gm = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
+        const int r = tile - grp * per_group;
+        tm = first_m + r % gm;
+        tn = r / gm;
+        if (tri && p.rev_m) tm = p.tiles_m - 1 - tm;
+        if (tri && p.rev_n) tn = p.tiles_n - 1 - tn;
+    }
+}
 
 static __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, int64_t bytes_left) {
     // Descriptors address at most 2 GiB from their base; tiles are re-based so that every
@@ -393,65 +453,26 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         else return __builtin_bit_cast(R, __builtin_bit_cast(uint64_t, x) ^ ((uint64_t)m << 32));
     };
 
-    // ---- tile assignment: contiguous chunk of the tile list per XCD, then walk
-    //      `group_m` tile rows at a time so that concurrently running workgroups of one
-    //      XCD share A and B panels in that XCD's L2. ----
-    int tile;
+    // ---- tile assignment: each XCD takes a contiguous chunk of the tile list (see
+    //      tile_coords for the order of that list); slices of the tail come last and are
+    //      dealt round-robin. ----
+    int tile, slice = -1;
     {
-        const int nwg = gridDim.x;
+        const int sliced = (TRI && p.tail_slices > 1) ? 1 : 0;
+        const int nwg = sliced ? p.tail_first : (int)gridDim.x;  // whole tiles
         const int id = blockIdx.x;
-        const int xcd = id & 7, q = id >> 3;
-        const int per = nwg >> 3, rem = nwg & 7;
-        tile = p.xcd_remap ? xcd * per + (xcd < rem ? xcd : rem) + q : id;
+        if (sliced && id >= nwg) {
+            const int u = id - nwg;
+            tile = nwg + u / p.tail_slices;
+            slice = u % p.tail_slices;
+        } else {
+            const int xcd = id & 7, q = id >> 3;
+            const int per = nwg >> 3, rem = nwg & 7;
+            tile = p.xcd_remap ? xcd * per + (xcd < rem ? xcd : rem) + q : id;
+        }
     }
     int tm, tn;
-    if (TRI && p.tri_c) {
-        // Only tiles that touch the stored triangle exist: row r holds the columns [0, last]
-        // (lower) or [first, tiles_n) (upper).  They are walked like the full grid - groups of
-        // `group_m` rows, column by column inside a group - so that neighbours in the list
-        // share panels; the walk is replayed here until `tile` is reached.
-        tm = 0;
-        tn = 0;
-        bool found = false;
-        for (int r0 = 0; r0 < p.tiles_m && !found; r0 += p.group_m) {
-            const int r1 = r0 + p.group_m < p.tiles_m ? r0 + p.group_m : p.tiles_m;
-            int in_group = 0;
-            for (int r = r0; r < r1; ++r) {
-                if (p.tri_c == 1) {
-                    const int last = (r * BM + BM - 1) / BN;
-                    in_group += last + 1 < p.tiles_n ? last + 1 : p.tiles_n;
-                } else {
-                    const int first = (r * BM) / BN;
-                    in_group += first < p.tiles_n ? p.tiles_n - first : 0;
-                }
-            }
-            if (tile >= in_group) { tile -= in_group; continue; }
-            for (int c = 0; c < p.tiles_n; ++c) {
-                int lo = r0, hi = r1;  // rows [lo, hi) of the group hold column c
-                if (p.tri_c == 1) {
-                    const int need = c * BN - BM + 1;  // first row index that reaches column c
-                    const int rmin = need <= 0 ? 0 : (need + BM - 1) / BM;
-                    lo = rmin > r0 ? rmin : r0;
-                } else {
-                    const int rmax = (c * BN + BN - 1) / BM;
-                    hi = rmax + 1 < r1 ? rmax + 1 : r1;
-                }
-                const int cnt = hi > lo ? hi - lo : 0;
-                if (tile < cnt) { tm = lo + tile; tn = c; found = true; break; }
-                tile -= cnt;
-            }
-        }
-    } else {
-        const int per_group = p.group_m * p.tiles_n;
-        const int grp = tile / per_group;
-        const int first_m = grp * p.group_m;
-        const int gm = (p.tiles_m - first_m) < p.group_m ? (p.tiles_m - first_m) : p.group_m;
-        const int r = tile - grp * per_group;
-        tm = first_m + r % gm;
-        tn = r / gm;
-        if (TRI && p.rev_m) tm = p.tiles_m - 1 - tm;
-        if (TRI && p.rev_n) tn = p.tiles_n - 1 - tn;
-    }
+    tile_coords(p, TRI, BM, BN, tile, tm, tn);
     const int m0 = tm * BM, n0 = tn * BN;
 
     // ---- K range of this workgroup ----
@@ -459,6 +480,10 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     if (SPLITK) {
         k_begin = blockIdx.y * p.k_per_split;
         k_end = k_begin + p.k_per_split < p.K ? k_begin + p.k_per_split : p.K;
+    }
+    if (TRI && slice >= 0) {
+        k_begin = slice * p.tail_kps;
+        k_end = k_begin + p.tail_kps < p.K ? k_begin + p.tail_kps : p.K;
     }
     if (TRI) {
         // Panels that lie wholly in the zero part of a triangular operand are skipped.
@@ -667,6 +692,17 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         alpha = el_one<T>();
         beta = T();
     }
+    int tri_c = TRI ? p.tri_c : 0;
+    if (TRI && slice >= 0) {
+        // partial tile, tile-local coordinates, finished by tail_reduce_kernel
+        const int u = (int)blockIdx.x - p.tail_first;
+        const int64_t shift = (int64_t)u * (BM * BN) - ((int64_t)n0 * BM + m0);  // may be negative
+        Cout = reinterpret_cast<T *>(reinterpret_cast<uintptr_t>(p.ws) + (uintptr_t)(shift * (int64_t)sizeof(T)));
+        ldc = BM;
+        alpha = el_one<T>();
+        beta = T();
+        tri_c = 0;
+    }
     const bool read_c = !el_is_zero(beta);
     const bool neg_im = CPLX && p.conj_b;  // Im = sB * Im'
     auto acc_elem = [&](int bn, int bm, int v) -> T {
@@ -707,9 +743,9 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 for (int ga = 0; ga < TM / VM; ++ga) {
                     const int m = m0 + wm * WM + ga * (MB * VM) + j * VM;
                     bool whole = true;  // all VM rows of this vector are stored
-                    if (TRI && p.tri_c) {
-                        if (p.tri_c == 1 ? m + VM - 1 < n : m > n) continue;  // none of them is
-                        whole = p.tri_c == 1 ? m >= n : m + VM - 1 <= n;
+                    if (TRI && tri_c) {
+                        if (tri_c == 1 ? m + VM - 1 < n : m > n) continue;  // none of them is
+                        whole = tri_c == 1 ? m >= n : m + VM - 1 <= n;
                     }
                     if (m + VM <= p.M && whole) {
                         UV ov;
@@ -723,7 +759,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     } else {
 #pragma unroll
                         for (int e = 0; e < VM; ++e) {
-                            const bool kept = !(TRI && p.tri_c) || (p.tri_c == 1 ? m + e >= n : m + e <= n);
+                            const bool kept = !(TRI && tri_c) || (tri_c == 1 ? m + e >= n : m + e <= n);
                             if (m + e < p.M && kept) {
                                 T r = el_scale(alpha, acc_elem(bn, ga * VM + e, v));
                                 if (read_c) r = el_axpy(beta, col[m + e], r);
@@ -752,6 +788,28 @@ splitk_reduce_kernel(const T *ws, int64_t ws_ld, int64_t ws_slice, int splits, i
     T r = el_scale(alpha, s);
     if (!el_is_zero(beta)) r = el_axpy(beta, *c, r);
     *c = r;
+}
+
+// Finishes the tiles whose K range was cut into slices (see GemmParams::tail_*): sums the
+// slices in a fixed order, applies alpha / beta once and honours tri_c.  Block (x, r) covers
+// elements [256 x, 256 x + 256) of sliced tile r (tile-local, column-major, pitch bm).
+template <typename T>
+__global__ void __launch_bounds__(256) tail_reduce_kernel(const GemmParams<T> p, int bm, int bn) {
+    const int r = blockIdx.y;
+    int tm, tn;
+    tile_coords(p, true, bm, bn, p.tail_first + r, tm, tn);
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= bm * bn) return;
+    const int m = tm * bm + e % bm, n = tn * bn + e / bm;
+    if (m >= p.M || n >= p.N) return;
+    if (p.tri_c && (p.tri_c == 1 ? m < n : m > n)) return;
+    const T *w = p.ws + (int64_t)r * p.tail_slices * (bm * bn) + e;
+    T s = T();
+    for (int i = 0; i < p.tail_slices; ++i) s = el_add(s, w[(int64_t)i * (bm * bn)]);
+    T *c = p.C + (int64_t)n * p.ldc + m;
+    T v = el_scale(p.alpha, s);
+    if (!el_is_zero(p.beta)) v = el_axpy(p.beta, *c, v);
+    *c = v;
 }
 
 // C <- beta * C (K == 0); beta == 0 stores zeros without reading C.

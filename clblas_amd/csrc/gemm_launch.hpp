@@ -89,9 +89,26 @@ static inline int64_t active_tiles(int M, int N, int bm, int bn, int tri_c) {
     return total;
 }
 
+// Sliced tail: with `t` equally long tiles over 256 CUs the last round holds r = t mod 256
+// tiles and leaves the other CUs idle.  Cutting each of those r tiles into s = 256 / r K
+// ranges fills the round and shortens it to 1/s (plus a small reduction pass).  Returns s, or
+// 1 where that does not apply or does not pay: fewer than one full round (split-K covers
+// that case), more than 24 rounds (the tail is a few percent), slices under 8 panels.
+static inline int tail_slices_for(int64_t t, int K, int bk, bool allowed) {
+    const int64_t kCUs = 256;
+    if (!allowed || t <= kCUs || t / kCUs > 24) return 1;
+    const int64_t r = t % kCUs;
+    if (r == 0) return 1;
+    int64_t s = kCUs / r;
+    const int64_t by_k = K / (8 * bk);
+    if (s > by_k) s = by_k;
+    if (s > 16) s = 16;
+    return s < 2 ? 1 : (int)s;
+}
+
 template <typename T>
 static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, bool need_tri, int tri_c,
-                        int *tile_out, int *splits_out) {
+                        bool tail_ok, int *tile_out, int *splits_out) {
     const int64_t kCUs = 256;
     int pick = ntab - 1;  // table is ordered large -> small
     if (force >= 0 && force < ntab && (!need_tri || tab[force].tri[0])) {
@@ -102,7 +119,10 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         for (int i = 0; i < ntab; ++i) {
             if (need_tri && !tab[i].tri[0]) continue;
             const int64_t t = active_tiles(M, N, tab[i].bm, tab[i].bn, tri_c);
-            double cost = (double)ceil_div64(t, kCUs) * tab[i].bm * tab[i].bn / tab[i].eff;
+            double rounds = (double)ceil_div64(t, kCUs);
+            const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
+            if (ts > 1) rounds = (double)(t / kCUs) + 1.0 / ts + 0.05;  // + the reduction pass
+            double cost = rounds * tab[i].bm * tab[i].bn / tab[i].eff;
             if (t <= kCUs) cost /= 0.85;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             if (!have || cost < best) { best = cost; pick = i; have = true; }
         }
@@ -147,7 +167,9 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     }
 
     int tile, splits;
-    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, need_tri ? tri->tri_c : 0, &tile, &splits);
+    // The tail may be sliced unless tiles differ in depth (triangular operands).
+    const bool tail_ok = !(need_tri && (tri->tri_a || tri->tri_b)) && debug_env_int("CLBLAS_AMD_GEMM_TAIL", 1) != 0;
+    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, need_tri ? tri->tri_c : 0, tail_ok, &tile, &splits);
     const TileEntry<T> &e = tab[tile];
 
     GemmParams<T> p;
@@ -179,6 +201,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
     p.k_per_split = K;
     p.tri_c = p.tri_a = p.tri_b = p.unit_a = p.unit_b = p.rev_m = p.rev_n = 0;
+    p.tail_first = 0; p.tail_slices = 1; p.tail_kps = K;
     const int idx = (tA ? 2 : 0) | (tB ? 1 : 0);
     int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return hipErrorInvalidValue;
@@ -200,6 +223,24 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             p.xcd_remap = 0;
         }
     }
+    int64_t grid_x = ntiles;
+    if (splits <= 1 && e.tri[idx]) {
+        const int ts = tail_slices_for(ntiles, K, e.bk, tail_ok);
+        if (ts > 1) {
+            const int64_t kps = ceil_div64(ceil_div64(K, ts), e.bk) * e.bk;
+            const int slices = (int)ceil_div64(K, kps);
+            const int64_t r = ntiles % 256;
+            void *w = workspace_get(stream, (size_t)(r * slices) * e.bm * e.bn * sizeof(T));
+            if (slices > 1 && w) {  // without workspace the plain schedule still works
+                fn = e.tri[idx];
+                p.tail_first = (int)(ntiles - r);
+                p.tail_slices = slices;
+                p.tail_kps = (int)kps;
+                p.ws = (T *)w;
+                grid_x = (ntiles - r) + r * slices;
+            }
+        }
+    }
     if (splits > 1) {
         int64_t kps = ceil_div64(ceil_div64(K, splits), e.bk) * e.bk;
         splits = (int)ceil_div64(K, kps);
@@ -218,9 +259,16 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         hipError_t err = ensure_dynamic_lds((const void *)fn, smem);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(fn, dim3((unsigned)ntiles, (unsigned)splits), dim3(e.threads), smem, stream, p);
+    hipLaunchKernelGGL(fn, dim3((unsigned)grid_x, (unsigned)splits), dim3(e.threads), smem, stream, p);
     hipError_t err = hipGetLastError();
     if (err != hipSuccess) return err;
+    if (p.tail_slices > 1) {
+        const int64_t r = ntiles - p.tail_first;
+        hipLaunchKernelGGL(tail_reduce_kernel<T>, dim3((unsigned)ceil_div64((int64_t)e.bm * e.bn, 256), (unsigned)r),
+                           dim3(256), 0, stream, p, e.bm, e.bn);
+        err = hipGetLastError();
+        if (err != hipSuccess) return err;
+    }
     if (splits > 1) {
         int mb = (int)ceil_div64(M, 256);
         hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, p.ws,

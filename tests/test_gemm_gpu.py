@@ -258,3 +258,25 @@ def test_two_streams_and_teardown(gpu):
         np.testing.assert_array_equal(d[5].cpu().numpy(), w2)
         clblas_amd.teardown()          # second pass runs after the scratch was released
     assert clblas_amd.setup() == 0
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex64, np.complex128])
+def test_sliced_tail_integer_exact(gpu, dtype):
+    """More than 256 tiles with a partly filled last round: the tiles of that round are cut into
+    K slices and finished by a reduction pass.  Exact-integer data, smallest tile forced so that
+    a modest problem has 18 x 16 = 288 tiles (32 in the last round, 4 slices of K = 520)."""
+    M, N, K = 1100, 1000, 520
+    cplx = np.dtype(dtype).kind == "c"
+    alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
+    small_tile = {np.float32: 2, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
+    for tA, tB in ((NOTRANS, NOTRANS), (TRANS, CONJ)):
+        lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
+        lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]
+        A = oracle.integers(na, 1, lim, dtype)
+        B = oracle.integers(nb, 2, lim, dtype)
+        C = oracle.integers(nc, 3, 8, dtype)
+        want = C.copy()
+        assert oracle.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, want, 7, ldc) == 0
+        st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, C, 7, ldc, tile=small_tile)
+        assert st == 0
+        np.testing.assert_array_equal(got, want)
