@@ -67,8 +67,9 @@ template <> struct Mma16<float> {
 // wavefront w owns equations [16w, 16w+16) as two 16 x 16 accumulator blocks (lane l:
 // right-hand side l%16 of each block, equations krow(l/16, v)).  Accumulator layout and
 // MFMA "B" operand layout coincide, so Y_s feeds the MFMAs as it is and X_s goes to the
-// other wavefronts through LDS in the same per-lane order.  Step s: wavefront s computes
-// X_s (8 MFMAs), publishes it, barrier, wavefronts w > s subtract L_ws X_s (8 MFMAs each).
+// other wavefronts through LDS in the same per-lane order.  Step s: wavefronts w > s subtract
+// L_ws X_s (8 MFMAs each); wavefront s+1 then computes X_(s+1) (8 MFMAs) and publishes it
+// while the others are still updating; one barrier per step.
 // For side=left a right-hand side is a column of B; the panel moves between HBM and the
 // accumulator layout through an LDS staging area so that global accesses run along columns.
 template <typename T> struct TrsmLeaf {
@@ -234,26 +235,32 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
             }
     }
 
+    // X_s = inv(L_ss) Y_s by the wavefront that owns row s; published in buffer s & 1.
+    auto solve_row = [&](int s) {
+        Acc x[NBK];
+#pragma unroll
+        for (int k = 0; k < NBK; ++k) x[k] = Acc{0, 0, 0, 0};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int k = 0; k < NBK; ++k) x[k] = M::run(ea[s % RING][c], y[k][c], x[k]);
+        T *Xs = X + (s & 1) * (NBK * 64 * 4);
+#pragma unroll
+        for (int k = 0; k < NBK; ++k) {
+            y[k] = x[k];
+            *reinterpret_cast<Acc *>(Xs + (k * 64 + lane) * 4) = x[k];
+        }
+    };
+    if (wave == 0) solve_row(0);
+    __syncthreads();
+    // Step s: every row w > s subtracts L_ws X_s; the owner of row s+1 then solves it at once,
+    // while the other wavefronts are still updating, so each step costs one barrier and the
+    // solves stay off the critical path of everyone else.
 #pragma unroll
     for (int s = 0; s < NBLK; ++s) {
         if (s < nsteps) {  // uniform over the workgroup
-            T *Xs = X + (s & 1) * (NBK * 64 * 4);
+            const T *Xs = X + (s & 1) * (NBK * 64 * 4);
             if (s + RING - 1 <= wave && wave < nsteps) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
-            if (wave == s) {
-                Acc x[NBK];
-#pragma unroll
-                for (int k = 0; k < NBK; ++k) x[k] = Acc{0, 0, 0, 0};
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int k = 0; k < NBK; ++k) x[k] = M::run(ea[s % RING][c], y[k][c], x[k]);
-#pragma unroll
-                for (int k = 0; k < NBK; ++k) {
-                    y[k] = x[k];
-                    *reinterpret_cast<Acc *>(Xs + (k * 64 + lane) * 4) = x[k];
-                }
-            }
-            __syncthreads();
             if (wave > s && wave < nsteps) {
                 Acc xb[NBK];
 #pragma unroll
@@ -262,7 +269,9 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
                 for (int c = 0; c < 4; ++c)
 #pragma unroll
                     for (int k = 0; k < NBK; ++k) y[k] = M::run(ea[s % RING][c], xb[k][c], y[k]);
+                if (wave == s + 1) solve_row(s + 1);
             }
+            __syncthreads();
         }
     }
 
