@@ -287,7 +287,13 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
     // (VEC rows apart) start 64 bytes = 16 banks apart.
     static constexpr int ROWS_PER_CHUNK = CHUNK / BX > 0 ? CHUNK / BX : 1;
     static constexpr int CHUNKS_APART = VEC / ROWS_PER_CHUNK > 0 ? VEC / ROWS_PER_CHUNK : 1;
-    static constexpr int CHUNK_PAD = MODE == LM_DMA_X ? (64 / (int)sizeof(T)) / CHUNKS_APART : 0;  // elements
+    // That is for the 32-lane groups of the FP32 MFMAs (512 contiguous bytes per group).  The
+    // FP64 MFMAs read in 16-lane groups of 256 bytes, and those are conflict-free exactly when
+    // all groups start in the same bank (measured: any stagger costs half of the LDS cycles),
+    // which the unpadded image gives (rows are multiples of 256 bytes apart).
+    static constexpr bool FP64_GROUPS = sizeof(typename Elem<T>::Real) == 8;
+    static constexpr int CHUNK_PAD =
+        (MODE == LM_DMA_X && !FP64_GROUPS) ? (64 / (int)sizeof(T)) / CHUNKS_APART : 0;  // elements
     static constexpr int CHUNK_PITCH = CHUNK + CHUNK_PAD;
     static constexpr int LDS_PITCH = MODE == LM_DMA_X ? BX : BK;
     static constexpr int LDS_ELEMS = (NVEC / 64) * CHUNK_PITCH;
