@@ -260,3 +260,38 @@ def test_validation_codes(gpu):
     assert clblas_amd.symm("S", COL, RIGHT, UPPER, 2, 4, 1, x, 0, 3, x, 0, 4, 0, x, 0, 4) == S.InvalidLeadDimA
     assert clblas_amd.symm("S", COL, LEFT, UPPER, 4, 4, 1, x, 0, 4, x, 0, 3, 0, x, 0, 4) == S.InvalidLeadDimB
     assert clblas_amd.symm("S", COL, LEFT, UPPER, 4, 4, 1, x, 0, 4, x, 0, 4, 0, x, 0, 3) == S.InvalidLeadDimC
+
+
+def test_workspaces_per_stream_growth_and_teardown(gpu):
+    """TRMM (copy of B) and TRSM (packed diagonal blocks) keep their workspaces per stream: two
+    streams run different problems at once, a later larger problem makes the workspaces grow,
+    and everything still works after clblasTeardown released them."""
+    import clblas_amd
+    import torch
+    dtype = np.float64
+    for rep, (M, N) in enumerate([(300, 200), (700, 520)]):
+        s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+        A1, lda1 = matrix(COL, M, M, 0, 0, 1 + rep, dtype, True, limit=4)
+        A2, lda2 = matrix(COL, N, N, 0, 0, 2 + rep, dtype, True, limit=4)
+        B1, ldb = matrix(COL, M, N, 0, 0, 3 + rep, dtype, True, limit=4)
+        B2 = oracle.integers(B1.size, 4 + rep, 4, dtype)
+        w1, w2 = B1.copy(), B2.copy()
+        assert oracle.trmm(COL, LEFT, LOWER, NOTRANS, NONUNIT, M, N, 2.0, A1, 0, lda1, w1, 0, ldb) == 0
+        assert oracle.trmm(COL, RIGHT, UPPER, TRANS, UNIT, M, N, 2.0, A2, 0, lda2, w2, 0, ldb) == 0
+        T1 = oracle.triangular(M, M, True, 5 + rep, dtype)
+        X = oracle.uniform(M * N, 6 + rep, dtype)
+        x_want = X.copy()
+        assert oracle.trsm_blocked(COL, LEFT, LOWER, NOTRANS, NONUNIT, M, N, 1.0, T1, 0, M, x_want, 0, M) == 0
+        d = [torch.from_numpy(x).cuda() for x in (A1, B1, A2, B2, T1, X)]
+        torch.cuda.synchronize()
+        assert clblas_amd.trmm("D", COL, LEFT, LOWER, NOTRANS, NONUNIT, M, N, 2.0, d[0], 0, lda1, d[1], 0, ldb, stream=s1) == 0
+        assert clblas_amd.trmm("D", COL, RIGHT, UPPER, TRANS, UNIT, M, N, 2.0, d[2], 0, lda2, d[3], 0, ldb, stream=s2) == 0
+        assert clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, M, N, 1.0, d[4], 0, M, d[5], 0, M, stream=s1) == 0
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(d[1].cpu().numpy(), w1)
+        np.testing.assert_array_equal(d[3].cpu().numpy(), w2)
+        got = d[5].cpu().numpy()
+        assert np.abs(got - x_want).max() <= 64 * M * np.finfo(dtype).eps * np.abs(x_want).max()
+        if rep == 0:
+            clblas_amd.teardown()
+    assert clblas_amd.setup() == 0
