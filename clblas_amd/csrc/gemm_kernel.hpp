@@ -1,4 +1,5 @@
-// MFMA GEMM kernel for gfx950 (CDNA4), FP32 and FP64, all four transpose combinations.
+// MFMA GEMM kernel for gfx950 (CDNA4): FP32, FP64 and their complex counterparts, all
+// transpose / conjugate combinations; the TRI variants also serve SYRK, TRMM and SYMM.
 //
 // Computes (column-major, after the host has folded row-major calls)
 //     C(m,n) <- alpha * sum_k opA(m,k) * opB(k,n) + beta * C(m,n)
@@ -34,6 +35,10 @@
 //         Re += ar*br,  Re += ai*(-bi),  Im += ar*bi,  Im += ai*br
 //     - four MFMAs per block and step, all of their flops useful, the only extra work one
 //     sign flip per B element.  Conjugation moves that flip to br and/or negates Im at the end.
+//   * Kernels instantiated with TRI = true additionally honour triangular structure (only a
+//     triangle of C exists; an operand is triangular: its zero half is skipped and the
+//     diagonal band is masked in LDS) and the sliced tail (the tiles of a partly filled last
+//     round are cut into K ranges); see GemmParams.  The plain instantiations carry none of it.
 #pragma once
 
 #include <hip/hip_runtime.h>
