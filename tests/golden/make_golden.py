@@ -1,5 +1,5 @@
 """Writes tests/golden/fixed_cases.json: the fixed-input cases the reference's own files hold
-for the xGEMM / xTRSM path, with expected outputs computed here in exact rational arithmetic
+for the xGEMM / xTRSM path and its SYMM / SYRK / TRMM neighbours, with expected outputs computed here in exact rational arithmetic
 (python Fractions) -- independent of both the oracle and the HIP library.
 
 Sources of the INPUT DATA (data only; no reference code is run or copied):
@@ -12,6 +12,12 @@ Sources of the INPUT DATA (data only; no reference code is run or copied):
                                 left/upper/notrans/nonunit, M=5, N=2, lda=ldb=32,
                                 a_rr=r+1, a_rc=1 (c>r), b_r = sum(1..M)-sum(1..r+1)+(r+1)^2
                                 => x_r = r+1 (closed form)
+  * src/samples/example_ssymm.c:30-63,146-148  row-major SSYMM left/lower, M=4, N=3,
+                                alpha=10, beta=20, upper triangle of A filled with -1
+  * src/samples/example_ssyrk.c:30-63,142-144  row-major SSYRK upper/notrans, sub-problem
+                                (N-1, K-1) at offA=K+1, offC=N+1, alpha=10, beta=20
+  * src/samples/example_strmm.c:30-63,140-142  row-major STRMM left/upper/notrans/nonunit,
+                                sub-problem (M-1, N-1) at offA=M+1, offB=N+1, alpha=10
 
 Run:  python tests/golden/make_golden.py
 """
@@ -86,6 +92,64 @@ def trsm_exact(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, 
     return out
 
 
+def tri_dense(order, uplo, tA, diag, n, A, offA, lda):
+    """Dense op(A) of a triangular matrix: zeros outside the `uplo` triangle, ones on a unit diagonal."""
+    opA = [[F(0)] * n for _ in range(n)]
+    for r in range(n):
+        for c in range(n):
+            rr, cc = (c, r) if tA != N_ else (r, c)
+            if not ((rr <= cc) if uplo == UPPER else (rr >= cc)):
+                continue
+            opA[r][c] = F(1) if (rr == cc and diag == UNIT) else F(A[offA + a_index(order, N_, rr, cc, lda)])
+    return opA
+
+
+def trmm_exact(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
+    n = M if side == LEFT else N
+    T = tri_dense(order, uplo, tA, diag, n, A, offA, lda)
+    out = [F(x) for x in B]
+    for i in range(M):
+        for j in range(N):
+            if side == LEFT:
+                s = sum(T[i][k] * F(B[offB + a_index(order, N_, k, j, ldb)]) for k in range(n))
+            else:
+                s = sum(F(B[offB + a_index(order, N_, i, k, ldb)]) * T[k][j] for k in range(n))
+            out[offB + a_index(order, N_, i, j, ldb)] = F(alpha) * s
+    return out
+
+
+def syrk_exact(order, uplo, tA, N, K, alpha, A, offA, lda, beta, C, offC, ldc):
+    out = [F(x) for x in C]
+    for i in range(N):
+        for j in range(N):
+            if not ((i <= j) if uplo == UPPER else (i >= j)):
+                continue
+            s = sum(F(A[offA + a_index(order, tA, i, k, lda)]) * F(A[offA + a_index(order, tA, j, k, lda)])
+                    for k in range(K))
+            ci = offC + a_index(order, N_, i, j, ldc)
+            out[ci] = F(alpha) * s + F(beta) * F(C[ci])
+    return out
+
+
+def symm_exact(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    n = M if side == LEFT else N
+
+    def a(r, c):  # symmetric element from the stored triangle
+        if not ((r <= c) if uplo == UPPER else (r >= c)):
+            r, c = c, r
+        return F(A[offA + a_index(order, N_, r, c, lda)])
+    out = [F(x) for x in C]
+    for i in range(M):
+        for j in range(N):
+            if side == LEFT:
+                s = sum(a(i, k) * F(B[offB + a_index(order, N_, k, j, ldb)]) for k in range(n))
+            else:
+                s = sum(F(B[offB + a_index(order, N_, i, k, ldb)]) * a(k, j) for k in range(n))
+            ci = offC + a_index(order, N_, i, j, ldc)
+            out[ci] = F(alpha) * s + F(beta) * F(C[ci])
+    return out
+
+
 def as_floats(v):
     return [float(x) for x in v]
 
@@ -131,6 +195,23 @@ def main():
         cases["extratest_" + dt] = dict(
             kind="trsm", dtype=dt, order=COL, side=LEFT, uplo=UPPER, transA=N_, diag=NONUNIT, M=Me, N=Ne, alpha=1,
             A=Ae, offA=0, lda=ld, B=Be, offB=0, ldb=ld, expected=as_floats(exp), tol=1e-5)
+    # SYMM / SYRK / TRMM samples
+    As = [11, -1, -1, -1, 21, 22, -1, -1, 31, 32, 33, -1, 41, 42, 43, 44]
+    Bs = [11, 12, 13, 21, 22, 23, 31, 32, 33, 41, 42, 43]
+    cases["sample_ssymm"] = dict(
+        kind="symm", dtype="f32", order=ROW, side=LEFT, uplo=LOWER, M=4, N=3, alpha=10, beta=20, A=As, offA=0, lda=4,
+        B=Bs, offB=0, ldb=3, C=list(Bs), offC=0, ldc=3,
+        expected=as_floats(symm_exact(ROW, LEFT, LOWER, 4, 3, 10, As, 0, 4, Bs, 0, 3, 20, Bs, 0, 3)))
+    Ak = [11, 12, 13, 14, 21, 22, 23, 24, 31, 32, 33, 34, 41, 42, 43, 44, 51, 52, 53, 54]
+    Ck = [11, 12, 13, 14, 15, 12, 22, 23, 24, 25, 13, 23, 33, 34, 35, 14, 24, 34, 44, 45, 15, 25, 35, 45, 55]
+    cases["sample_ssyrk_offsets"] = dict(
+        kind="syrk", dtype="f32", order=ROW, uplo=UPPER, transA=N_, N=4, K=3, alpha=10, beta=20, A=Ak, offA=5, lda=4,
+        C=Ck, offC=6, ldc=5,
+        expected=as_floats(syrk_exact(ROW, UPPER, N_, 4, 3, 10, Ak, 5, 4, 20, Ck, 6, 5)))
+    cases["sample_strmm_offsets"] = dict(
+        kind="trmm", dtype="f32", order=ROW, side=LEFT, uplo=UPPER, transA=N_, diag=NONUNIT, M=3, N=4, alpha=10,
+        A=At, offA=5, lda=4, B=Bt, offB=6, ldb=5,
+        expected=as_floats(trmm_exact(ROW, LEFT, UPPER, N_, NONUNIT, 3, 4, 10, At, 5, 4, Bt, 6, 5)))
     with open(os.path.join(HERE, "fixed_cases.json"), "w") as f:
         json.dump(cases, f, indent=1)
     print("wrote", len(cases), "cases")

@@ -295,3 +295,25 @@ def test_workspaces_per_stream_growth_and_teardown(gpu):
         if rep == 0:
             clblas_amd.teardown()
     assert clblas_amd.setup() == 0
+
+
+@pytest.mark.parametrize("name", ["sample_ssymm", "sample_ssyrk_offsets", "sample_strmm_offsets"])
+def test_level3_golden(gpu, name):
+    """Fixed inputs of src/samples/example_ssymm.c, example_ssyrk.c, example_strmm.c with expected
+    values computed in exact arithmetic (integers: the results are exact)."""
+    from helpers import golden_cases
+    c = golden_cases()[name]
+    dt = np.float32
+    A = np.array(c["A"], dtype=dt)
+    if c["kind"] == "syrk":
+        st, out = gpu.syrk(c["order"], c["uplo"], c["transA"], c["N"], c["K"], c["alpha"], A, c["offA"], c["lda"],
+                           c["beta"], np.array(c["C"], dtype=dt), c["offC"], c["ldc"])
+    elif c["kind"] == "trmm":
+        st, out = gpu.trmm(c["order"], c["side"], c["uplo"], c["transA"], c["diag"], c["M"], c["N"], c["alpha"], A,
+                           c["offA"], c["lda"], np.array(c["B"], dtype=dt), c["offB"], c["ldb"])
+    else:
+        st, out = gpu.symm(c["order"], c["side"], c["uplo"], c["M"], c["N"], c["alpha"], A, c["offA"], c["lda"],
+                           np.array(c["B"], dtype=dt), c["offB"], c["ldb"], c["beta"], np.array(c["C"], dtype=dt),
+                           c["offC"], c["ldc"])
+    assert st == 0
+    np.testing.assert_array_equal(out, np.array(c["expected"], dtype=dt))

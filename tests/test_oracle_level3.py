@@ -223,3 +223,33 @@ def test_symm_checks():
     assert oracle.symm(COL, RIGHT, UPPER, 2, 4, 1.0, A, 0, 3, A, 0, 4, 0.0, A, 0, 4) == -1016
     assert oracle.symm(COL, LEFT, UPPER, 4, 4, 1.0, A, 0, 4, A, 0, 3, 0.0, A, 0, 4) == -1015
     assert oracle.symm(COL, LEFT, UPPER, 4, 4, 1.0, A, 0, 4, A, 0, 4, 0.0, A, 0, 3) == -1014
+
+
+# ------------------------------------------------------------------------------- golden fixtures
+def _run_golden(mod_syrk, mod_trmm, mod_symm, c):
+    """Runs one fixed case (inputs from the reference's sample programs, expected values in
+    exact arithmetic) through the given routines; returns (status, result buffer)."""
+    dt = np.float32
+    A = np.array(c["A"], dtype=dt)
+    if c["kind"] == "syrk":
+        C = np.array(c["C"], dtype=dt)
+        return mod_syrk(c["order"], c["uplo"], c["transA"], c["N"], c["K"], c["alpha"], A, c["offA"], c["lda"],
+                        c["beta"], C, c["offC"], c["ldc"]), C
+    if c["kind"] == "trmm":
+        B = np.array(c["B"], dtype=dt)
+        return mod_trmm(c["order"], c["side"], c["uplo"], c["transA"], c["diag"], c["M"], c["N"], c["alpha"], A,
+                        c["offA"], c["lda"], B, c["offB"], c["ldb"]), B
+    B, C = np.array(c["B"], dtype=dt), np.array(c["C"], dtype=dt)
+    return mod_symm(c["order"], c["side"], c["uplo"], c["M"], c["N"], c["alpha"], A, c["offA"], c["lda"], B, c["offB"],
+                    c["ldb"], c["beta"], C, c["offC"], c["ldc"]), C
+
+
+@pytest.mark.parametrize("name", ["sample_ssymm", "sample_ssyrk_offsets", "sample_strmm_offsets"])
+def test_level3_golden(name):
+    """Fixed inputs of src/samples/example_ssymm.c, example_ssyrk.c, example_strmm.c (integers:
+    the results are exact)."""
+    from helpers import golden_cases
+    c = golden_cases()[name]
+    st, out = _run_golden(oracle.syrk, oracle.trmm, oracle.symm, c)
+    assert st == 0
+    np.testing.assert_array_equal(out, np.array(c["expected"], dtype=np.float32))
