@@ -100,6 +100,70 @@ def test_trsm_validation_matches_reference_checks(fn):
     assert f(COL, 5, LOWER, NOTRANS, NONUNIT, 4, 4, 1.0, FAKE, 0, 4, FAKE, 0, 4, stream=0) == clblas_amd.Status.InvalidValue
 
 
+@pytest.mark.parametrize("fn", ["cgemm", "zgemm"])
+def test_complex_gemm_validation(fn):
+    f = getattr(clblas_amd, fn)
+    for (order, tA, tB, M, N, K, lda, ldb, ldc) in GEMM_BAD:
+        want = oracle.check_gemm(order, tA, tB, M, N, K, 1, 0, lda, 0, 1, 0, ldb, 0, 1, 0, ldc, 0)
+        if want == 0:
+            continue
+        assert f(order, tA, tB, M, N, K, 1 + 1j, FAKE, 0, lda, FAKE, 0, ldb, 0, FAKE, 0, ldc, stream=0) == want
+    assert f(COL, 0, 0, 4, 4, 4, 1, None, 0, 4, FAKE, 0, 4, 0, FAKE, 0, 4, stream=0) == -1022
+    assert f(COL, 0, 3, 4, 4, 4, 1, FAKE, 0, 4, FAKE, 0, 4, 0, FAKE, 0, 4, stream=0) == clblas_amd.Status.InvalidValue
+
+
+def _np_of(prefix):
+    import numpy as np
+    return {"S": np.float32, "D": np.float64, "C": np.complex64, "Z": np.complex128}[prefix]
+
+
+@pytest.mark.parametrize("prefix", ["S", "D", "C", "Z"])
+def test_level3_validation_matches_the_oracle_checks(prefix):
+    """SYRK / TRMM / SYMM: for every invalid argument set the library returns what the oracle's
+    restatement of doSyrk / doTrmm / doSymm returns (the oracle gets a small real buffer, the
+    library fake non-null pointers, which it never touches because validation fails first)."""
+    import numpy as np
+    buf = np.zeros(4096, dtype=_np_of(prefix))
+    S = clblas_amd.Status
+    hit = set()
+    for order, uplo, tA in itertools.product([ROW, COL], [UPPER, LOWER], [NOTRANS, TRANS, CONJ]):
+        for (N, K, lda, ldc) in [(0, 4, 8, 8), (4, 0, 8, 8), (6, 4, 3, 8), (4, 6, 3, 8), (6, 4, 8, 5), (5, 5, 4, 4)]:
+            want = oracle.syrk(order, uplo, tA, N, K, 1, buf, 0, lda, 0, buf, 0, ldc)
+            if want == 0:
+                continue  # valid arguments (the oracle just computed on its scratch buffer)
+            got = clblas_amd.syrk(prefix, order, uplo, tA, N, K, 1, FAKE, 0, lda, 0, FAKE, 0, ldc, stream=0)
+            assert got == want, ("syrk", order, uplo, tA, N, K, lda, ldc)
+            hit.add(want)
+    for order, side, tA in itertools.product([ROW, COL], [LEFT, RIGHT], [NOTRANS, TRANS]):
+        for (M, N, lda, ldb) in [(0, 4, 8, 8), (4, 0, 8, 8), (6, 4, 5, 8), (4, 6, 5, 8), (6, 4, 8, 3), (4, 6, 8, 3)]:
+            want = oracle.trmm(order, side, LOWER, tA, NONUNIT, M, N, 1, buf, 0, lda, buf, 0, ldb)
+            if want != 0:
+                got = clblas_amd.trmm(prefix, order, side, LOWER, tA, NONUNIT, M, N, 1, FAKE, 0, lda, FAKE, 0, ldb, stream=0)
+                assert got == want, ("trmm", order, side, tA, M, N, lda, ldb)
+                hit.add(want)
+            for ldc in (8, 3):
+                want = oracle.symm(order, side, LOWER, M, N, 1, buf, 0, lda, buf, 0, ldb, 0, buf, 0, ldc)
+                if want != 0:
+                    got = clblas_amd.symm(prefix, order, side, LOWER, M, N, 1, FAKE, 0, lda, FAKE, 0, ldb, 0, FAKE, 0, ldc,
+                                          stream=0)
+                    assert got == want, ("symm", order, side, M, N, lda, ldb, ldc)
+                    hit.add(want)
+    assert {-1017, -1016, -1015, -1014} <= hit
+    if prefix in "CZ":
+        assert S.InvalidValue in hit  # ConjTrans SYRK on a complex type (xsyrk.c:61-63)
+    # null objects and enum values outside the reference's enums
+    assert clblas_amd.syrk(prefix, COL, LOWER, NOTRANS, 4, 4, 1, None, 0, 4, 0, FAKE, 0, 4, stream=0) == S.InvalidMatA
+    assert clblas_amd.syrk(prefix, COL, LOWER, NOTRANS, 4, 4, 1, FAKE, 0, 4, 0, None, 0, 4, stream=0) == S.InvalidMatC
+    assert clblas_amd.syrk(prefix, COL, 7, NOTRANS, 4, 4, 1, FAKE, 0, 4, 0, FAKE, 0, 4, stream=0) == S.InvalidValue
+    assert clblas_amd.trmm(prefix, COL, LEFT, LOWER, NOTRANS, NONUNIT, 4, 4, 1, None, 0, 4, FAKE, 0, 4, stream=0) == S.InvalidMatA
+    assert clblas_amd.trmm(prefix, COL, LEFT, LOWER, NOTRANS, NONUNIT, 4, 4, 1, FAKE, 0, 4, None, 0, 4, stream=0) == S.InvalidMatB
+    assert clblas_amd.trmm(prefix, COL, LEFT, LOWER, NOTRANS, 9, 4, 4, 1, FAKE, 0, 4, FAKE, 0, 4, stream=0) == S.InvalidValue
+    assert clblas_amd.symm(prefix, COL, LEFT, LOWER, 4, 4, 1, None, 0, 4, FAKE, 0, 4, 0, FAKE, 0, 4, stream=0) == S.InvalidMatA
+    assert clblas_amd.symm(prefix, COL, LEFT, LOWER, 4, 4, 1, FAKE, 0, 4, None, 0, 4, 0, FAKE, 0, 4, stream=0) == S.InvalidMatB
+    assert clblas_amd.symm(prefix, COL, LEFT, LOWER, 4, 4, 1, FAKE, 0, 4, FAKE, 0, 4, 0, None, 0, 4, stream=0) == S.InvalidMatC
+    assert clblas_amd.symm(prefix, 2, LEFT, LOWER, 4, 4, 1, FAKE, 0, 4, FAKE, 0, 4, 0, FAKE, 0, 4, stream=0) == S.InvalidValue
+
+
 def test_product_package_does_not_touch_the_oracle():
     pkg = os.path.join(ROOT, "clblas_amd")
     for dirpath, _, files in os.walk(pkg):
