@@ -73,6 +73,8 @@ EXPORTED_SYMBOLS = (
     "clblasZgemm",
     "clblasStrsm",
     "clblasDtrsm",
+    "clblasCtrsm",
+    "clblasZtrsm",
 ) + tuple("clblas%s%s" % (t, f) for f in ("syrk", "trmm", "symm") for t in "SDCZ")
 
 _lib = None
@@ -102,6 +104,10 @@ def _declare(lib):
         fn = getattr(lib, name)
         fn.restype = i
         fn.argtypes = [i, i, i, i, i, sz, sz, real, vp, sz, sz, vp, sz, sz, vp]
+    for name, cplx in (("clblasCtrsm", FloatComplex), ("clblasZtrsm", DoubleComplex)):
+        fn = getattr(lib, name)
+        fn.restype = i
+        fn.argtypes = [i, i, i, i, i, sz, sz, cplx, vp, sz, sz, vp, sz, sz, vp]
     scalars = {"S": ctypes.c_float, "D": ctypes.c_double, "C": FloatComplex, "Z": DoubleComplex}
     for t, sc in scalars.items():
         fn = getattr(lib, "clblas%ssyrk" % t)
@@ -203,6 +209,18 @@ def strsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, l
 def dtrsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):
     return load_library().clblasDtrsm(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha,
                                       _ptr(A), offA, lda, _ptr(B), offB, ldb, _stream(stream))
+
+
+def ctrsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):
+    """alpha: Python complex; A, B: complex64 tensors (or device addresses)."""
+    return load_library().clblasCtrsm(int(order), int(side), int(uplo), int(transA), int(diag), M, N,
+                                      _scalar("C", alpha), _ptr(A), offA, lda, _ptr(B), offB, ldb, _stream(stream))
+
+
+def ztrsm(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream=None):
+    """alpha: Python complex; A, B: complex128 tensors (or device addresses)."""
+    return load_library().clblasZtrsm(int(order), int(side), int(uplo), int(transA), int(diag), M, N,
+                                      _scalar("Z", alpha), _ptr(A), offA, lda, _ptr(B), offB, ldb, _stream(stream))
 
 
 def _scalar(prefix, x):

@@ -44,7 +44,7 @@ void usage() {
         "  -o/--order 0|1                                0 = row major, 1 = column major\n"
         "  --transposeA 0|1|2  --transposeB 0|1|2\n"
         "  --side 0|1  --uplo 0|1  --diag 0|1            0 = left/upper/unit\n"
-        "  -f/--function gemm|trsm|trmm|syrk|symm   -r/--precision s|d|c|z (trsm: s|d)\n"
+        "  -f/--function gemm|trsm|trmm|syrk|symm   -r/--precision s|d|c|z\n"
         "  -p/--profile N                                timed samples (default 20)\n"
         "  --apiCallCount N                              calls per sample (default 10)\n"
         "  --label TEXT  --noheader");
@@ -151,10 +151,15 @@ clblasStatus trsm(clblasOrder o, clblasSide sd, clblasUplo u, clblasTranspose ta
                   double al, const double *a, size_t oa, size_t lda, double *b, size_t ob, size_t ldb, hipStream_t s) {
     return clblasDtrsm(o, sd, u, ta, d, m, n, al, a, oa, lda, b, ob, ldb, s);
 }
-template <typename T>
-clblasStatus trsm(clblasOrder, clblasSide, clblasUplo, clblasTranspose, clblasDiag, size_t, size_t, T, const T *, size_t,
-                  size_t, T *, size_t, size_t, hipStream_t) {
-    return clblasNotImplemented;  // complex TRSM is not part of this library
+clblasStatus trsm(clblasOrder o, clblasSide sd, clblasUplo u, clblasTranspose ta, clblasDiag d, size_t m, size_t n,
+                  FloatComplex al, const FloatComplex *a, size_t oa, size_t lda, FloatComplex *b, size_t ob, size_t ldb,
+                  hipStream_t s) {
+    return clblasCtrsm(o, sd, u, ta, d, m, n, al, a, oa, lda, b, ob, ldb, s);
+}
+clblasStatus trsm(clblasOrder o, clblasSide sd, clblasUplo u, clblasTranspose ta, clblasDiag d, size_t m, size_t n,
+                  DoubleComplex al, const DoubleComplex *a, size_t oa, size_t lda, DoubleComplex *b, size_t ob,
+                  size_t ldb, hipStream_t s) {
+    return clblasZtrsm(o, sd, u, ta, d, m, n, al, a, oa, lda, b, ob, ldb, s);
 }
 
 enum Fn { FN_GEMM, FN_TRSM, FN_TRMM, FN_SYRK, FN_SYMM };
@@ -267,8 +272,8 @@ int main(int argc, char **argv) {
     for (int i = 0; i < 5; ++i)
         if (o.function == fnames[i]) fn = i;
     const bool real = o.precision == "s" || o.precision == "d", cplx = o.precision == "c" || o.precision == "z";
-    if (fn < 0 || !(real || cplx) || (fn == FN_TRSM && !real)) {
-        std::fprintf(stderr, "this library implements -f gemm|trmm|syrk|symm with -r s|d|c|z and -f trsm with -r s|d\n");
+    if (fn < 0 || !(real || cplx)) {
+        std::fprintf(stderr, "this library implements -f gemm|trsm|trmm|syrk|symm with -r s|d|c|z\n");
         return 2;
     }
     if (clblasSetup() != clblasSuccess) { std::fprintf(stderr, "clblasSetup failed (needs a gfx950 device)\n"); return 1; }

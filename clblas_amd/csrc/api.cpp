@@ -257,8 +257,8 @@ static_assert(sizeof(FloatComplex) == sizeof(cba::Cx<float>) && sizeof(DoubleCom
 inline cba::Cx<float> cx(FloatComplex z) { return cba::Cx<float>{z.s[0], z.s[1]}; }
 inline cba::Cx<double> cx(DoubleComplex z) { return cba::Cx<double>{z.s[0], z.s[1]}; }
 
-template <typename T, typename Fn>
-clblasStatus trsm_front(Fn launch, clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+template <typename T>
+clblasStatus trsm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
                         clblasDiag diag, size_t M, size_t N, T alpha, const T *A, size_t offA, size_t lda, T *B,
                         size_t offB, size_t ldb, hipStream_t stream) {
     // Order of checks follows doTrsm (functor_xtrsm.cc:57-75): objects, A (msize^2), B (M x N).
@@ -282,8 +282,9 @@ clblasStatus trsm_front(Fn launch, clblasOrder order, clblasSide side, clblasUpl
         right = !right;
         lower = !lower;
     }
-    return map_hip_error(launch(right, lower, transA != clblasNoTrans, diag == clblasUnit, (int)M, (int)N, alpha,
-                                A + offA, (int64_t)lda, B + offB, (int64_t)ldb, stream));
+    return map_hip_error(cba::trsm_colmajor<T>(right, lower, transA != clblasNoTrans, transA == clblasConjTrans,
+                                               diag == clblasUnit, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
+                                               B + offB, (int64_t)ldb, stream));
 }
 
 }  // namespace
@@ -357,15 +358,31 @@ clblasStatus clblasZgemm(clblasOrder order, clblasTranspose transA, clblasTransp
 clblasStatus clblasStrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
                          clblasDiag diag, size_t M, size_t N, float alpha, const float *A, size_t offA, size_t lda,
                          float *B, size_t offB, size_t ldb, hipStream_t stream) {
-    return trsm_front<float>(cba::strsm_colmajor, order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
+    return trsm_front<float>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
                              offB, ldb, stream);
 }
 
 clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
                          clblasDiag diag, size_t M, size_t N, double alpha, const double *A, size_t offA,
                          size_t lda, double *B, size_t offB, size_t ldb, hipStream_t stream) {
-    return trsm_front<double>(cba::dtrsm_colmajor, order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
+    return trsm_front<double>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
                               offB, ldb, stream);
+}
+
+clblasStatus clblasCtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, FloatComplex alpha, const FloatComplex *A, size_t offA,
+                         size_t lda, FloatComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<cba::Cx<float>>(order, side, uplo, transA, diag, M, N, cx(alpha),
+                                      reinterpret_cast<const cba::Cx<float> *>(A), offA, lda,
+                                      reinterpret_cast<cba::Cx<float> *>(B), offB, ldb, stream);
+}
+
+clblasStatus clblasZtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
+                         clblasDiag diag, size_t M, size_t N, DoubleComplex alpha, const DoubleComplex *A, size_t offA,
+                         size_t lda, DoubleComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<cba::Cx<double>>(order, side, uplo, transA, diag, M, N, cx(alpha),
+                                       reinterpret_cast<const cba::Cx<double> *>(A), offA, lda,
+                                       reinterpret_cast<cba::Cx<double> *>(B), offB, ldb, stream);
 }
 
 clblasStatus clblasSsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,

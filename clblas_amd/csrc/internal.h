@@ -78,10 +78,10 @@ template <typename T>
 hipError_t symm_colmajor(bool right, bool lower, int M, int N, T alpha, const T *A, int64_t lda, const T *B,
                          int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream);
 
-// Column-major TRSM drivers (same conventions).
-hipError_t strsm_colmajor(bool right, bool lower, bool trans, bool unit, int M, int N, float alpha, const float *A,
-                          int64_t lda, float *B, int64_t ldb, hipStream_t stream);
-hipError_t dtrsm_colmajor(bool right, bool lower, bool trans, bool unit, int M, int N, double alpha,
-                          const double *A, int64_t lda, double *B, int64_t ldb, hipStream_t stream);
+// Column-major TRSM driver (trsm.hip), all four types: solves op(A) X = alpha B (left) or
+// X op(A) = alpha B (right) in place; `conj` conjugates op(A) (complex, clblasConjTrans).
+template <typename T>
+hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool conj, bool unit, int M, int N, T alpha, const T *A,
+                         int64_t lda, T *B, int64_t ldb, hipStream_t stream);
 
 }  // namespace cba

@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "gemm_kernel.hpp"
 #include "internal.h"
 
 namespace cba {
@@ -73,22 +74,62 @@ template <> struct Mma16<float> {
 // For side=left a right-hand side is a column of B; the panel moves between HBM and the
 // accumulator layout through an LDS staging area so that global accesses run along columns.
 template <typename T> struct TrsmLeaf {
-    static constexpr int NB = 256, IB = 16, NBLK = NB / IB, CW = 32, NBK = CW / 16, THREADS = 64 * NBLK;
+    typedef typename Elem<T>::Real R;
+    static constexpr bool CPLX = Elem<T>::CPLX;
+    static constexpr int NB = 256, IB = 16, NBLK = NB / IB, THREADS = 64 * NBLK;
+    // Right-hand sides per workgroup: complex elements cost four MFMAs per product and twice
+    // the staging space, so they take half as many.
+    static constexpr int CW = CPLX ? 16 : 32, NBK = CW / 16;
     static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;  // sub-blocks (bi,bj), bi >= bj, at bi*(bi+1)/2 + bj
-    static constexpr int PACK_ELEMS = N_EBLK * IB * IB;   // per diagonal block
-    static constexpr int X_ELEMS = 2 * NBK * 64 * 4;      // two buffers of X_s in per-lane order
-    static constexpr int SP = NB + 2;                     // pitch of the right-hand-side staging area
+    // Packed sub-block: PLANES x 64 lanes x 4 reals.  Real: the values.  Complex: real parts,
+    // imaginary parts, negated imaginary parts (so that no sign has to be flipped in the solve).
+    static constexpr int PLANES = CPLX ? 3 : 1;
+    static constexpr int SUB_REALS = PLANES * IB * IB;
+    static constexpr int PACK_REALS = N_EBLK * SUB_REALS;  // per diagonal block
+    static constexpr int NP = CPLX ? 2 : 1;                // accumulators per block (re, im)
+    static constexpr int X_REALS = 2 * NP * NBK * 64 * 4;  // two buffers of X_s in per-lane order
+    static constexpr int SP = NB + 2;                      // pitch of the right-hand-side staging area
     static constexpr int S_ELEMS = CW * SP;
-    static constexpr size_t SMEM = (size_t)(X_ELEMS + S_ELEMS) * sizeof(T);
+    static constexpr size_t SMEM = (size_t)X_REALS * sizeof(R) + (size_t)S_ELEMS * sizeof(T);
 };
+
+// Element helpers for the packing pass (real and complex).
+static __device__ __forceinline__ float tr_conj_if(float x, bool) { return x; }
+static __device__ __forceinline__ double tr_conj_if(double x, bool) { return x; }
+template <typename R> static __device__ __forceinline__ Cx<R> tr_conj_if(Cx<R> x, bool c) { return Cx<R>{x.re, c ? -x.im : x.im}; }
+static __device__ __forceinline__ float tr_mul(float a, float b) { return a * b; }
+static __device__ __forceinline__ double tr_mul(double a, double b) { return a * b; }
+template <typename R> static __device__ __forceinline__ Cx<R> tr_mul(Cx<R> a, Cx<R> b) {
+    return Cx<R>{a.re * b.re - a.im * b.im, a.re * b.im + a.im * b.re};
+}
+static __device__ __forceinline__ float tr_sub(float a, float b) { return a - b; }
+static __device__ __forceinline__ double tr_sub(double a, double b) { return a - b; }
+template <typename R> static __device__ __forceinline__ Cx<R> tr_sub(Cx<R> a, Cx<R> b) { return Cx<R>{a.re - b.re, a.im - b.im}; }
+static __device__ __forceinline__ float tr_div(float a, float b) { return a / b; }
+static __device__ __forceinline__ double tr_div(double a, double b) { return a / b; }
+template <typename R> static __device__ __forceinline__ Cx<R> tr_div(Cx<R> a, Cx<R> b) {
+    const R d = b.re * b.re + b.im * b.im;
+    return Cx<R>{(a.re * b.re + a.im * b.im) / d, (a.im * b.re - a.re * b.im) / d};
+}
+// Writes value v (to be used as it is) into the planes of a packed sub-block at index w.
+static __device__ __forceinline__ void tr_put(float *sub, int w, float v) { sub[w] = v; }
+static __device__ __forceinline__ void tr_put(double *sub, int w, double v) { sub[w] = v; }
+template <typename R> static __device__ __forceinline__ void tr_put(R *sub, int w, Cx<R> v) {
+    sub[w] = v.re;
+    sub[256 + w] = v.im;
+    sub[512 + w] = -v.im;
+}
 
 // Packs all diagonal blocks of the n x n triangle (see above).  Workgroup (bi, b) of 256
 // threads packs sub-block row bi of diagonal block b (rows/columns [256 b, 256 b + nb)).
+// `conj` conjugates the coefficients (complex, clblasConjTrans).
 template <typename T, bool FORWARD>
 __global__ void __launch_bounds__(256)
-trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool unit, T *__restrict__ pack) {
+trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool conj, bool unit,
+                 typename Elem<T>::Real *__restrict__ pack) {
     typedef TrsmLeaf<T> L;
-    typedef Mma16<T> M;
+    typedef typename Elem<T>::Real R;
+    typedef Mma16<R> M;
     constexpr int IB = L::IB;
     __shared__ T Ld[IB][IB + 1];  // the diagonal sub-triangle, then its inverse
     const int tid = threadIdx.x;
@@ -96,29 +137,27 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool un
     const int i0 = blockIdx.y * L::NB;
     const int nb = n - i0 < L::NB ? n - i0 : L::NB;
     const T *Ablk = A + i0 + (int64_t)i0 * lda;
-    T *out = pack + (int64_t)blockIdx.y * L::PACK_ELEMS + (int64_t)(bi * (bi + 1) / 2) * (IB * IB);
-    auto coef = [&](int P, int Q) -> T {  // Q < P < nb
+    R *out = pack + (int64_t)blockIdx.y * L::PACK_REALS + (int64_t)(bi * (bi + 1) / 2) * L::SUB_REALS;
+    auto coef = [&](int P, int Q) -> T {  // Q <= P < nb
         const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
-        return teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
+        return tr_conj_if(teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda], conj);
     };
     // off-diagonal sub-blocks (bi, 0..bi-1), negated; rows past nb are zero
     for (int e = tid; e < bi * IB * IB; e += 256) {
         const int bj = e / (IB * IB), w = e % (IB * IB);
         const int lane = w / 4, c = w % 4;
         const int P = bi * IB + lane % 16, Q = bj * IB + M::krow(lane / 16, c);
-        out[e] = (P < nb) ? -coef(P, Q) : (T)0;  // Q < P always holds here; Q < nb follows from P < nb
+        // Q < P always holds here; Q < nb follows from P < nb
+        tr_put(out + bj * L::SUB_REALS, w, (P < nb) ? tr_sub(T(), coef(P, Q)) : T());
     }
     // diagonal sub-triangle into LDS (identity where the block is short)
     {
         const int p = tid / IB, q = tid % IB;
         const int P = bi * IB + p, Q = bi * IB + q;
-        T v = (T)0;
+        T v = T();
         if (p == q) {
-            v = (T)1;
-            if (!unit && P < nb) {
-                const int ip = FORWARD ? P : nb - 1 - P;
-                v = Ablk[ip + (int64_t)ip * lda];
-            }
+            v = el_one<T>();
+            if (!unit && P < nb) v = coef(P, P);
         } else if (q < p && P < nb) {
             v = coef(P, Q);
         }
@@ -131,11 +170,11 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool un
     if (tid < IB) {
 #pragma unroll
         for (int p = 0; p < IB; ++p) {
-            T acc = (p == zc) ? (T)1 : (T)0;
+            T acc = (p == zc) ? el_one<T>() : T();
 #pragma unroll
             for (int q = 0; q < IB; ++q)
-                if (q < p) acc -= Ld[p][q] * z[q];
-            z[p] = (p < zc) ? (T)0 : acc / Ld[p][p];
+                if (q < p) acc = tr_sub(acc, tr_mul(Ld[p][q], z[q]));
+            z[p] = (p < zc) ? T() : tr_div(acc, Ld[p][p]);
         }
     }
     __syncthreads();
@@ -146,22 +185,26 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool un
     __syncthreads();
     {
         const int lane = tid / 4, c = tid % 4;
-        out[bi * (IB * IB) + tid] = Ld[lane % 16][M::krow(lane / 16, c)];
+        tr_put(out + bi * L::SUB_REALS, tid, Ld[lane % 16][M::krow(lane / 16, c)]);
     }
 }
 
 template <typename T, bool RIGHT, bool FORWARD>
 __global__ void __launch_bounds__(TrsmLeaf<T>::THREADS)
-trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk, int64_t ldb, int nrhs) {
+trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk,
+                 int64_t ldb, int nrhs) {
     typedef TrsmLeaf<T> L;
-    typedef Mma16<T> M;
+    typedef typename Elem<T>::Real R;
+    typedef Mma16<R> M;
     typedef typename M::Acc Acc;
-    constexpr int IB = L::IB, CW = L::CW, NBK = L::NBK, NT = L::THREADS, NBLK = L::NBLK;
-    constexpr int V = 16 / (int)sizeof(T);  // elements per 16 bytes
-    typedef T VT __attribute__((ext_vector_type(V)));
+    constexpr bool CPLX = L::CPLX;
+    constexpr int IB = L::IB, CW = L::CW, NBK = L::NBK, NT = L::THREADS, NBLK = L::NBLK, NP = L::NP;
+    constexpr int PLANES = L::PLANES;
+    constexpr int V = 16 / (int)sizeof(R);  // reals per 16 bytes
+    typedef R VT __attribute__((ext_vector_type(V)));
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    T *X = reinterpret_cast<T *>(smem_raw);
-    T *S = X + L::X_ELEMS;
+    R *X = reinterpret_cast<R *>(smem_raw);
+    T *S = reinterpret_cast<T *>(X + L::X_REALS);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -170,26 +213,37 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
     const int64_t j0 = (int64_t)blockIdx.x * CW;
     const int nsteps = (nb + IB - 1) / IB;  // sub-block rows that exist
 
-    // A lane's four values of sub-block (wave, s): MFMA "A" operand, chunk c = element c.
-    const T *erow = packed + (int64_t)(wave * (wave + 1) / 2) * (IB * IB) + lane * 4;
-    auto load_e = [&](int s, T (&a)[4]) {
-        const T *src = erow + s * (IB * IB);
+    // A lane's values of sub-block (wave, s): MFMA "A" operand, plane pl, chunk c = element c.
+    const R *erow = packed + (int64_t)(wave * (wave + 1) / 2) * L::SUB_REALS + lane * 4;
+    auto load_e = [&](int s, R (&a)[PLANES][4]) {
 #pragma unroll
-        for (int c = 0; c < 4; c += V) {
-            VT t = *reinterpret_cast<const VT *>(src + c);
+        for (int pl = 0; pl < PLANES; ++pl) {
+            const R *src = erow + s * L::SUB_REALS + pl * (IB * IB);
 #pragma unroll
-            for (int e = 0; e < V && c + e < 4; ++e) a[c + e] = t[e];
+            for (int c = 0; c < 4; c += V) {
+                VT t = *reinterpret_cast<const VT *>(src + c);
+#pragma unroll
+                for (int e = 0; e < V && c + e < 4; ++e) a[pl][c + e] = t[e];
+            }
         }
     };
-    constexpr int RING = 3;  // sub-blocks in flight: this step's and the next two
-    T ea[RING][4];
+    constexpr int RING = CPLX ? 2 : 3;  // sub-blocks in flight: this step's and the next one or two
+    R ea[RING][PLANES][4];
 #pragma unroll
     for (int s = 0; s < RING - 1; ++s)
         if (s <= wave && wave < nsteps) load_e(s, ea[s]);
 
-    // ---- right-hand sides into the accumulator layout: y[k][v] = alpha * b(equation krow(g,v) of
-    //      this wavefront, right-hand side j0 + 16k + jj) ----
-    Acc y[NBK];
+    // ---- right-hand sides into the accumulator layout: y[.][k][v] = alpha * b(equation krow(g,v)
+    //      of this wavefront, right-hand side j0 + 16k + jj); complex: [0] real, [1] imaginary ----
+    Acc y[NP][NBK];
+    auto put_y = [&](int k, int v, T b) {
+        const T ab = el_scale(alpha, b);
+        if constexpr (CPLX) { y[0][k][v] = ab.re; y[1][k][v] = ab.im; } else { y[0][k][v] = ab; }
+    };
+    auto get_y = [&](int k, int v) -> T {
+        if constexpr (CPLX) return T{y[0][k][v], y[1][k][v]};
+        else return y[0][k][v];
+    };
     auto mem_row = [&](int P) { return FORWARD ? P : nb - 1 - P; };
     if (RIGHT) {
 #pragma unroll
@@ -198,9 +252,9 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int P = wave * IB + M::krow(g, v);
-                T b = (T)0;
+                T b = T();
                 if (P < nb && j < nrhs) b = Bblk[j + (int64_t)mem_row(P) * ldb];
-                y[k][v] = alpha * b;
+                put_y(k, v, b);
             }
         }
     } else {
@@ -210,8 +264,8 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
         for (int u = 0; u < NLD; ++u) {
             const int e = tid + u * NT;
             const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-            v0[u] = (T)0;
-            v1[u] = (T)0;
+            v0[u] = T();
+            v1[u] = T();
             if (j0 + c < nrhs) {
                 const T *src = Bblk + r + (j0 + c) * ldb;
                 if (r < nb) v0[u] = src[0];
@@ -231,25 +285,43 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int P = wave * IB + M::krow(g, v);
-                y[k][v] = (P < nb) ? alpha * S[(16 * k + jj) * L::SP + mem_row(P)] : (T)0;
+                put_y(k, v, (P < nb) ? S[(16 * k + jj) * L::SP + mem_row(P)] : T());
             }
     }
 
-    // X_s = inv(L_ss) Y_s by the wavefront that owns row s; published in buffer s & 1.
-    auto solve_row = [&](int s) {
-        Acc x[NBK];
-#pragma unroll
-        for (int k = 0; k < NBK; ++k) x[k] = Acc{0, 0, 0, 0};
+    // out (+)= E * in for one sub-block E (this lane's packed values e) and the blocks `in` in
+    // MFMA "B" operand order.  Complex: Re += er*inr + (-ei)*ini, Im += er*ini + ei*inr.
+    auto block_mma = [&](const R (&e)[PLANES][4], const Acc (&in)[NP][NBK], Acc (&out)[NP][NBK]) {
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
-            for (int k = 0; k < NBK; ++k) x[k] = M::run(ea[s % RING][c], y[k][c], x[k]);
-        T *Xs = X + (s & 1) * (NBK * 64 * 4);
+            for (int k = 0; k < NBK; ++k) {
+                if constexpr (CPLX) {
+                    out[0][k] = M::run(e[0][c], in[0][k][c], out[0][k]);
+                    out[1][k] = M::run(e[0][c], in[1][k][c], out[1][k]);
+                    out[0][k] = M::run(e[2][c], in[1][k][c], out[0][k]);
+                    out[1][k] = M::run(e[1][c], in[0][k][c], out[1][k]);
+                } else {
+                    out[0][k] = M::run(e[0][c], in[0][k][c], out[0][k]);
+                }
+            }
+    };
+    // X_s = inv(L_ss) Y_s by the wavefront that owns row s; published in buffer s & 1.
+    auto solve_row = [&](int s) {
+        Acc x[NP][NBK];
 #pragma unroll
-        for (int k = 0; k < NBK; ++k) {
-            y[k] = x[k];
-            *reinterpret_cast<Acc *>(Xs + (k * 64 + lane) * 4) = x[k];
-        }
+        for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+            for (int k = 0; k < NBK; ++k) x[pp][k] = Acc{0, 0, 0, 0};
+        block_mma(ea[s % RING], y, x);
+        R *Xs = X + (s & 1) * (NP * NBK * 64 * 4);
+#pragma unroll
+        for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+            for (int k = 0; k < NBK; ++k) {
+                y[pp][k] = x[pp][k];
+                *reinterpret_cast<Acc *>(Xs + ((pp * NBK + k) * 64 + lane) * 4) = x[pp][k];
+            }
     };
     if (wave == 0) solve_row(0);
     __syncthreads();
@@ -259,16 +331,16 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
 #pragma unroll
     for (int s = 0; s < NBLK; ++s) {
         if (s < nsteps) {  // uniform over the workgroup
-            const T *Xs = X + (s & 1) * (NBK * 64 * 4);
+            const R *Xs = X + (s & 1) * (NP * NBK * 64 * 4);
             if (s + RING - 1 <= wave && wave < nsteps) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
             if (wave > s && wave < nsteps) {
-                Acc xb[NBK];
+                Acc xb[NP][NBK];
 #pragma unroll
-                for (int k = 0; k < NBK; ++k) xb[k] = *reinterpret_cast<const Acc *>(Xs + (k * 64 + lane) * 4);
+                for (int pp = 0; pp < NP; ++pp)
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int k = 0; k < NBK; ++k) y[k] = M::run(ea[s % RING][c], xb[k][c], y[k]);
+                    for (int k = 0; k < NBK; ++k)
+                        xb[pp][k] = *reinterpret_cast<const Acc *>(Xs + ((pp * NBK + k) * 64 + lane) * 4);
+                block_mma(ea[s % RING], xb, y);
                 if (wave == s + 1) solve_row(s + 1);
             }
             __syncthreads();
@@ -282,17 +354,17 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int P = wave * IB + M::krow(g, v);
-                if (P < nb && j < nrhs) Bblk[j + (int64_t)mem_row(P) * ldb] = y[k][v];
+                if (P < nb && j < nrhs) Bblk[j + (int64_t)mem_row(P) * ldb] = get_y(k, v);
             }
         }
     } else {
-        // The staging area was last read before the first step's barrier.
+        // The staging area was last read before the first barrier of the solve.
 #pragma unroll
         for (int k = 0; k < NBK; ++k)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int P = wave * IB + M::krow(g, v);
-                if (P < nb) S[(16 * k + jj) * L::SP + mem_row(P)] = y[k][v];
+                if (P < nb) S[(16 * k + jj) * L::SP + mem_row(P)] = get_y(k, v);
             }
         __syncthreads();
         constexpr int NLD = CW * (L::NB / 2) / NT;
@@ -309,43 +381,38 @@ trsm_diag_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ 
     }
 }
 
-template <typename T> struct GemmOf;
-template <> struct GemmOf<float> {
-    static hipError_t run(bool tA, bool tB, int M, int N, int K, float alpha, const float *A, int64_t lda,
-                          const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t s) {
-        return sgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s);
-    }
-};
-template <> struct GemmOf<double> {
-    static hipError_t run(bool tA, bool tB, int M, int N, int K, double alpha, const double *A, int64_t lda,
-                          const double *B, int64_t ldb, double beta, double *C, int64_t ldc, hipStream_t s) {
-        return dgemm_colmajor(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, s);
-    }
-};
-
 template <typename T> struct TrsmDriver {
+    typedef typename Elem<T>::Real R;
     static constexpr int NBL = TrsmLeaf<T>::NB;
-    bool right, trans, unit, forward, teff;
+    bool right, trans, conj, unit, forward, teff;
     int M, N;
     const T *A;
     int64_t lda;
     T *B;
     int64_t ldb;
     hipStream_t stream;
-    const T *pack;  // packed diagonal blocks, TrsmLeaf<T>::PACK_ELEMS each
+    const R *pack;  // packed diagonal blocks, TrsmLeaf<T>::PACK_REALS each
+
+    static T minus_one() { return el_scale_host(-1); }
+    static T el_scale_host(int v) {
+        if constexpr (Elem<T>::CPLX) return T{(R)v, (R)0};
+        else return (T)v;
+    }
 
     // Packs every diagonal block of the triangle (one launch per call).
     hipError_t prepare() {
         typedef TrsmLeaf<T> L;
         const int n = right ? N : M;
         const int nblk = (n + NBL - 1) / NBL;
-        T *w = (T *)workspace_get(stream, (size_t)nblk * L::PACK_ELEMS * sizeof(T), 2);
+        R *w = (R *)workspace_get(stream, (size_t)nblk * L::PACK_REALS * sizeof(R), 2);
         if (!w) return hipErrorOutOfMemory;
         pack = w;
         if (forward)
-            hipLaunchKernelGGL((trsm_pack_kernel<T, true>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff, unit, w);
+            hipLaunchKernelGGL((trsm_pack_kernel<T, true>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
+                               conj, unit, w);
         else
-            hipLaunchKernelGGL((trsm_pack_kernel<T, false>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff, unit, w);
+            hipLaunchKernelGGL((trsm_pack_kernel<T, false>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
+                               conj, unit, w);
         return hipGetLastError();
     }
 
@@ -353,8 +420,8 @@ template <typename T> struct TrsmDriver {
         const int nrhs = right ? M : N;
         T *Bblk = right ? B + (int64_t)i0 * ldb : B + i0;
         typedef TrsmLeaf<T> L;
-        const T *packed = pack + (int64_t)(i0 / NBL) * L::PACK_ELEMS;
-        void (*fn)(const T *, int, T, T *, int64_t, int);
+        const R *packed = pack + (int64_t)(i0 / NBL) * L::PACK_REALS;
+        void (*fn)(const R *, int, T, T *, int64_t, int);
         if (right) fn = forward ? trsm_diag_kernel<T, true, true> : trsm_diag_kernel<T, true, false>;
         else fn = forward ? trsm_diag_kernel<T, false, true> : trsm_diag_kernel<T, false, false>;
         if (L::SMEM > 64 * 1024) {
@@ -372,11 +439,12 @@ template <typename T> struct TrsmDriver {
         if (!right) {
             // rows: B[d0.., :] -= op(A)[d0.., s0..] * B[s0.., :]
             const T *Ablk = trans ? A + s0 + (int64_t)d0 * lda : A + d0 + (int64_t)s0 * lda;
-            return GemmOf<T>::run(trans, false, nd, N, ns, (T)-1, Ablk, lda, B + s0, ldb, beta, B + d0, ldb, stream);
+            return launch_gemm<T>(trans, false, conj, false, nd, N, ns, minus_one(), Ablk, lda, B + s0, ldb, beta, B + d0,
+                                  ldb, stream);
         }
         // columns: B[:, d0..] -= B[:, s0..] * op(A)[s0.., d0..]
         const T *Ablk = trans ? A + d0 + (int64_t)s0 * lda : A + s0 + (int64_t)d0 * lda;
-        return GemmOf<T>::run(false, trans, M, nd, ns, (T)-1, B + (int64_t)s0 * ldb, ldb, Ablk, lda, beta,
+        return launch_gemm<T>(false, trans, false, conj, M, nd, ns, minus_one(), B + (int64_t)s0 * ldb, ldb, Ablk, lda, beta,
                               B + (int64_t)d0 * ldb, ldb, stream);
     }
 
@@ -392,19 +460,19 @@ template <typename T> struct TrsmDriver {
         if (forward) {
             if ((e = solve(i0, n_lo, alpha)) != hipSuccess) return e;
             if ((e = update(i0 + n_lo, n_hi, i0, n_lo, alpha)) != hipSuccess) return e;
-            return solve(i0 + n_lo, n_hi, (T)1);
+            return solve(i0 + n_lo, n_hi, el_scale_host(1));
         }
         if ((e = solve(i0 + n_lo, n_hi, alpha)) != hipSuccess) return e;
         if ((e = update(i0, n_lo, i0 + n_lo, n_hi, alpha)) != hipSuccess) return e;
-        return solve(i0, n_lo, (T)1);
+        return solve(i0, n_lo, el_scale_host(1));
     }
 };
 
 template <typename T>
-static hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool unit, int M, int N, T alpha, const T *A,
-                                int64_t lda, T *B, int64_t ldb, hipStream_t stream) {
+hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool conj, bool unit, int M, int N, T alpha, const T *A,
+                         int64_t lda, T *B, int64_t ldb, hipStream_t stream) {
     TrsmDriver<T> d;
-    d.right = right; d.trans = trans; d.unit = unit;
+    d.right = right; d.trans = trans; d.conj = conj && Elem<T>::CPLX; d.unit = unit;
     // Left: equations run forward when op(A) is lower triangular; right: when it is upper.
     d.forward = right ? (lower == trans) : (lower != trans);
     d.teff = trans != right;
@@ -414,14 +482,13 @@ static hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool unit, i
     return d.solve(0, right ? N : M, alpha);
 }
 
-hipError_t strsm_colmajor(bool right, bool lower, bool trans, bool unit, int M, int N, float alpha, const float *A,
-                          int64_t lda, float *B, int64_t ldb, hipStream_t stream) {
-    return trsm_colmajor<float>(right, lower, trans, unit, M, N, alpha, A, lda, B, ldb, stream);
-}
-
-hipError_t dtrsm_colmajor(bool right, bool lower, bool trans, bool unit, int M, int N, double alpha,
-                          const double *A, int64_t lda, double *B, int64_t ldb, hipStream_t stream) {
-    return trsm_colmajor<double>(right, lower, trans, unit, M, N, alpha, A, lda, B, ldb, stream);
-}
+template hipError_t trsm_colmajor<float>(bool, bool, bool, bool, bool, int, int, float, const float *, int64_t, float *,
+                                         int64_t, hipStream_t);
+template hipError_t trsm_colmajor<double>(bool, bool, bool, bool, bool, int, int, double, const double *, int64_t,
+                                          double *, int64_t, hipStream_t);
+template hipError_t trsm_colmajor<Cx<float>>(bool, bool, bool, bool, bool, int, int, Cx<float>, const Cx<float> *,
+                                             int64_t, Cx<float> *, int64_t, hipStream_t);
+template hipError_t trsm_colmajor<Cx<double>>(bool, bool, bool, bool, bool, int, int, Cx<double>, const Cx<double> *,
+                                              int64_t, Cx<double> *, int64_t, hipStream_t);
 
 }  // namespace cba

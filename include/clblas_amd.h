@@ -162,6 +162,19 @@ clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo,
                          double alpha, const double *A, size_t offA, size_t lda,
                          double *B, size_t offB, size_t ldb, hipStream_t stream);
 
+/* Replaces clblasCtrsm (src/clBLAS.h:8132-8152, src/library/blas/xtrsm.cc:1789-1850).
+ * transA == clblasConjTrans solves with the conjugate transpose of A. */
+clblasStatus clblasCtrsm(clblasOrder order, clblasSide side, clblasUplo uplo,
+                         clblasTranspose transA, clblasDiag diag, size_t M, size_t N,
+                         FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                         FloatComplex *B, size_t offB, size_t ldb, hipStream_t stream);
+
+/* Replaces clblasZtrsm (src/clBLAS.h:8202-8222, src/library/blas/xtrsm.cc:1852-1914). */
+clblasStatus clblasZtrsm(clblasOrder order, clblasSide side, clblasUplo uplo,
+                         clblasTranspose transA, clblasDiag diag, size_t M, size_t N,
+                         DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                         DoubleComplex *B, size_t offB, size_t ldb, hipStream_t stream);
+
 /* ---- GEMM-shaped neighbours on the same MFMA core: SYRK, TRMM, SYMM (all four types) ---- */
 
 /* Replace clblas{S,D,C,Z}syrk (src/clBLAS.h:8278-8503, src/library/blas/xsyrk.c:27-233).

@@ -61,6 +61,10 @@ def lib():
             f = getattr(L, name)
             f.restype = _i
             f.argtypes = [_i, _i, _i, _i, _i, _sz, _sz, real, _vp, _sz, _sz, _vp, _sz, _sz]
+        for name in ("oracle_ctrsm_naive", "oracle_ztrsm_naive"):
+            f = getattr(L, name)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz]
         for t in "sdcz":
             f = getattr(L, "oracle_%ssyrk" % t)
             f.restype = _i
@@ -113,6 +117,8 @@ def ref_lib():
         L.ref_naive_syrk.argtypes = [_i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _vp, _sz]
         L.ref_naive_trmm.restype = None
         L.ref_naive_trmm.argtypes = [_i, _i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _sz]
+        L.ref_naive_trsm.restype = None
+        L.ref_naive_trsm.argtypes = [_i, _i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _sz]
         for name, real in (("ref_naive_strsm", ctypes.c_float), ("ref_naive_dtrsm", ctypes.c_double)):
             f = getattr(L, name)
             f.restype = None
@@ -180,6 +186,10 @@ def gemm_exact(transA, transB, K, alpha, A, lda, B, ldb, beta, C, ldc, rows, col
 
 def trsm_naive(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
     ref = B if B is not None else A
+    if _is_complex(ref):
+        f = lib().oracle_ctrsm_naive if ref.dtype == np.complex64 else lib().oracle_ztrsm_naive
+        return f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, _p(_scalar(alpha, ref.dtype)),
+                 _p(A), offA, lda, _p(B), offB, ldb)
     f = lib().oracle_strsm_naive if ref.dtype == np.float32 else lib().oracle_dtrsm_naive
     return f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha, _p(A), offA, lda, _p(B), offB,
              ldb)
@@ -266,6 +276,10 @@ def ref_gemm(order, transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc
 
 
 def ref_trsm(order, side, uplo, transA, diag, M, N, alpha, A, lda, B, ldb):
+    if _is_complex(B):
+        ref_lib().ref_naive_trsm(2 if B.dtype == np.complex64 else 3, int(order), int(side), int(uplo), int(transA),
+                                 int(diag), M, N, _p(_scalar(alpha, B.dtype)), _p(A), lda, _p(B), ldb)
+        return
     f = ref_lib().ref_naive_strsm if B.dtype == np.float32 else ref_lib().ref_naive_dtrsm
     f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha, _p(A), lda, _p(B), ldb)
 

@@ -24,6 +24,10 @@
  *   oracle_{s,d}trsm_naive  - TRSM_extratest closed form (src/tests/correctness/corr-trsm.cpp:
  *                             240-452, X_r = r+1); src/samples/example_strsm.c:30-63 fixed
  *                             input; oracle/_ref naive trsm; residual identities.
+ *   oracle_{c,z}trsm_naive  - src/samples/example_ctrsm.c fixed input solved exactly; oracle/_ref
+ *                             naive trsm<FloatComplex/DoubleComplex>; residual against a complex
+ *                             product computed with numpy; real-embedding identity (a complex
+ *                             system with zero imaginary parts equals the real routine).
  *   oracle_{s,d}trsm_blocked- the same, plus agreement with the naive solver within the
  *                             reference's own per-element bound (trsm-delta.h:44-240 style),
  *                             NaN-poisoned unused triangle, zero-diagonal -> 1 behaviour.
@@ -466,6 +470,78 @@ CGEMM_EXACT(oracle_zgemm_exact, double, long double, fabsl)
 
 TRSM_NAIVE(oracle_strsm_naive, float)
 TRSM_NAIVE(oracle_dtrsm_naive, double)
+
+/* The same statement for complex elements (interleaved re, im; alpha by address): the template
+ * above instantiated with FloatComplex / DoubleComplex, whose product and quotient are
+ * naive_blas.cpp:300-390 ((a*b).re = ar*br - ai*bi, (a*b).im = ar*bi + br*ai;
+ * a/b = (ar*br + ai*bi, br*ai - ar*bi) / (br^2 + bi^2)).  transA == ConjTrans conjugates every
+ * element read from A (MatrixAccessor conj_, naive_blas.cpp:494, 466-472).  Right-hand sides
+ * are independent of each other, so the loop over them is outermost here (and parallel); the
+ * arithmetic on each is in the reference's order. */
+#define CTRSM_NAIVE(NAME, R)                                                                                   \
+    int NAME(int order, int side, int uplo, int transA, int diag, size_t M, size_t N, const R *alpha,          \
+             const R *A, size_t offA, size_t lda, R *B, size_t offB, size_t ldb) {                             \
+        int st = oracle_check_trsm(order, side, transA, M, N, A != NULL, offA, lda, 0, B != NULL, offB, ldb,   \
+                                   0);                                                                         \
+        size_t rowsA, colsB, a_rowstride, a_colstride, b_rowstride, b_colstride;                               \
+        ptrdiff_t jj;                                                                                          \
+        int rev, tra;                                                                                          \
+        const R csign = transA == CONJ_TRANS ? (R)-1 : (R)1;                                                   \
+        if (st) return st;                                                                                     \
+        A += 2 * offA;                                                                                         \
+        B += 2 * offB;                                                                                         \
+        rowsA = side == LEFT ? M : N;                                                                          \
+        colsB = side == LEFT ? N : M;                                                                          \
+        tra = transA != NO_TRANS;                                                                              \
+        rev = (uplo == UPPER) ^ tra;                                                                           \
+        if (side == RIGHT) {                                                                                   \
+            tra = !tra;                                                                                        \
+            rev = !rev;                                                                                        \
+        }                                                                                                      \
+        if ((order == COL_MAJOR) != tra) { a_rowstride = 1; a_colstride = lda; }                               \
+        else { a_rowstride = lda; a_colstride = 1; }                                                           \
+        if ((order == COL_MAJOR) != (side == RIGHT)) { b_rowstride = 1; b_colstride = ldb; }                   \
+        else { b_rowstride = ldb; b_colstride = 1; }                                                           \
+        _Pragma("omp parallel for schedule(static)")                                                           \
+        for (jj = 0; jj < (ptrdiff_t)colsB; ++jj) {                                                            \
+            const size_t j = (size_t)jj;                                                                       \
+            size_t i, k;                                                                                       \
+            for (i = 0; i < rowsA; ++i) {                                                                      \
+                const size_t row = rev ? rowsA - i - 1 : i;                                                    \
+                const size_t boundK = rev ? rowsA - row - 1 : row;                                             \
+                R *bx = B + 2 * (b_rowstride * row + b_colstride * j);                                         \
+                R tr = 0, ti = 0;                                                                              \
+                for (k = 0; k <= boundK; ++k) {                                                                \
+                    const size_t col = rev ? rowsA - k - 1 : k;                                                \
+                    const R *ap = A + 2 * (a_rowstride * row + a_colstride * col);                             \
+                    if (col == row) {                                                                          \
+                        const R ar = diag == UNIT ? (R)1 : ap[0], ai = diag == UNIT ? (R)0 : csign * ap[1];    \
+                        const R nr = bx[0] - tr, ni = bx[1] - ti, div = ar * ar + ai * ai;                     \
+                        tr = (nr * ar + ni * ai) / div;                                                        \
+                        ti = (ar * ni - nr * ai) / div;                                                        \
+                    } else {                                                                                   \
+                        const R ar = ap[0], ai = csign * ap[1];                                                \
+                        const R *bp = B + 2 * (b_rowstride * col + b_colstride * j);                           \
+                        const R pr = ar * bp[0] - ai * bp[1], pi = ar * bp[1] + bp[0] * ai;                    \
+                        tr = tr + pr;                                                                          \
+                        ti = ti + pi;                                                                          \
+                    }                                                                                          \
+                }                                                                                              \
+                bx[0] = tr;                                                                                    \
+                bx[1] = ti;                                                                                    \
+            }                                                                                                  \
+            for (i = 0; i < rowsA; ++i) {                                                                      \
+                R *bx = B + 2 * (b_rowstride * i + b_colstride * j);                                           \
+                const R xr = bx[0], xi = bx[1];                                                                \
+                bx[0] = xr * alpha[0] - xi * alpha[1];                                                         \
+                bx[1] = xr * alpha[1] + alpha[0] * xi;                                                         \
+            }                                                                                                  \
+        }                                                                                                      \
+        return ST_SUCCESS;                                                                                     \
+    }
+
+CTRSM_NAIVE(oracle_ctrsm_naive, float)
+CTRSM_NAIVE(oracle_ztrsm_naive, double)
 
 /* The reference's device algorithm for DTRSM: gpu_dtrsm128, src/library/blas/xtrsm.cc:1136-1507.
  *   1. InvA <- explicit inverses of the NB x NB (NB = 128) diagonal blocks of A

@@ -101,4 +101,12 @@ void ref_naive_trmm(int type, int order, int side, int uplo, int trans, int diag
                                      (T *)B, ldb)))
 }
 
+void ref_naive_trsm(int type, int order, int side, int uplo, int trans, int diag, size_t M, size_t N,
+                    const void *alpha, const void *A, size_t lda, void *B, size_t ldb) {
+    REF_DISPATCH((NaiveBlas::trsm<T>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasSide)side,
+                                     (NaiveBlas::clblasUplo)uplo, (NaiveBlas::clblasTranspose)trans,
+                                     (NaiveBlas::clblasDiag)diag, M, N, ref_scalar<T, R>(alpha), (const T *)A, lda,
+                                     (T *)B, ldb)))
+}
+
 }  // extern "C"

@@ -12,6 +12,8 @@ Sources of the INPUT DATA (data only; no reference code is run or copied):
                                 left/upper/notrans/nonunit, M=5, N=2, lda=ldb=32,
                                 a_rr=r+1, a_rc=1 (c>r), b_r = sum(1..M)-sum(1..r+1)+(r+1)^2
                                 => x_r = r+1 (closed form)
+  * src/samples/example_ctrsm.c:30-63,145-147  the same numbers as FloatComplex with zero imaginary
+                                parts, same call (clblasCtrsm)
   * src/samples/example_ssymm.c:30-63,146-148  row-major SSYMM left/lower, M=4, N=3,
                                 alpha=10, beta=20, upper triangle of A filled with -1
   * src/samples/example_ssyrk.c:30-63,142-144  row-major SSYRK upper/notrans, sub-problem
@@ -212,6 +214,12 @@ def main():
         kind="trmm", dtype="f32", order=ROW, side=LEFT, uplo=UPPER, transA=N_, diag=NONUNIT, M=3, N=4, alpha=10,
         A=At, offA=5, lda=4, B=Bt, offB=6, ldb=5,
         expected=as_floats(trmm_exact(ROW, LEFT, UPPER, N_, NONUNIT, 3, 4, 10, At, 5, 4, Bt, 6, 5)))
+    # The CTRSM sample holds the STRSM sample's numbers as complex values with zero imaginary
+    # parts, so its exact solution is the real one (imaginary parts stay zero).
+    cases["sample_ctrsm_offsets"] = dict(
+        kind="trsm", dtype="c64", order=ROW, side=LEFT, uplo=UPPER, transA=N_, diag=NONUNIT, M=3, N=4, alpha=10,
+        A=At, offA=5, lda=4, B=Bt, offB=6, ldb=5,
+        expected=as_floats(trsm_exact(ROW, LEFT, UPPER, N_, NONUNIT, 3, 4, 10, At, 5, 4, Bt, 6, 5)))
     with open(os.path.join(HERE, "fixed_cases.json"), "w") as f:
         json.dump(cases, f, indent=1)
     print("wrote", len(cases), "cases")

@@ -27,7 +27,8 @@ def gemm(order, tA, tB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, off
 
 
 def trsm(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
-    fn = clblas_amd.strsm if B.dtype == np.float32 else clblas_amd.dtrsm
+    fn = {np.dtype(np.float32): clblas_amd.strsm, np.dtype(np.float64): clblas_amd.dtrsm,
+          np.dtype(np.complex64): clblas_amd.ctrsm, np.dtype(np.complex128): clblas_amd.ztrsm}[B.dtype]
     dA, dB = _dev(A), _dev(B)
     st = fn(order, side, uplo, tA, diag, M, N, alpha, dA, offA, lda, dB, offB, ldb)
     torch.cuda.synchronize()

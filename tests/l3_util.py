@@ -86,3 +86,37 @@ def bound(K, mag, dtype, c=2.0):
 def err(got, want):
     d = got - want
     return np.maximum(np.abs(d.real), np.abs(d.imag)) if np.iscomplexobj(d) else np.abs(d)
+
+
+# ---- complex triangular systems (CTRSM / ZTRSM) -------------------------------------------
+
+def ctrsm_inputs(order, side, uplo, diag, M, N, dtype, seed, offA=5, offB=7):
+    """Conditioned complex triangular A (real part from the real generator - strict triangle
+    uniform/n, diagonal in [1,2) - plus an imaginary part of the same size; NaN outside the
+    triangle and on a unit diagonal) and a uniform complex B, with offsets and padded leading
+    dimensions."""
+    real = np.float32 if np.dtype(dtype) == np.dtype(np.complex64) else np.float64
+    n = M if side == LEFT else N
+    lda = n + 3
+    lower_in_memory = (uplo == LOWER) == (order == COL)
+    re = oracle.triangular(n, lda, lower_in_memory, seed, real, poison_diag=(diag == UNIT))
+    im = oracle.triangular(n, lda, lower_in_memory, seed + 100, real, poison_diag=(diag == UNIT))
+    sq = im[:n * lda].reshape(n, lda)[:, :n]
+    sq[np.eye(n, dtype=bool)] -= real(1.5)  # diagonal imaginary parts in [-0.5, 0.5)
+    A = np.concatenate([np.full(offA, nan_of(dtype), dtype=dtype), (re + 1j * im).astype(dtype)])
+    ib, ob = (M, N) if order == COL else (N, M)
+    ldb = ib + 2
+    B = oracle.uniform(offB + ob * ldb, seed + 1, dtype)
+    return A, lda, B, ldb
+
+
+def trsm_backward_error(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B0, X, offB, ldb):
+    """Normwise backward error ||op(A) X - alpha B|| / (||op(A)|| ||X|| + |alpha| ||B||) (infinity
+    norms; X op(A) for side == right), evaluated with numpy in complex128."""
+    n = M if side == LEFT else N
+    Am = op(tri_dense(A, order, n, offA, lda, uplo, diag == UNIT), tA)
+    Xm = logical_view(X, order, NOTRANS, M, N, offB, ldb).astype(np.complex128)
+    Bm = logical_view(B0, order, NOTRANS, M, N, offB, ldb).astype(np.complex128)
+    R = (Am @ Xm if side == LEFT else Xm @ Am) - alpha * Bm
+    nrm = lambda Z: np.abs(Z).sum(axis=1).max()
+    return nrm(R) / (nrm(Am) * nrm(Xm) + abs(alpha) * nrm(Bm))

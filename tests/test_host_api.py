@@ -81,7 +81,7 @@ def test_gemm_validation_matches_reference_checks(fn):
     assert f(COL, 3, 0, 4, 4, 4, 1.0, FAKE, 0, 4, FAKE, 0, 4, 0.0, FAKE, 0, 4, stream=0) == clblas_amd.Status.InvalidValue
 
 
-@pytest.mark.parametrize("fn", ["strsm", "dtrsm"])
+@pytest.mark.parametrize("fn", ["strsm", "dtrsm", "ctrsm", "ztrsm"])
 def test_trsm_validation_matches_reference_checks(fn):
     f = getattr(clblas_amd, fn)
     hit = set()
