@@ -12,6 +12,10 @@
 // The block sweep directions are those of xtrsm.cc:1226-1477; alpha is applied exactly once
 // to every element of B (xtrsm.cc:1236-1240).
 //
+// Complex types (clblasCtrsm / clblasZtrsm, xtrsm.cc:1789-1914) run through the same driver and
+// kernels: the packing pass conjugates for clblasConjTrans and splits every sub-block into real
+// planes, the leaf does four real MFMAs per complex product, the updates are CGEMM / ZGEMM.
+//
 // A zero on a non-unit diagonal gives Inf/NaN (1/0); the reference's inversion kernel
 // substitutes 1 instead (trtri/diag_dtrtri_lower_128_16.cpp:93-96).
 #include <hip/hip_runtime.h>
