@@ -75,7 +75,8 @@ EXPORTED_SYMBOLS = (
     "clblasDtrsm",
     "clblasCtrsm",
     "clblasZtrsm",
-) + tuple("clblas%s%s" % (t, f) for f in ("syrk", "trmm", "symm") for t in "SDCZ")
+) + tuple("clblas%s%s" % (t, f) for f in ("syrk", "trmm", "symm", "syr2k") for t in "SDCZ") + tuple(
+    "clblas%s%s" % (t, f) for f in ("herk", "her2k", "hemm") for t in "CZ")
 
 _lib = None
 
@@ -117,6 +118,19 @@ def _declare(lib):
         fn.restype = i
         fn.argtypes = [i, i, i, i, i, sz, sz, sc, vp, sz, sz, vp, sz, sz, vp]
         fn = getattr(lib, "clblas%ssymm" % t)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, sc, vp, sz, sz, vp, sz, sz, sc, vp, sz, sz, vp]
+        fn = getattr(lib, "clblas%ssyr2k" % t)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, sc, vp, sz, sz, vp, sz, sz, sc, vp, sz, sz, vp]
+    for t, sc, real in (("C", FloatComplex, ctypes.c_float), ("Z", DoubleComplex, ctypes.c_double)):
+        fn = getattr(lib, "clblas%sherk" % t)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, real, vp, sz, sz, real, vp, sz, sz, vp]
+        fn = getattr(lib, "clblas%sher2k" % t)
+        fn.restype = i
+        fn.argtypes = [i, i, i, sz, sz, sc, vp, sz, sz, vp, sz, sz, real, vp, sz, sz, vp]
+        fn = getattr(lib, "clblas%shemm" % t)
         fn.restype = i
         fn.argtypes = [i, i, i, sz, sz, sc, vp, sz, sz, vp, sz, sz, sc, vp, sz, sz, vp]
     lib.clblasSetup.restype = i
@@ -251,5 +265,33 @@ def trmm(prefix, order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, 
 def symm(prefix, order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
     """clblas{prefix}symm, prefix in "SDCZ" (src/clBLAS.h:8897-9145)."""
     fn = getattr(load_library(), "clblas%ssymm" % prefix)
+    return fn(int(order), int(side), int(uplo), M, N, _scalar(prefix, alpha), _ptr(A), offA, lda, _ptr(B), offB, ldb,
+              _scalar(prefix, beta), _ptr(C), offC, ldc, _stream(stream))
+
+
+def syr2k(prefix, order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    """clblas{prefix}syr2k, prefix in "SDCZ" (src/clBLAS.h:8568-8819)."""
+    fn = getattr(load_library(), "clblas%ssyr2k" % prefix)
+    return fn(int(order), int(uplo), int(transAB), N, K, _scalar(prefix, alpha), _ptr(A), offA, lda, _ptr(B), offB, ldb,
+              _scalar(prefix, beta), _ptr(C), offC, ldc, _stream(stream))
+
+
+def herk(prefix, order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, stream=None):
+    """clblas{prefix}herk, prefix in "CZ"; alpha and beta real (src/clBLAS.h:9389-9476)."""
+    fn = getattr(load_library(), "clblas%sherk" % prefix)
+    return fn(int(order), int(uplo), int(transA), N, K, float(alpha), _ptr(A), offA, lda, float(beta), _ptr(C), offC,
+              ldc, _stream(stream))
+
+
+def her2k(prefix, order, uplo, trans, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    """clblas{prefix}her2k, prefix in "CZ"; alpha complex, beta real (src/clBLAS.h:9545-9644)."""
+    fn = getattr(load_library(), "clblas%sher2k" % prefix)
+    return fn(int(order), int(uplo), int(trans), N, K, _scalar(prefix, alpha), _ptr(A), offA, lda, _ptr(B), offB, ldb,
+              float(beta), _ptr(C), offC, ldc, _stream(stream))
+
+
+def hemm(prefix, order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    """clblas{prefix}hemm, prefix in "CZ" (src/clBLAS.h:9224-9326)."""
+    fn = getattr(load_library(), "clblas%shemm" % prefix)
     return fn(int(order), int(side), int(uplo), M, N, _scalar(prefix, alpha), _ptr(A), offA, lda, _ptr(B), offB, ldb,
               _scalar(prefix, beta), _ptr(C), offC, ldc, _stream(stream))

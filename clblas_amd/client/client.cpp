@@ -1,7 +1,8 @@
 // clblas_amd-client: benchmark command line for libclblas_amd.so.
 //
 // Takes the place of the reference's clBLAS-client (src/client/client.cpp:80-112 for the
-// option names, src/client/clfunc_x{gemm,trsm,trmm,syrk,symm}.hpp for the GFLOP/s formulas)
+// option names, src/client/clfunc_x{gemm,trsm,trmm,syrk,symm,syr2k,herk,her2k,hemm}.hpp for the GFLOP/s
+// formulas)
 // for the function families this library implements, and prints the
 // CSV schema of the reference's published benchmark files (doc/performance/**.csv):
 //   m,n,k,lda,ldb,ldc,offa,offb,offc,alpha,beta,order,transa,transb,side,uplo,diag,
@@ -44,7 +45,7 @@ void usage() {
         "  -o/--order 0|1                                0 = row major, 1 = column major\n"
         "  --transposeA 0|1|2  --transposeB 0|1|2\n"
         "  --side 0|1  --uplo 0|1  --diag 0|1            0 = left/upper/unit\n"
-        "  -f/--function gemm|trsm|trmm|syrk|symm   -r/--precision s|d|c|z\n"
+        "  -f/--function gemm|trsm|trmm|syrk|symm|syr2k|herk|her2k|hemm   -r/--precision s|d|c|z\n"
         "  -p/--profile N                                timed samples (default 20)\n"
         "  --apiCallCount N                              calls per sample (default 10)\n"
         "  --label TEXT  --noheader");
@@ -137,6 +138,11 @@ template <> struct Type<DoubleComplex> {
                       size_t lda, const T *b, size_t ob, size_t ldb, T be, T *c, size_t oc, size_t ldc,              \
                       hipStream_t s) {                                                                               \
         return clblas##L##symm(o, sd, u, m, n, al, a, oa, lda, b, ob, ldb, be, c, oc, ldc, s);                       \
+    }                                                                                                                \
+    clblasStatus syr2k(clblasOrder o, clblasUplo u, clblasTranspose t, size_t n, size_t k, T al, const T *a,         \
+                       size_t oa, size_t lda, const T *b, size_t ob, size_t ldb, T be, T *c, size_t oc, size_t ldc,  \
+                       hipStream_t s) {                                                                              \
+        return clblas##L##syr2k(o, u, t, n, k, al, a, oa, lda, b, ob, ldb, be, c, oc, ldc, s);                       \
     }
 CLIENT_OVERLOADS(float, S)
 CLIENT_OVERLOADS(double, D)
@@ -162,7 +168,31 @@ clblasStatus trsm(clblasOrder o, clblasSide sd, clblasUplo u, clblasTranspose ta
     return clblasZtrsm(o, sd, u, ta, d, m, n, al, a, oa, lda, b, ob, ldb, s);
 }
 
-enum Fn { FN_GEMM, FN_TRSM, FN_TRMM, FN_SYRK, FN_SYMM };
+// Hermitian routines exist for the complex types only; alpha (HERK) and beta (HERK, HER2K) are real.
+#define CLIENT_HERMITIAN(T, L)                                                                                       \
+    clblasStatus herk(clblasOrder o, clblasUplo u, clblasTranspose t, size_t n, size_t k, T al, const T *a,          \
+                      size_t oa, size_t lda, T be, T *c, size_t oc, size_t ldc, hipStream_t s) {                     \
+        return clblas##L##herk(o, u, t, n, k, al.s[0], a, oa, lda, be.s[0], c, oc, ldc, s);                          \
+    }                                                                                                                \
+    clblasStatus her2k(clblasOrder o, clblasUplo u, clblasTranspose t, size_t n, size_t k, T al, const T *a,         \
+                       size_t oa, size_t lda, const T *b, size_t ob, size_t ldb, T be, T *c, size_t oc, size_t ldc,  \
+                       hipStream_t s) {                                                                              \
+        return clblas##L##her2k(o, u, t, n, k, al, a, oa, lda, b, ob, ldb, be.s[0], c, oc, ldc, s);                  \
+    }                                                                                                                \
+    clblasStatus hemm(clblasOrder o, clblasSide sd, clblasUplo u, size_t m, size_t n, T al, const T *a, size_t oa,   \
+                      size_t lda, const T *b, size_t ob, size_t ldb, T be, T *c, size_t oc, size_t ldc,              \
+                      hipStream_t s) {                                                                               \
+        return clblas##L##hemm(o, sd, u, m, n, al, a, oa, lda, b, ob, ldb, be, c, oc, ldc, s);                       \
+    }
+CLIENT_HERMITIAN(FloatComplex, C)
+CLIENT_HERMITIAN(DoubleComplex, Z)
+#undef CLIENT_HERMITIAN
+// real types: rejected in main() before any call
+template <typename T, typename... Rest> clblasStatus herk(clblasOrder, clblasUplo, clblasTranspose, size_t, size_t, T, Rest...) { return clblasNotImplemented; }
+template <typename T, typename... Rest> clblasStatus her2k(clblasOrder, clblasUplo, clblasTranspose, size_t, size_t, T, Rest...) { return clblasNotImplemented; }
+template <typename T, typename... Rest> clblasStatus hemm(clblasOrder, clblasSide, clblasUplo, size_t, size_t, T, Rest...) { return clblasNotImplemented; }
+
+enum Fn { FN_GEMM, FN_TRSM, FN_TRMM, FN_SYRK, FN_SYMM, FN_SYR2K, FN_HERK, FN_HER2K, FN_HEMM, FN_COUNT };
 
 template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t n, size_t k, bool &ok) {
     typedef typename Type<T>::Real R;
@@ -173,13 +203,14 @@ template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t 
     // shapes of A, B, C as the routine sees them
     size_t ar = m, ac = k, br = k, bc = n, cr = m, cc = n;
     int ta = o.transA, tb = o.transB;
-    if (tri || fn == FN_SYMM) { ar = ac = an; ta = 0; br = m; bc = n; tb = 0; }
-    if (fn == FN_SYRK) { ar = n; ac = k; cr = cc = n; }
+    const bool rank_k = fn == FN_SYRK || fn == FN_HERK, rank_2k = fn == FN_SYR2K || fn == FN_HER2K;
+    if (tri || fn == FN_SYMM || fn == FN_HEMM) { ar = ac = an; ta = 0; br = m; bc = n; tb = 0; }
+    if (rank_k || rank_2k) { ar = n; ac = k; cr = cc = n; br = n; bc = k; tb = ta; }
     const size_t lda = o.lda ? o.lda : tight(ta, ar, ac);
     const size_t ldb = o.ldb ? o.ldb : tight(tb, br, bc);
     const size_t ldc = o.ldc ? o.ldc : tight(0, cr, cc);
     const size_t na = footprint(o.order, ta, ar, ac, o.offA, lda);
-    const size_t nb = fn == FN_SYRK ? 1 : footprint(o.order, tb, br, bc, o.offBX, ldb);
+    const size_t nb = rank_k ? 1 : footprint(o.order, tb, br, bc, o.offBX, ldb);
     const size_t nc = (tri) ? 1 : footprint(o.order, 0, cr, cc, o.offCY, ldc);
     std::vector<R> ha(na * NC), hb(nb * NC), hc(nc * NC);
     fill(ha, 1, tri ? 1.0 / (double)an : 1.0);
@@ -215,7 +246,12 @@ template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t 
         case FN_TRSM: return trsm(ord, side, uplo, tA, diag, m, n, alpha, (const T *)da, o.offA, lda, db, o.offBX, ldb, stream);
         case FN_TRMM: return trmm(ord, side, uplo, tA, diag, m, n, alpha, da, o.offA, lda, db, o.offBX, ldb, stream);
         case FN_SYRK: return syrk(ord, uplo, tA, n, k, alpha, da, o.offA, lda, beta, dc, o.offCY, ldc, stream);
-        default: return symm(ord, side, uplo, m, n, alpha, da, o.offA, lda, db, o.offBX, ldb, beta, dc, o.offCY, ldc, stream);
+        case FN_SYMM: return symm(ord, side, uplo, m, n, alpha, da, o.offA, lda, db, o.offBX, ldb, beta, dc, o.offCY, ldc, stream);
+        case FN_SYR2K: return syr2k(ord, uplo, tA, n, k, alpha, da, o.offA, lda, db, o.offBX, ldb, beta, dc, o.offCY, ldc, stream);
+        // (const pointers: an exact match, so that the complex overloads win over the catch-all templates)
+        case FN_HERK: return herk(ord, uplo, tA, n, k, alpha, (const T *)da, o.offA, lda, beta, dc, o.offCY, ldc, stream);
+        case FN_HER2K: return her2k(ord, uplo, tA, n, k, alpha, (const T *)da, o.offA, lda, (const T *)db, o.offBX, ldb, beta, dc, o.offCY, ldc, stream);
+        default: return hemm(ord, side, uplo, m, n, alpha, (const T *)da, o.offA, lda, (const T *)db, o.offBX, ldb, beta, dc, o.offCY, ldc, stream);
         }
     };
 
@@ -239,14 +275,18 @@ template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t 
         std::sort(samples.begin(), samples.end());
         const double ns = samples[samples.size() / 2];
         // flop counts of the reference client: clfunc_xgemm.hpp:95-107,1199-1210, clfunc_xtrsm.hpp:70-92,
-        // clfunc_xtrmm.hpp:85-95,757-784, clfunc_xsyrk.hpp:65-68,588-649, clfunc_xsymm.hpp:63-69,628-645
+        // clfunc_xtrmm.hpp:85-95,757-784, clfunc_xsyrk.hpp:65-68,588-649, clfunc_xsymm.hpp:63-69,628-645,
+        // clfunc_xsyr2k.hpp:70-73,754-757, clfunc_xherk.hpp:60-63, clfunc_xher2k.hpp:65-68, clfunc_xhemm.hpp:83-93
         const double cplx = NC == 2 ? 4.0 : 1.0, M = (double)m, N = (double)n, K = (double)k;
         double flop = 0;
         switch (fn) {
         case FN_GEMM: flop = 2.0 * cplx * M * N * K; break;
         case FN_TRSM:
         case FN_TRMM: flop = cplx * (o.side == 0 ? M * (M + 1) * N : M * (N + 1) * N); break;
-        case FN_SYRK: flop = cplx * N * (N + 1) * K; break;
+        case FN_SYRK:
+        case FN_HERK: flop = cplx * N * (N + 1) * K; break;
+        case FN_SYR2K:
+        case FN_HER2K: flop = 2.0 * cplx * K * N * N + (NC == 2 ? 2.0 : 1.0) * N; break;
         default: flop = 2.0 * cplx * (o.side == 0 ? M * M * N : N * N * M); break;
         }
         gflops = flop / ns;
@@ -267,13 +307,14 @@ const char *trans_name(int t) { return t == 0 ? "none" : (t == 1 ? "transpose" :
 int main(int argc, char **argv) {
     Options o;
     if (!parse(argc, argv, o)) { usage(); return 2; }
-    const char *fnames[] = {"gemm", "trsm", "trmm", "syrk", "symm"};
+    const char *fnames[] = {"gemm", "trsm", "trmm", "syrk", "symm", "syr2k", "herk", "her2k", "hemm"};
     int fn = -1;
-    for (int i = 0; i < 5; ++i)
+    for (int i = 0; i < FN_COUNT; ++i)
         if (o.function == fnames[i]) fn = i;
     const bool real = o.precision == "s" || o.precision == "d", cplx = o.precision == "c" || o.precision == "z";
-    if (fn < 0 || !(real || cplx)) {
-        std::fprintf(stderr, "this library implements -f gemm|trsm|trmm|syrk|symm with -r s|d|c|z\n");
+    if (fn < 0 || !(real || cplx) || (real && fn >= FN_HERK)) {
+        std::fprintf(stderr, "this library implements -f gemm|trsm|trmm|syrk|symm|syr2k with -r s|d|c|z and "
+                             "-f herk|her2k|hemm with -r c|z\n");
         return 2;
     }
     if (clblasSetup() != clblasSuccess) { std::fprintf(stderr, "clblasSetup failed (needs a gfx950 device)\n"); return 1; }

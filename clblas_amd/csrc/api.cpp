@@ -226,7 +226,7 @@ clblasStatus trmm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clb
 // SYMM front end.  Checks as doSymm (src/library/blas/xsymm.c:50-71): objects A, B, C; A is
 // M x M (left) or N x N (right); B and C are M x N.  Row major swaps M and N and flips side
 // and triangle (xsymm.c:104-124).
-template <typename T>
+template <typename T, bool HERM = false>
 clblasStatus symm_front(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, T alpha, const T *A,
                         size_t offA, size_t lda, const T *B, size_t offB, size_t ldb, T beta, T *C, size_t offC,
                         size_t ldc, hipStream_t stream) {
@@ -248,8 +248,72 @@ clblasStatus symm_front(clblasOrder order, clblasSide side, clblasUplo uplo, siz
         right = !right;
         lower = !lower;
     }
-    return map_hip_error(cba::symm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda, B + offB,
-                                               (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+    if constexpr (HERM)  // HEMM goes through doSymm as well (xhemm.c:69-73), same checks and folding
+        return map_hip_error(cba::hemm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
+                                                   B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+    else
+        return map_hip_error(cba::symm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
+                                                   B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+}
+
+// SYR2K front end.  Checks as doSyr2k (src/library/blas/xsyr2k.c:58-76): objects A, B, C;
+// ConjTrans is invalid for complex types; A and B are N x K, C is N x N.  Row-major folding as
+// for SYRK.
+template <typename T>
+clblasStatus syr2k_front(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K, T alpha,
+                         const T *A, size_t offA, size_t lda, const T *B, size_t offB, size_t ldb, T beta, T *C,
+                         size_t offC, size_t ldc, hipStream_t stream) {
+    if (!A) return clblasInvalidMatA;
+    if (!B) return clblasInvalidMatB;
+    if (!C) return clblasInvalidMatC;
+    if (!valid_order(order) || !valid_trans(transAB) || (uplo != clblasUpper && uplo != clblasLower))
+        return clblasInvalidValue;
+    if (IsComplex<T>::value && transAB == clblasConjTrans) return clblasInvalidValue;
+    clblasStatus st;
+    if ((st = check_matrix_sizes(order, transAB, N, K, lda, MAT_A)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, transAB, N, K, ldb, MAT_B)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if (N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
+    bool lower = uplo == clblasLower, trans = transAB != clblasNoTrans;
+    if (order == clblasRowMajor) {
+        lower = !lower;
+        trans = !trans;
+    }
+    return map_hip_error(cba::syr2k_colmajor<T>(lower, trans, (int)N, (int)K, alpha, A + offA, (int64_t)lda, B + offB,
+                                                (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+}
+
+// HERK / HER2K front end (B == nullptr with `two` false: HERK).  Checks as doHerk / doHer2k
+// (src/library/blas/xherk.c:64-84, xher2k.c:73-97): objects; plain Trans is invalid; A (and B)
+// N x K, C N x N.  Row major (xherk.c:88-89, xher2k.c:99-100, 192-195): the same memory read
+// column-major holds the transposes, so flip the triangle, swap NoTrans <-> ConjTrans and
+// conjugate alpha.
+template <typename R>
+clblasStatus herk_front(bool two, clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
+                        cba::Cx<R> alpha, const cba::Cx<R> *A, size_t offA, size_t lda, const cba::Cx<R> *B,
+                        size_t offB, size_t ldb, R beta, cba::Cx<R> *C, size_t offC, size_t ldc, hipStream_t stream) {
+    if (!A) return clblasInvalidMatA;
+    if (two && !B) return clblasInvalidMatB;
+    if (!C) return clblasInvalidMatC;
+    if (!valid_order(order) || !valid_trans(trans) || (uplo != clblasUpper && uplo != clblasLower))
+        return clblasInvalidValue;
+    if (trans == clblasTrans) return clblasInvalidValue;
+    clblasStatus st;
+    if ((st = check_matrix_sizes(order, trans, N, K, lda, MAT_A)) != clblasSuccess) return st;
+    if (two && (st = check_matrix_sizes(order, trans, N, K, ldb, MAT_B)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if (N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
+    bool lower = uplo == clblasLower, ctrans = trans != clblasNoTrans;
+    if (order == clblasRowMajor) {
+        lower = !lower;
+        ctrans = !ctrans;
+        alpha.im = -alpha.im;
+    }
+    if (!two)
+        return map_hip_error(cba::herk_colmajor<R>(lower, ctrans, (int)N, (int)K, alpha.re, A + offA, (int64_t)lda,
+                                                   beta, C + offC, (int64_t)ldc, stream));
+    return map_hip_error(cba::her2k_colmajor<R>(lower, ctrans, (int)N, (int)K, alpha, A + offA, (int64_t)lda,
+                                                B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
 }
 
 static_assert(sizeof(FloatComplex) == sizeof(cba::Cx<float>) && sizeof(DoubleComplex) == sizeof(cba::Cx<double>),
@@ -455,6 +519,72 @@ clblasStatus clblasZsymm(clblasOrder order, clblasSide side, clblasUplo uplo, si
                          const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta, DoubleComplex *C,
                          size_t offC, size_t ldc, hipStream_t stream) {
     return symm_front<cba::Cx<double>>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasSsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          float alpha, const float *A, size_t offA, size_t lda, const float *B, size_t offB, size_t ldb,
+                          float beta, float *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syr2k_front<float>(order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasDsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          double alpha, const double *A, size_t offA, size_t lda, const double *B, size_t offB, size_t ldb,
+                          double beta, double *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syr2k_front<double>(order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
+}
+
+clblasStatus clblasCsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb,
+                          FloatComplex beta, FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syr2k_front<cba::Cx<float>>(order, uplo, transAB, N, K, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasZsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb,
+                          DoubleComplex beta, DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syr2k_front<cba::Cx<double>>(order, uplo, transAB, N, K, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasCherk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, float alpha,
+                         const FloatComplex *A, size_t offA, size_t lda, float beta, FloatComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return herk_front<float>(false, order, uplo, transA, N, K, cba::Cx<float>{alpha, 0}, reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, nullptr, 0, 0, beta,
+                          reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasCher2k(clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
+                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb,
+                          float beta, FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return herk_front<float>(true, order, uplo, trans, N, K, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, beta,
+                          reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasChemm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, FloatComplex alpha,
+                         const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta,
+                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return symm_front<cba::Cx<float>, true>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, cx(beta),
+                                reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasZherk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, double alpha,
+                         const DoubleComplex *A, size_t offA, size_t lda, double beta, DoubleComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return herk_front<double>(false, order, uplo, transA, N, K, cba::Cx<double>{alpha, 0}, reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, nullptr, 0, 0, beta,
+                          reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasZher2k(clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
+                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb,
+                          double beta, DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return herk_front<double>(true, order, uplo, trans, N, K, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, beta,
+                          reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+}
+
+clblasStatus clblasZhemm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, DoubleComplex alpha,
+                         const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
+                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return symm_front<cba::Cx<double>, true>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, cx(beta),
+                                reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
 }
 
 }  // extern "C"

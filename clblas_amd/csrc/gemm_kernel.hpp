@@ -81,6 +81,10 @@ template <typename R> __device__ __forceinline__ Cx<R> el_scale(Cx<R> alpha, Cx<
     im = fma(alpha.im, x.re, im);
     return Cx<R>{re, im};
 }
+// x with its imaginary part dropped (x itself for real types)
+__device__ __forceinline__ float el_real_only(float x) { return x; }
+__device__ __forceinline__ double el_real_only(double x) { return x; }
+template <typename R> __device__ __forceinline__ Cx<R> el_real_only(Cx<R> x) { return Cx<R>{x.re, (R)0}; }
 // r + beta * c
 __device__ __forceinline__ float el_axpy(float beta, float c, float r) { return r + beta * c; }
 __device__ __forceinline__ double el_axpy(double beta, double c, double r) { return r + beta * c; }
@@ -193,10 +197,12 @@ template <typename T> struct GemmParams {
     //          wholly outside it are not enumerated at all (grid = number of active tiles).
     //   tri_a / tri_b: op(A)(m,k) / op(B)(k,n) is triangular: elements with k > x (1) or
     //          k < x (2), x = m resp. n, count as zero whatever memory holds; unit_* = 1: the
-    //          diagonal k == x counts as one, 2: as zero.  Panels outside the triangle are
-    //          skipped.
+    //          diagonal k == x counts as one, 2: as zero, 3: as its real part.  Panels outside
+    //          the triangle are skipped.
+    //   herm_c (with tri_c, complex types): the diagonal of C is read and stored with a zero
+    //          imaginary part.
     //   rev_m / rev_n: walk the tile rows / columns from the far end (longest tiles first).
-    int tri_c, tri_a, tri_b, unit_a, unit_b, rev_m, rev_n;
+    int tri_c, tri_a, tri_b, unit_a, unit_b, rev_m, rev_n, herm_c;
     // Sliced tail (TRI kernels only): the last tiles of the list - those of the final, partly
     // filled round of 256 CUs - are each cut into `tail_slices` K ranges of `tail_kps`, so that
     // the round lasts 1/tail_slices as long.  Workgroup ids from `tail_first` on are slices
@@ -357,6 +363,7 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
             const bool keep = mode == 1 ? kg <= xg : kg >= xg;
             if (!keep || (unit == 2 && kg == xg)) v = T();
             else if (unit == 1 && kg == xg) v = el_one<T>();
+            else if (unit == 3 && kg == xg) v = el_real_only(v);
         };
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
@@ -704,6 +711,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         beta = T();
     }
     int tri_c = TRI ? p.tri_c : 0;
+    bool herm_c = TRI && p.herm_c;  // Hermitian C: diagonal elements are stored with a zero imaginary part
     if (TRI && slice >= 0) {
         // partial tile, tile-local coordinates, finished by tail_reduce_kernel
         const int u = (int)blockIdx.x - p.tail_first;
@@ -713,6 +721,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         alpha = el_one<T>();
         beta = T();
         tri_c = 0;
+        herm_c = false;
     }
     const bool read_c = !el_is_zero(beta);
     const bool neg_im = CPLX && p.conj_b;  // Im = sB * Im'
@@ -763,7 +772,13 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 #pragma unroll
                         for (int e = 0; e < VM; ++e) {
                             T r = el_scale(alpha, acc_elem(bn, ga * VM + e, v));
-                            if (read_c) r = el_axpy(beta, VC::get(cold[dv][ga], e), r);
+                            if (TRI && CPLX && herm_c && m + e == n) {
+                                // the stored imaginary part of a Hermitian diagonal is not part of the matrix
+                                if (read_c) r = el_axpy(beta, el_real_only(VC::get(cold[dv][ga], e)), r);
+                                r = el_real_only(r);
+                            } else if (read_c) {
+                                r = el_axpy(beta, VC::get(cold[dv][ga], e), r);
+                            }
                             VC::set(ov, e, r);
                         }
                         *reinterpret_cast<UV *>(col + m) = ov;
@@ -773,7 +788,12 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                             const bool kept = !(TRI && tri_c) || (tri_c == 1 ? m + e >= n : m + e <= n);
                             if (m + e < p.M && kept) {
                                 T r = el_scale(alpha, acc_elem(bn, ga * VM + e, v));
-                                if (read_c) r = el_axpy(beta, col[m + e], r);
+                                if (TRI && CPLX && herm_c && m + e == n) {
+                                    if (read_c) r = el_axpy(beta, el_real_only(col[m + e]), r);
+                                    r = el_real_only(r);
+                                } else if (read_c) {
+                                    r = el_axpy(beta, col[m + e], r);
+                                }
                                 col[m + e] = r;
                             }
                         }
@@ -819,7 +839,9 @@ __global__ void __launch_bounds__(256) tail_reduce_kernel(const GemmParams<T> p,
     for (int i = 0; i < p.tail_slices; ++i) s = el_add(s, w[(int64_t)i * (bm * bn)]);
     T *c = p.C + (int64_t)n * p.ldc + m;
     T v = el_scale(p.alpha, s);
-    if (!el_is_zero(p.beta)) v = el_axpy(p.beta, *c, v);
+    const bool herm_diag = p.herm_c && m == n;
+    if (!el_is_zero(p.beta)) v = el_axpy(p.beta, herm_diag ? el_real_only(*c) : *c, v);
+    if (herm_diag) v = el_real_only(v);
     *c = v;
 }
 

@@ -200,7 +200,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     p.xcd_remap = debug_env_int("CLBLAS_AMD_GEMM_XCD", 1);
     p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
     p.k_per_split = K;
-    p.tri_c = p.tri_a = p.tri_b = p.unit_a = p.unit_b = p.rev_m = p.rev_n = 0;
+    p.tri_c = p.tri_a = p.tri_b = p.unit_a = p.unit_b = p.rev_m = p.rev_n = p.herm_c = 0;
     p.tail_first = 0; p.tail_slices = 1; p.tail_kps = K;
     const int idx = (tA ? 2 : 0) | (tB ? 1 : 0);
     int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n;
@@ -212,6 +212,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         fn = e.tri[idx];
         p.tri_c = tri->tri_c; p.tri_a = tri->tri_a; p.tri_b = tri->tri_b;
         p.unit_a = tri->unit_a; p.unit_b = tri->unit_b;
+        p.herm_c = tri->herm_c;
         if (p.tri_c) ntiles = active_tiles(M, N, e.bm, e.bn, p.tri_c);  // the kernel enumerates the same set
         if (p.tri_a || p.tri_b) {
             // Tiles differ in depth (by tile row for a triangular A, by tile column for B):

@@ -34,9 +34,11 @@ hipError_t ensure_dynamic_lds(const void *fn, size_t bytes);
 //   tri_c: only the lower (1) / upper (2) triangle of C is computed and stored.
 //   tri_a / tri_b: op(A)(m,k) / op(B)(k,n) is triangular: entries with k > x (1) or k < x (2),
 //   x = m resp. n, count as zero whatever memory holds; unit_* = 1: the diagonal counts as
-//   one, 2: as zero (strict triangle).
+//   one, 2: as zero (strict triangle), 3: as its real part (diagonal of a Hermitian matrix).
+//   herm_c (with tri_c, complex types): C is Hermitian, its diagonal is stored with zero
+//   imaginary parts.
 struct GemmTri {
-    int tri_c = 0, tri_a = 0, tri_b = 0, unit_a = 0, unit_b = 0;
+    int tri_c = 0, tri_a = 0, tri_b = 0, unit_a = 0, unit_b = 0, herm_c = 0;
     bool any() const { return tri_c || tri_a || tri_b; }
 };
 
@@ -77,6 +79,23 @@ hipError_t trmm_colmajor(bool right, bool lower, bool trans, bool conj, bool uni
 template <typename T>
 hipError_t symm_colmajor(bool right, bool lower, int M, int N, T alpha, const T *A, int64_t lda, const T *B,
                          int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream);
+// syr2k: C <- alpha (op(A) op(B)^T + op(B) op(A)^T) + beta C on one triangle of C.
+template <typename T>
+hipError_t syr2k_colmajor(bool lower, bool trans, int N, int K, T alpha, const T *A, int64_t lda, const T *B,
+                          int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream);
+// herk: C <- alpha op(A) op(A)^H + beta C; her2k: C <- alpha op(A) op(B)^H + conj(alpha) op(B) op(A)^H
+// + beta C; op = identity or conjugate transpose (`ctrans`), real beta (and alpha for herk), C Hermitian.
+template <typename R>
+hipError_t herk_colmajor(bool lower, bool ctrans, int N, int K, R alpha, const Cx<R> *A, int64_t lda, R beta,
+                         Cx<R> *C, int64_t ldc, hipStream_t stream);
+template <typename R>
+hipError_t her2k_colmajor(bool lower, bool ctrans, int N, int K, Cx<R> alpha, const Cx<R> *A, int64_t lda,
+                          const Cx<R> *B, int64_t ldb, R beta, Cx<R> *C, int64_t ldc, hipStream_t stream);
+// hemm: as symm with A Hermitian (complex types).
+template <typename T>
+hipError_t hemm_colmajor(bool right, bool lower, int M, int N, T alpha, const T *A, int64_t lda, const T *B,
+                         int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream);
+
 
 // Column-major TRSM driver (trsm.hip), all four types: solves op(A) X = alpha B (left) or
 // X op(A) = alpha B (right) in place; `conj` conjugates op(A) (complex, clblasConjTrans).

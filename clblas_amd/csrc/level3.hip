@@ -1,4 +1,4 @@
-// SYRK, TRMM and SYMM as GEMM-shaped calls on the MFMA GEMM core.
+// SYRK, SYR2K, HERK, HER2K, TRMM, SYMM and HEMM as GEMM-shaped calls on the MFMA GEMM core.
 //
 // The reference runs these through its generated solver kernels (src/library/blas/xsyrk.c,
 // xtrmm.c, xsymm.c; xsymm.c:150-330 already composes SYMM from GEMM passes).  Here each is
@@ -10,6 +10,12 @@
 //   SYMM  A = T + S^T with T the stored triangle and S its strict part:
 //         C <- alpha T B + beta C, then C <- alpha S^T B + C (two half-depth launches, no
 //         workspace).
+//   SYR2K two SYRK-shaped launches (A B^T, then B A^T accumulated).
+//   HERK / HER2K  the same with the second operand conjugate-transposed; the diagonal of C is
+//         stored with zero imaginary parts (the reference does this in its GEMM epilogue,
+//         src/library/blas/gens/clTemplates/gemm.cl:1034-1056; xherk.c:88-110, xher2k.c:96-149).
+//   HEMM  as SYMM with a conjugated mirror pass; the stored diagonal counts with its real
+//         part only (xhemm.c:36-112 -> doSymm).
 #include "gemm_kernel.hpp"
 #include "internal.h"
 
@@ -109,16 +115,96 @@ hipError_t symm_colmajor(bool right, bool lower, int M, int N, T alpha, const T 
                           &mirrored);
 }
 
+template <typename T>
+hipError_t syr2k_colmajor(bool lower, bool trans, int N, int K, T alpha, const T *A, int64_t lda, const T *B,
+                          int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream) {
+    GemmTri tri;
+    tri.tri_c = lower ? 1 : 2;
+    // C <- alpha op(A) op(B)^T + beta C, then C <- alpha op(B) op(A)^T + C
+    hipError_t err =
+        launch_gemm<T>(trans, !trans, false, false, N, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, &tri);
+    if (err != hipSuccess) return err;
+    return launch_gemm<T>(trans, !trans, false, false, N, N, K, alpha, B, ldb, A, lda, el_one<T>(), C, ldc, stream,
+                          &tri);
+}
+
+template <typename R>
+hipError_t herk_colmajor(bool lower, bool ctrans, int N, int K, R alpha, const Cx<R> *A, int64_t lda, R beta,
+                         Cx<R> *C, int64_t ldc, hipStream_t stream) {
+    typedef Cx<R> T;
+    GemmTri tri;
+    tri.tri_c = lower ? 1 : 2;
+    tri.herm_c = 1;
+    // A A^H (second operand conjugate-transposed) or A^H A (first operand)
+    return launch_gemm<T>(ctrans, !ctrans, ctrans, !ctrans, N, N, K, T{alpha, (R)0}, A, lda, A, lda, T{beta, (R)0}, C,
+                          ldc, stream, &tri);
+}
+
+template <typename R>
+hipError_t her2k_colmajor(bool lower, bool ctrans, int N, int K, Cx<R> alpha, const Cx<R> *A, int64_t lda,
+                          const Cx<R> *B, int64_t ldb, R beta, Cx<R> *C, int64_t ldc, hipStream_t stream) {
+    typedef Cx<R> T;
+    GemmTri tri;
+    tri.tri_c = lower ? 1 : 2;
+    tri.herm_c = 1;
+    // C <- alpha op(A) op(B)^H + beta C, then C <- conj(alpha) op(B) op(A)^H + C
+    // (the two passes of xher2k.c:117-149)
+    hipError_t err = launch_gemm<T>(ctrans, !ctrans, ctrans, !ctrans, N, N, K, alpha, A, lda, B, ldb, T{beta, (R)0}, C,
+                                    ldc, stream, &tri);
+    if (err != hipSuccess) return err;
+    return launch_gemm<T>(ctrans, !ctrans, ctrans, !ctrans, N, N, K, T{alpha.re, -alpha.im}, B, ldb, A, lda,
+                          el_one<T>(), C, ldc, stream, &tri);
+}
+
+template <typename T>
+hipError_t hemm_colmajor(bool right, bool lower, int M, int N, T alpha, const T *A, int64_t lda, const T *B,
+                         int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream) {
+    // As SYMM, with A = T + S^H: the mirrored pass conjugates, and the diagonal of the stored
+    // triangle counts with its real part only.
+    GemmTri stored, mirrored;
+    hipError_t err;
+    if (!right) {
+        stored.tri_a = lower ? 1 : 2;
+        stored.unit_a = 3;
+        mirrored.tri_a = lower ? 2 : 1;
+        mirrored.unit_a = 2;
+        err = launch_gemm<T>(false, false, false, false, M, N, M, alpha, A, lda, B, ldb, beta, C, ldc, stream, &stored);
+        if (err != hipSuccess) return err;
+        return launch_gemm<T>(true, false, true, false, M, N, M, alpha, A, lda, B, ldb, el_one<T>(), C, ldc, stream,
+                              &mirrored);
+    }
+    stored.tri_b = lower ? 2 : 1;
+    stored.unit_b = 3;
+    mirrored.tri_b = lower ? 1 : 2;
+    mirrored.unit_b = 2;
+    err = launch_gemm<T>(false, false, false, false, M, N, N, alpha, B, ldb, A, lda, beta, C, ldc, stream, &stored);
+    if (err != hipSuccess) return err;
+    return launch_gemm<T>(false, true, false, true, M, N, N, alpha, B, ldb, A, lda, el_one<T>(), C, ldc, stream,
+                          &mirrored);
+}
+
 #define CBA_INSTANTIATE(T)                                                                                         \
     template hipError_t syrk_colmajor<T>(bool, bool, int, int, T, const T *, int64_t, T, T *, int64_t, hipStream_t); \
     template hipError_t trmm_colmajor<T>(bool, bool, bool, bool, bool, int, int, T, const T *, int64_t, T *, int64_t, \
                                          hipStream_t);                                                             \
     template hipError_t symm_colmajor<T>(bool, bool, int, int, T, const T *, int64_t, const T *, int64_t, T, T *,   \
-                                         int64_t, hipStream_t);
+                                         int64_t, hipStream_t);                                                    \
+    template hipError_t syr2k_colmajor<T>(bool, bool, int, int, T, const T *, int64_t, const T *, int64_t, T, T *,  \
+                                          int64_t, hipStream_t);
 CBA_INSTANTIATE(float)
 CBA_INSTANTIATE(double)
 CBA_INSTANTIATE(Cx<float>)
 CBA_INSTANTIATE(Cx<double>)
 #undef CBA_INSTANTIATE
+#define CBA_INSTANTIATE_HERM(R)                                                                                     \
+    template hipError_t herk_colmajor<R>(bool, bool, int, int, R, const Cx<R> *, int64_t, R, Cx<R> *, int64_t,       \
+                                         hipStream_t);                                                              \
+    template hipError_t her2k_colmajor<R>(bool, bool, int, int, Cx<R>, const Cx<R> *, int64_t, const Cx<R> *,       \
+                                          int64_t, R, Cx<R> *, int64_t, hipStream_t);                               \
+    template hipError_t hemm_colmajor<Cx<R>>(bool, bool, int, int, Cx<R>, const Cx<R> *, int64_t, const Cx<R> *,    \
+                                             int64_t, Cx<R>, Cx<R> *, int64_t, hipStream_t);
+CBA_INSTANTIATE_HERM(float)
+CBA_INSTANTIATE_HERM(double)
+#undef CBA_INSTANTIATE_HERM
 
 }  // namespace cba

@@ -175,7 +175,7 @@ clblasStatus clblasZtrsm(clblasOrder order, clblasSide side, clblasUplo uplo,
                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
                          DoubleComplex *B, size_t offB, size_t ldb, hipStream_t stream);
 
-/* ---- GEMM-shaped neighbours on the same MFMA core: SYRK, TRMM, SYMM (all four types) ---- */
+/* ---- GEMM-shaped neighbours on the same MFMA core: SYRK, TRMM, SYMM, SYR2K (all four types), HERK, HER2K, HEMM ---- */
 
 /* Replace clblas{S,D,C,Z}syrk (src/clBLAS.h:8278-8503, src/library/blas/xsyrk.c:27-233).
  *   C <- alpha * op(A) * op(A)^T + beta * C, C is N x N and only its `uplo` triangle is read
@@ -238,6 +238,64 @@ clblasStatus clblasZsymm(clblasOrder order, clblasSide side, clblasUplo uplo, si
                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
                          const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
                          DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9123-9145 */
+
+/* Replace clblas{S,D,C,Z}syr2k (src/clBLAS.h:8568-8819, src/library/blas/xsyr2k.c:27-251).
+ *   C <- alpha * (op(A) * op(B)^T + op(B) * op(A)^T) + beta * C on the `uplo` triangle of the
+ * N x N matrix C; op(A), op(B) are N x K.  Validation follows doSyr2k (xsyr2k.c:58-76): null
+ * A/B/C, clblasConjTrans with a complex type -> clblasInvalidValue, sizes of A, B, then C. */
+clblasStatus clblasSsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          float alpha, const float *A, size_t offA, size_t lda,
+                          const float *B, size_t offB, size_t ldb, float beta,
+                          float *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8568-8589 */
+clblasStatus clblasDsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          double alpha, const double *A, size_t offA, size_t lda,
+                          const double *B, size_t offB, size_t ldb, double beta,
+                          double *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8648-8669 */
+clblasStatus clblasCsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                          const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta,
+                          FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8722-8743 */
+clblasStatus clblasZsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
+                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                          const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
+                          DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:8798-8819 */
+
+/* Replace clblas{C,Z}herk (src/clBLAS.h:9389-9476, src/library/blas/xherk.c:132-210).
+ *   C <- alpha * op(A) * op(A)^H + beta * C, alpha and beta real, C Hermitian N x N: only its
+ * `uplo` triangle is read or written, imaginary parts of its diagonal are ignored on input and
+ * stored as zero.  transA is NoTrans or ConjTrans; Trans is rejected with clblasInvalidValue, xherk.c:69-71. */
+clblasStatus clblasCherk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         float alpha, const FloatComplex *A, size_t offA, size_t lda, float beta,
+                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9389-9407 */
+clblasStatus clblasZherk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
+                         double alpha, const DoubleComplex *A, size_t offA, size_t lda, double beta,
+                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9458-9476 */
+
+/* Replace clblas{C,Z}her2k (src/clBLAS.h:9545-9644, src/library/blas/xher2k.c:155-245).
+ *   C <- alpha * op(A) * op(B)^H + conj(alpha) * op(B) * op(A)^H + beta * C, beta real, C
+ * Hermitian as for herk.  Validation follows doHer2k (xher2k.c:73-97). */
+clblasStatus clblasCher2k(clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
+                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                          const FloatComplex *B, size_t offB, size_t ldb, float beta,
+                          FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9545-9566 */
+clblasStatus clblasZher2k(clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
+                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                          const DoubleComplex *B, size_t offB, size_t ldb, double beta,
+                          DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9623-9644 */
+
+/* Replace clblas{C,Z}hemm (src/clBLAS.h:9224-9326, src/library/blas/xhemm.c:36-112).
+ *   side == Left : C <- alpha * A * B + beta * C,  A Hermitian M x M
+ *   side == Right: C <- alpha * B * A + beta * C,  A Hermitian N x N
+ * Only the `uplo` triangle of A is read; imaginary parts of its diagonal are ignored.
+ * Validation and row-major folding are SYMM's (xhemm.c:69-73 -> doSymm, xsymm.c:50-124). */
+clblasStatus clblasChemm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N,
+                         FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                         const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta,
+                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9224-9245 */
+clblasStatus clblasZhemm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N,
+                         DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                         const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
+                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9305-9326 */
 
 #ifdef __cplusplus
 }

@@ -75,6 +75,19 @@ def lib():
             f = getattr(L, "oracle_%ssymm" % t)
             f.restype = _i
             f.argtypes = [_i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _sz, _sz]
+            f = getattr(L, "oracle_%ssyr2k" % t)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _sz, _sz]
+        for t, real in (("c", ctypes.c_float), ("z", ctypes.c_double)):
+            f = getattr(L, "oracle_%sherk" % t)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, real, _vp, _sz, _sz, real, _vp, _sz, _sz]
+            f = getattr(L, "oracle_%sher2k" % t)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz, real, _vp, _sz, _sz]
+            f = getattr(L, "oracle_%shemm" % t)
+            f.restype = _i
+            f.argtypes = [_i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _sz, _sz]
         L.oracle_check_gemm.restype = _i
         L.oracle_check_gemm.argtypes = [_i, _i, _i, _sz, _sz, _sz, _i, _sz, _sz, _sz, _i, _sz, _sz, _sz, _i, _sz,
                                         _sz, _sz]
@@ -115,6 +128,8 @@ def ref_lib():
             f.argtypes = [_i, _i, _i, _sz, _sz, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz]
         L.ref_naive_syrk.restype = None
         L.ref_naive_syrk.argtypes = [_i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _vp, _sz]
+        L.ref_naive_syr2k.restype = None
+        L.ref_naive_syr2k.argtypes = [_i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _sz, _vp, _vp, _sz]
         L.ref_naive_trmm.restype = None
         L.ref_naive_trmm.argtypes = [_i, _i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _vp, _sz]
         L.ref_naive_trsm.restype = None
@@ -237,6 +252,42 @@ def symm(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, of
     al, be = _sc(alpha, ref), _sc(beta, ref)
     return getattr(lib(), "oracle_%ssymm" % prefix(ref))(int(order), int(side), int(uplo), M, N, _p(al), _p(A), offA,
                                                          lda, _p(B), offB, ldb, _p(be), _p(C), offC, ldc)
+
+
+def syr2k(order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    ref = C if C is not None else (A if A is not None else B)
+    al, be = _sc(alpha, ref), _sc(beta, ref)
+    return getattr(lib(), "oracle_%ssyr2k" % prefix(ref))(int(order), int(uplo), int(transAB), N, K, _p(al), _p(A),
+                                                          offA, lda, _p(B), offB, ldb, _p(be), _p(C), offC, ldc)
+
+
+def herk(order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc):
+    """alpha, beta real; A, C complex64 / complex128."""
+    ref = C if C is not None else A
+    return getattr(lib(), "oracle_%sherk" % prefix(ref))(int(order), int(uplo), int(transA), N, K, float(alpha), _p(A),
+                                                         offA, lda, float(beta), _p(C), offC, ldc)
+
+
+def her2k(order, uplo, trans, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    """alpha complex, beta real."""
+    ref = C if C is not None else (A if A is not None else B)
+    return getattr(lib(), "oracle_%sher2k" % prefix(ref))(int(order), int(uplo), int(trans), N, K,
+                                                          _p(_sc(alpha, ref)), _p(A), offA, lda, _p(B), offB, ldb,
+                                                          float(beta), _p(C), offC, ldc)
+
+
+def hemm(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    ref = C if C is not None else (A if A is not None else B)
+    al, be = _sc(alpha, ref), _sc(beta, ref)
+    return getattr(lib(), "oracle_%shemm" % prefix(ref))(int(order), int(side), int(uplo), M, N, _p(al), _p(A), offA,
+                                                         lda, _p(B), offB, ldb, _p(be), _p(C), offC, ldc)
+
+
+def ref_syr2k(order, uplo, transAB, N, K, alpha, A, lda, B, ldb, beta, C, ldc):
+    """Reference naive syr2k (no offsets)."""
+    al, be = _sc(alpha, C), _sc(beta, C)
+    ref_lib().ref_naive_syr2k("sdcz".index(prefix(C)), int(order), int(uplo), int(transAB), N, K, _p(al), _p(A), lda,
+                              _p(B), ldb, _p(be), _p(C), ldc)
 
 
 def ref_syrk(order, uplo, transA, N, K, alpha, A, lda, beta, C, ldc):

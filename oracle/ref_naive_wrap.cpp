@@ -93,6 +93,13 @@ void ref_naive_syrk(int type, int order, int uplo, int trans, size_t N, size_t K
                                      lda, ref_scalar<T, R>(beta), (T *)C, ldc)))
 }
 
+void ref_naive_syr2k(int type, int order, int uplo, int trans, size_t N, size_t K, const void *alpha, const void *A,
+                     size_t lda, const void *B, size_t ldb, const void *beta, void *C, size_t ldc) {
+    REF_DISPATCH((NaiveBlas::syr2k<T>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasUplo)uplo,
+                                      (NaiveBlas::clblasTranspose)trans, N, K, ref_scalar<T, R>(alpha), (const T *)A,
+                                      lda, (const T *)B, ldb, ref_scalar<T, R>(beta), (T *)C, ldc)))
+}
+
 void ref_naive_trmm(int type, int order, int side, int uplo, int trans, int diag, size_t M, size_t N,
                     const void *alpha, const void *A, size_t lda, void *B, size_t ldb) {
     REF_DISPATCH((NaiveBlas::trmm<T>((NaiveBlas::clblasOrder)order, (NaiveBlas::clblasSide)side,

@@ -18,6 +18,14 @@ Sources of the INPUT DATA (data only; no reference code is run or copied):
                                 alpha=10, beta=20, upper triangle of A filled with -1
   * src/samples/example_ssyrk.c:30-63,142-144  row-major SSYRK upper/notrans, sub-problem
                                 (N-1, K-1) at offA=K+1, offC=N+1, alpha=10, beta=20
+  * src/samples/example_ssyr2k.c:30-73,156-159  row-major SSYR2K upper/notrans, sub-problem (N-1, K-1) at
+                                offA=offB=K+1, offC=N+1, alpha=10, beta=20, B == A
+  * src/samples/example_cherk.cpp:30-68,152-154  column-major CHERK lower/notrans, N=5, K=4, A all ones
+                                (lda=5), alpha=10, beta=1, C lower triangle with non-zero imaginary diagonal
+  * src/samples/example_cher2k.c:30-67,153-154  column-major CHER2K lower/notrans, alpha=(10,1), beta=1,
+                                the same C
+  * src/samples/example_chemm.cpp:30-64,146-148  row-major CHEMM left/lower, M=4, N=3, alpha=(10,10),
+                                beta=(20,20), complex diagonal of A, upper triangle filled with (-1,-1)
   * src/samples/example_strmm.c:30-63,140-142  row-major STRMM left/upper/notrans/nonunit,
                                 sub-problem (M-1, N-1) at offA=M+1, offB=N+1, alpha=10
 
@@ -152,6 +160,104 @@ def symm_exact(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta,
     return out
 
 
+class G:
+    """Gaussian integer / rational: exact complex arithmetic on Fractions."""
+
+    def __init__(self, re, im=0):
+        self.re, self.im = F(re), F(im)
+
+    @staticmethod
+    def of(x):
+        return x if isinstance(x, G) else (G(x[0], x[1]) if isinstance(x, (list, tuple)) else G(x))
+
+    def __add__(self, o):
+        o = G.of(o)
+        return G(self.re + o.re, self.im + o.im)
+
+    def __mul__(self, o):
+        o = G.of(o)
+        return G(self.re * o.re - self.im * o.im, self.re * o.im + self.im * o.re)
+
+    def conj(self):
+        return G(self.re, -self.im)
+
+    def pair(self):
+        return [float(self.re), float(self.im)]
+
+
+def gsum(terms):
+    s = G(0)
+    for t in terms:
+        s = s + t
+    return s
+
+
+def syr2k_exact(order, uplo, tAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    out = [F(x) for x in C]
+    a = lambda i, k: F(A[offA + a_index(order, tAB, i, k, lda)])
+    b = lambda i, k: F(B[offB + a_index(order, tAB, i, k, ldb)])
+    for i in range(N):
+        for j in range(N):
+            if not ((i <= j) if uplo == UPPER else (i >= j)):
+                continue
+            s = sum(a(i, k) * b(j, k) + b(i, k) * a(j, k) for k in range(K))
+            ci = offC + a_index(order, N_, i, j, ldc)
+            out[ci] = F(alpha) * s + F(beta) * F(C[ci])
+    return out
+
+
+def her2k_exact(order, uplo, trans, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    """C = alpha op(A) op(B)^H + conj(alpha) op(B) op(A)^H + beta C on one triangle, op = identity
+    (trans == N_) or conjugate transpose; diagonal real.  B is None: herk, C = alpha op(A) op(A)^H + beta C
+    with real alpha."""
+    def el(X, off, ld, i, k):   # op(X)(i, k)
+        v = G.of(X[off + a_index(order, N_ if trans == N_ else T_, i, k, ld)])
+        return v if trans == N_ else v.conj()
+    out = [G.of(x) for x in C]
+    al = G.of(alpha)
+    for i in range(N):
+        for j in range(N):
+            if not ((i <= j) if uplo == UPPER else (i >= j)):
+                continue
+            if B is None:
+                s = al * gsum(el(A, offA, lda, i, k) * el(A, offA, lda, j, k).conj() for k in range(K))
+            else:
+                s = al * gsum(el(A, offA, lda, i, k) * el(B, offB, ldb, j, k).conj() for k in range(K)) + \
+                    al.conj() * gsum(el(B, offB, ldb, i, k) * el(A, offA, lda, j, k).conj() for k in range(K))
+            ci = offC + a_index(order, N_, i, j, ldc)
+            c0 = G.of(C[ci])
+            if i == j:
+                c0 = G(c0.re, 0)
+            r = s + G(beta) * c0
+            out[ci] = G(r.re, 0) if i == j else r
+    return out
+
+
+def hemm_exact(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc):
+    n = M if side == LEFT else N
+
+    def a(r, c):  # Hermitian element from the stored triangle; stored diagonal imaginary parts ignored
+        if r == c:
+            return G(G.of(A[offA + a_index(order, N_, r, c, lda)]).re, 0)
+        if (r <= c) if uplo == UPPER else (r >= c):
+            return G.of(A[offA + a_index(order, N_, r, c, lda)])
+        return G.of(A[offA + a_index(order, N_, c, r, lda)]).conj()
+    out = [G.of(x) for x in C]
+    for i in range(M):
+        for j in range(N):
+            if side == LEFT:
+                s = gsum(a(i, k) * G.of(B[offB + a_index(order, N_, k, j, ldb)]) for k in range(n))
+            else:
+                s = gsum(G.of(B[offB + a_index(order, N_, i, k, ldb)]) * a(k, j) for k in range(n))
+            ci = offC + a_index(order, N_, i, j, ldc)
+            out[ci] = G.of(alpha) * s + G.of(beta) * G.of(C[ci])
+    return out
+
+
+def as_pairs(v):
+    return [G.of(x).pair() for x in v]
+
+
 def as_floats(v):
     return [float(x) for x in v]
 
@@ -220,6 +326,39 @@ def main():
         kind="trsm", dtype="c64", order=ROW, side=LEFT, uplo=UPPER, transA=N_, diag=NONUNIT, M=3, N=4, alpha=10,
         A=At, offA=5, lda=4, B=Bt, offB=6, ldb=5,
         expected=as_floats(trsm_exact(ROW, LEFT, UPPER, N_, NONUNIT, 3, 4, 10, At, 5, 4, Bt, 6, 5)))
+    # SYR2K / HERK / HER2K / HEMM samples.  Complex buffers are lists of [re, im] pairs.
+    A2 = [11, 12, 13, 14, 21, 22, 23, 24, 31, 32, 33, 34, 41, 42, 43, 44, 51, 52, 53, 54]
+    C2 = [11, 12, 13, 14, 15, 12, 22, 23, 24, 25, 13, 23, 33, 34, 35, 14, 24, 34, 44, 45, 15, 25, 35, 45, 55]
+    cases["sample_ssyr2k_offsets"] = dict(
+        kind="syr2k", dtype="f32", order=ROW, uplo=UPPER, transA=N_, N=4, K=3, alpha=10, beta=20, A=A2, offA=5,
+        lda=4, B=A2, offB=5, ldb=4, C=C2, offC=6, ldc=5,
+        expected=as_floats(syr2k_exact(ROW, UPPER, N_, 4, 3, 10, A2, 5, 4, A2, 5, 4, 20, C2, 6, 5)))
+    Ch = [[0, 0]] * 25
+    for j, (d, im) in enumerate([(11, 1), (22, 2), (33, 4), (44, 5), (55, 6)]):
+        Ch[j * 5 + j] = [d, im]
+        for i in range(j + 1, 5):
+            Ch[j * 5 + i] = [10 * (j + 1) + i + 1, 0]
+    Aones = [[1, 0]] * 20
+    cases["sample_cherk"] = dict(
+        kind="herk", dtype="c64", order=COL, uplo=LOWER, transA=N_, N=5, K=4, alpha=10, beta=1, A=Aones, offA=0,
+        lda=5, C=Ch, offC=0, ldc=5,
+        expected=as_pairs(her2k_exact(COL, LOWER, N_, 5, 4, 10, Aones, 0, 5, None, 0, 0, 1, Ch, 0, 5)))
+    Ah = [[x, 0] for x in A2]
+    Bh = [[x, 0] for x in [1, 2, 3, 4, 2, 2, 3, 4, 3, 2, 3, 3, 4, 4, 4, 4, 5, 5, 5, 5]]
+    cases["sample_cher2k"] = dict(
+        kind="her2k", dtype="c64", order=COL, uplo=LOWER, transA=N_, N=5, K=4, alpha=[10, 1], beta=1, A=Ah, offA=0,
+        lda=5, B=Bh, offB=0, ldb=5, C=Ch, offC=0, ldc=5,
+        expected=as_pairs(her2k_exact(COL, LOWER, N_, 5, 4, [10, 1], Ah, 0, 5, Bh, 0, 5, 1, Ch, 0, 5)))
+    Am = [[11, 12], [-1, -1], [-1, -1], [-1, -1], [21, 22], [22, 23], [-1, -1], [-1, -1],
+          [31, 32], [32, 33], [33, 34], [-1, -1], [41, 61], [42, 62], [43, 73], [44, 23]]
+    Bm = [[11, -21], [-12, 23], [13, 33], [21, 12], [22, -10], [23, 5], [31, 1], [-32, 65], [33, -1],
+          [1, 41], [-33, 42], [12, 43]]
+    Cm = [[11, 11], [-12, 12], [13, 33], [21, -32], [22, -1], [23, 0], [31, 13], [-32, 78], [33, 45],
+          [41, 14], [0, 42], [43, -1]]
+    cases["sample_chemm"] = dict(
+        kind="hemm", dtype="c64", order=ROW, side=LEFT, uplo=LOWER, M=4, N=3, alpha=[10, 10], beta=[20, 20], A=Am,
+        offA=0, lda=4, B=Bm, offB=0, ldb=3, C=Cm, offC=0, ldc=3,
+        expected=as_pairs(hemm_exact(ROW, LEFT, LOWER, 4, 3, [10, 10], Am, 0, 4, Bm, 0, 3, [20, 20], Cm, 0, 3)))
     with open(os.path.join(HERE, "fixed_cases.json"), "w") as f:
         json.dump(cases, f, indent=1)
     print("wrote", len(cases), "cases")

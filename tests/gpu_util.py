@@ -73,3 +73,38 @@ def symm(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, of
                              offC, ldc)
         torch.cuda.synchronize()
     return st, dC.cpu().numpy()
+
+
+def syr2k(order, uplo, tAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, tile=None):
+    dA, dB, dC = _dev(A), _dev(B), _dev(C)
+    with _forced_tile(tile):
+        st = clblas_amd.syr2k(_PREFIX[C.dtype], order, uplo, tAB, N, K, alpha, dA, offA, lda, dB, offB, ldb, beta, dC,
+                              offC, ldc)
+        torch.cuda.synchronize()
+    return st, dC.cpu().numpy()
+
+
+def herk(order, uplo, tA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, tile=None):
+    dA, dC = _dev(A), _dev(C)
+    with _forced_tile(tile):
+        st = clblas_amd.herk(_PREFIX[C.dtype], order, uplo, tA, N, K, alpha, dA, offA, lda, beta, dC, offC, ldc)
+        torch.cuda.synchronize()
+    return st, dC.cpu().numpy()
+
+
+def her2k(order, uplo, trans, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, tile=None):
+    dA, dB, dC = _dev(A), _dev(B), _dev(C)
+    with _forced_tile(tile):
+        st = clblas_amd.her2k(_PREFIX[C.dtype], order, uplo, trans, N, K, alpha, dA, offA, lda, dB, offB, ldb, beta,
+                              dC, offC, ldc)
+        torch.cuda.synchronize()
+    return st, dC.cpu().numpy()
+
+
+def hemm(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, tile=None):
+    dA, dB, dC = _dev(A), _dev(B), _dev(C)
+    with _forced_tile(tile):
+        st = clblas_amd.hemm(_PREFIX[C.dtype], order, side, uplo, M, N, alpha, dA, offA, lda, dB, offB, ldb, beta, dC,
+                             offC, ldc)
+        torch.cuda.synchronize()
+    return st, dC.cpu().numpy()

@@ -77,3 +77,15 @@ def cgemm_bound(K, mag, dtype, c=2.0):
     mag = (|al.re|+|al.im|) (|A.re|+|A.im|)(|B.re|+|B.im|) + (|be.re|+|be.im|)(|C.re|+|C.im|)."""
     real = np.float32 if np.dtype(dtype) == np.dtype(np.complex64) else np.float64
     return c * (2 * K + 6) * EPS[np.dtype(dtype)] * mag + np.finfo(real).tiny
+
+
+def golden_array(values, dtype):
+    """A fixture buffer as a numpy array; complex buffers are stored as [re, im] pairs."""
+    a = np.array(values, dtype=np.float64)
+    if a.ndim == 2:
+        a = a[:, 0] + 1j * a[:, 1]
+    return a.astype(dtype)
+
+
+def golden_scalar(v):
+    return complex(v[0], v[1]) if isinstance(v, list) else v

@@ -120,3 +120,45 @@ def trsm_backward_error(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, 
     R = (Am @ Xm if side == LEFT else Xm @ Am) - alpha * Bm
     nrm = lambda Z: np.abs(Z).sum(axis=1).max()
     return nrm(R) / (nrm(Am) * nrm(Xm) + abs(alpha) * nrm(Bm))
+
+
+# ---- SYR2K / HERK / HER2K / HEMM -----------------------------------------------------------
+
+def herm_dense(buf, order, n, off, ld, uplo):
+    """The Hermitian matrix the routines see: the stored triangle, its conjugate mirror, and the
+    real parts of the stored diagonal."""
+    v = logical_view(buf, order, NOTRANS, n, n, off, ld)
+    t = np.where(tri_mask(n, uplo == LOWER), v, 0).astype(np.complex128)
+    d = np.diag(t).real.copy()
+    np.fill_diagonal(t, 0)
+    return t + t.conj().T + np.diag(d)
+
+
+def rank2k_want(kind, order, uplo, trans, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C0, offC, ldc):
+    """Expected stored triangle (N x N, wide precision; entries outside it are meaningless) and the
+    magnitude sum |alpha|(|A||B|^T ...) + |beta||C| for error bounds, for kind in
+    {"syr2k", "herk", "her2k"}, evaluated with numpy."""
+    wide = np.complex128 if is_cplx(C0.dtype) else np.float64
+    rows, cols = (N, K) if trans == NOTRANS else (K, N)
+    Av = logical_view(A, order, NOTRANS, rows, cols, offA, lda).astype(wide)
+    Aop = op(Av, trans)
+    Cv = logical_view(C0, order, NOTRANS, N, N, offC, ldc).astype(wide)
+    if kind == "herk":
+        want = alpha * (Aop @ Aop.conj().T)
+        mag = abs(alpha) * (abs1(Aop) @ abs1(Aop).T)
+    else:
+        Bop = op(logical_view(B, order, NOTRANS, rows, cols, offB, ldb).astype(wide), trans)
+        if kind == "syr2k":
+            want = alpha * (Aop @ Bop.T + Bop @ Aop.T)
+        else:
+            want = alpha * (Aop @ Bop.conj().T) + np.conj(alpha) * (Bop @ Aop.conj().T)
+        mag = 2 * abs1(np.asarray(alpha)) * (abs1(Aop) @ abs1(Bop).T + abs1(Bop) @ abs1(Aop).T)
+    if beta != 0:
+        Cin = Cv.copy()
+        if kind != "syr2k":
+            Cin[np.eye(N, dtype=bool)] = Cin[np.eye(N, dtype=bool)].real
+        want = want + beta * Cin
+        mag = mag + abs1(np.asarray(beta)) * abs1(np.nan_to_num(Cin))
+    if kind != "syr2k":
+        want[np.eye(N, dtype=bool)] = want[np.eye(N, dtype=bool)].real
+    return want, mag

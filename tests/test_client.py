@@ -39,11 +39,14 @@ def test_csv_rows():
     assert row["function"] == "dtrsm" and row["uplo"] == "lower" and float(row["GFLOPS"]) > 0
     for fn, prec, extra in (("gemm", "z", ["--transposeA", "2"]), ("trmm", "c", ["--side", "1"]),
                             ("trsm", "z", ["--transposeA", "2", "--uplo", "1"]),
+                            ("syr2k", "s", ["--transposeA", "1"]), ("herk", "c", ["--transposeA", "2"]),
+                            ("her2k", "z", ["--uplo", "1"]), ("hemm", "c", ["--side", "1", "--uplo", "1"]),
                             ("syrk", "d", ["--uplo", "1", "--transposeA", "1"]), ("symm", "s", ["--side", "1"])):
         r = subprocess.run([CLIENT, "-f", fn, "-r", prec, "-m", "300", "-n", "200", "-k", "100", "-p", "2",
                             "--apiCallCount", "1", "--noheader"] + extra, capture_output=True, text=True, timeout=120)
         assert r.returncode == 0, r.stderr
         row = dict(zip(HEADER.split(","), r.stdout.strip().split(",")))
         assert row["function"] == prec + fn and float(row["GFLOPS"]) > 0
-    r = subprocess.run([CLIENT, "-f", "trsv", "-r", "z"], capture_output=True, text=True, timeout=120)
-    assert r.returncode == 2
+    for fn, prec in (("trsv", "z"), ("herk", "d")):
+        r = subprocess.run([CLIENT, "-f", fn, "-r", prec], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 2

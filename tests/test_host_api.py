@@ -6,6 +6,7 @@ import itertools
 import os
 import re
 
+import numpy as np
 import pytest
 
 import clblas_amd
@@ -171,3 +172,53 @@ def test_product_package_does_not_touch_the_oracle():
             if fn.endswith((".py", ".cpp", ".hip", ".hpp", ".h")):
                 text = open(os.path.join(dirpath, fn)).read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, fn)
+
+
+@pytest.mark.parametrize("prefix", ["S", "D", "C", "Z"])
+def test_syr2k_validation(prefix):
+    f = lambda *a: clblas_amd.syr2k(prefix, *a, stream=0)
+    N, K = 6, 4
+    ok = (COL, LOWER, NOTRANS, N, K, 1.0, FAKE, 0, N, FAKE, 0, N, 0.0, FAKE, 0, N)
+    def with_(**kw):
+        names = ["order", "uplo", "trans", "N", "K", "alpha", "A", "offA", "lda", "B", "offB", "ldb", "beta", "C", "offC",
+                 "ldc"]
+        a = list(ok)
+        for k, v in kw.items():
+            a[names.index(k)] = v
+        return f(*a)
+    assert with_(A=None) == -1022 and with_(B=None) == -1021 and with_(C=None) == -1020
+    assert with_(K=0) == -1017 and with_(lda=N - 1) == -1016 and with_(ldb=N - 1) == -1015 and with_(ldc=N - 1) == -1014
+    assert with_(uplo=7) == clblas_amd.Status.InvalidValue
+    if prefix in "CZ":
+        assert with_(trans=CONJ, lda=K, ldb=K) == clblas_amd.Status.InvalidValue
+    for order, tr in itertools.product([ROW, COL], [NOTRANS, TRANS]):
+        for lda in (3, 4, 5, 6):
+            want = oracle.syr2k(order, LOWER, tr, N, K, 1.0, np.zeros(64, dtype=np.float32), 0, lda,
+                                np.zeros(64, dtype=np.float32), 0, 6, 0.0, np.zeros(64, dtype=np.float32), 0, N)
+            if want != 0:
+                assert with_(order=order, trans=tr, lda=lda, ldb=6) == want
+
+
+@pytest.mark.parametrize("prefix", ["C", "Z"])
+def test_hermitian_validation(prefix):
+    N, K = 6, 4
+    herk = lambda **kw: clblas_amd.herk(prefix, kw.get("order", COL), LOWER, kw.get("trans", NOTRANS), N, kw.get("K", K),
+                                        1.0, kw.get("A", FAKE), 0, kw.get("lda", N), 0.0, kw.get("C", FAKE), 0,
+                                        kw.get("ldc", N), stream=0)
+    her2k = lambda **kw: clblas_amd.her2k(prefix, COL, LOWER, kw.get("trans", NOTRANS), N, kw.get("K", K), 1 + 1j,
+                                          kw.get("A", FAKE), 0, kw.get("lda", N), kw.get("B", FAKE), 0,
+                                          kw.get("ldb", N), 0.0, kw.get("C", FAKE), 0, kw.get("ldc", N), stream=0)
+    for f in (herk, her2k):
+        assert f(A=None) == -1022 and f(C=None) == -1020
+        assert f(trans=TRANS, lda=K, ldb=K) == clblas_amd.Status.InvalidValue  # xherk.c:69-71, xher2k.c:79-81
+        assert f(K=0) == -1017 and f(lda=N - 1) == -1016 and f(ldc=N - 1) == -1014
+        assert f(trans=CONJ, lda=K - 1, ldb=K) == -1016
+    assert her2k(B=None) == -1021 and her2k(ldb=N - 1) == -1015
+    assert herk(order=ROW, lda=K - 1) == -1016
+    M = 5
+    hemm = lambda **kw: clblas_amd.hemm(prefix, kw.get("order", COL), kw.get("side", LEFT), UPPER, M, N, 1.0,
+                                        kw.get("A", FAKE), 0, kw.get("lda", 6), kw.get("B", FAKE), 0, kw.get("ldb", M),
+                                        0.0, kw.get("C", FAKE), 0, kw.get("ldc", M), stream=0)
+    assert hemm(A=None) == -1022 and hemm(B=None) == -1021 and hemm(C=None) == -1020
+    assert hemm(lda=4) == -1016 and hemm(side=RIGHT, lda=5) == -1016 and hemm(ldb=4) == -1015 and hemm(ldc=4) == -1014
+    assert hemm(side=9) == clblas_amd.Status.InvalidValue
