@@ -38,6 +38,15 @@
  *                             and trmm (oracle/_ref); SYMM, which has no naive statement in the
  *                             reference, against oracle GEMM on the explicitly symmetrised
  *                             matrix; TRMM followed by TRSM returns the input.
+ *   oracle_{s,d,c,z}syr2k, oracle_{c,z}{herk,her2k,hemm} (level3.inc)
+ *                           - src/samples/example_{ssyr2k.c,cherk.cpp,cher2k.c,chemm.cpp} fixed
+ *                             inputs against exact expected values (complex diagonals with
+ *                             non-zero imaginary parts included); exact-integer inputs against
+ *                             products evaluated with numpy for every order / side / triangle /
+ *                             transpose combination, unused triangle NaN-poisoned; the
+ *                             reference's own naive syr2k (oracle/_ref); HEMM against oracle
+ *                             GEMM on the explicitly formed Hermitian matrix; HER2K with B == A
+ *                             against HERK.  (The reference has no naive herk / her2k / hemm.)
  *   oracle_check_*          - expectations of src/tests/functional/func-error.cpp:58-104 and
  *                             the branch table of generic/common.c:585-688.
  *   Bit-for-bit output of the OpenCL kernels (implementation-defined `mad` contraction,
