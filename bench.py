@@ -198,7 +198,7 @@ def main():
                        "pct_of_matrix_peak": round(100 * c_tflops / peak, 2)}
         del A, B, C
 
-    # ---- SYRK / TRMM / SYMM at the same size (useful flops only: the reference client's counts) ----
+    # ---- SYRK / TRMM / SYMM / SYR2K and the complex-only routines at the same size (useful flops only: the reference client's counts) ----
     if args.only in ("", "level3"):
         lv = {}
         for pre, dt, peak in (("S", torch.float32, PEAK_FP32_MATRIX), ("D", torch.float64, PEAK_FP64_MATRIX)):
@@ -213,18 +213,51 @@ def main():
                  lambda: clblas_amd.trmm(pre, COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, A, 0, n, B, 0, n)),
                 ("symm", 2.0 * n * n * n, None,
                  lambda: clblas_amd.symm(pre, COL, LEFT, LOWER, n, n, 1.0, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+                ("syr2k", 2.0 * n * n * n + n, None,
+                 lambda: clblas_amd.syr2k(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
             )
             for name, fl, before, fn in cases:
                 def call(fn=fn, name=name):
                     st = fn()
                     if st != 0:
                         raise RuntimeError("clblas%s%s returned %d" % (pre, name, st))
-                wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 1, before_each=before)
+                wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 2, before_each=before)
                 tf = fl / (ev_ms * 1e-3) / 1e12
                 lv[pre.lower() + name] = {"tflops": round(tf, 2), "ms_per_call": round(ev_ms, 4),
                                           "pct_of_matrix_peak": round(100 * tf / peak, 1)}
             del A, B, B0, C
-        lv["workload"] = "column-major, lower, left, no transpose, N=M=K=%d, alpha=beta=1" % n
+        # complex types: the Hermitian routines and the triangular solve (flop counts of the reference client)
+        for pre, dt, peak in (("C", torch.complex64, PEAK_FP32_MATRIX), ("Z", torch.complex128, PEAK_FP64_MATRIX)):
+            rdt = torch.float32 if dt == torch.complex64 else torch.float64
+            A, B0, C = (torch.view_as_complex(torch.rand(n * n, 2, device="cuda", dtype=rdt, generator=gen) * 2 - 1)
+                        for _ in range(3))
+            B = B0.clone()
+            T = A / n  # well-conditioned triangle: small off-diagonal entries, diagonal in [1, 2)
+            T.view(n, n).diagonal().copy_(torch.rand(n, device="cuda", dtype=rdt, generator=gen) + 1)
+            trsm = clblas_amd.ctrsm if pre == "C" else clblas_amd.ztrsm
+            cases = (
+                ("herk", 4.0 * n * n * (n + 1), None,
+                 lambda: clblas_amd.herk(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, 1.0, C, 0, n)),
+                ("her2k", 8.0 * n * n * n + 2 * n, None,
+                 lambda: clblas_amd.her2k(pre, COL, LOWER, NOTRANS, n, n, 1.0 + 0.5j, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+                ("hemm", 8.0 * n * n * n, None,
+                 lambda: clblas_amd.hemm(pre, COL, LEFT, LOWER, n, n, 1.0 + 0.5j, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+                ("trsm", 4.0 * n * (n + 1) * n, lambda: B.copy_(B0),
+                 lambda: trsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, T, 0, n, B, 0, n)),
+            )
+            for name, fl, before, fn in cases:
+                def call(fn=fn, name=name):
+                    st = fn()
+                    if st != 0:
+                        raise RuntimeError("clblas%s%s returned %d" % (pre, name, st))
+                wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 2, before_each=before)
+                tf = fl / (ev_ms * 1e-3) / 1e12
+                lv[pre.lower() + name] = {"tflops": round(tf, 2), "ms_per_call": round(ev_ms, 4),
+                                          "pct_of_matrix_peak": round(100 * tf / peak, 1)}
+            if not bool(torch.isfinite(torch.view_as_real(B)).all().item()):
+                raise RuntimeError("clblas%strsm produced non-finite values" % pre)
+            del A, B, B0, C, T
+        lv["workload"] = "column-major, lower, left, no transpose, N=M=K=%d, alpha=beta=1 (complex: alpha=1+0.5i)" % n
         extra["level3"] = lv
 
     # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
