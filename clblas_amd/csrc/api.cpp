@@ -3,8 +3,10 @@
 // This is the host front end that stands where the reference has
 //   src/library/blas/xgemm.cc:667-905  (clblasSgemm / clblasDgemm / clblasCgemm / clblasZgemm),
 //   src/library/blas/xgemm.cc:341-383  (clblasGemm<T>: ConjTrans and row-major folding),
-//   src/library/blas/xtrsm.cc:1600-1785 (clblasStrsm / clblasDtrsm),
+//   src/library/blas/xtrsm.cc:1600-1914 (clblasStrsm / clblasDtrsm / clblasCtrsm / clblasZtrsm),
 //   src/library/blas/xsyrk.c:27-233, xtrmm.c:27-245, xsymm.c:33-429 (SYRK / TRMM / SYMM),
+//   src/library/blas/xsyr2k.c:27-251, xherk.c:29-210, xher2k.c:30-245, xhemm.c:36-112
+//   (SYR2K / HERK / HER2K / HEMM),
 //   src/library/blas/functor/functor_xtrsm.cc:57-75 (doTrsm validation),
 //   src/library/blas/generic/common.c:585-688 (checkMatrixSizes),
 //   src/library/blas/init.c:33-263 (GetVersion / Setup / Teardown).
