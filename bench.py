@@ -121,7 +121,7 @@ def main():
             "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MATRIX,
                          "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MATRIX, 4),
                          "traffic": SGEMM_8192_TRAFFIC_BYTES if n == 8192 else None,
-                         "kernel": "gemm_mfma_kernel<float,128,128,16,...> (one launch per call)",
+                         "kernel": "gemm_mfma_kernel<float,256,128,16,...> (one launch per call)",
                          "launch_ms": round(ev_ms, 4)},
         }
         extra["sgemm_pct_of_fp32_matrix_peak"] = round(100 * tflops / PEAK_FP32_MATRIX, 2)

@@ -18,7 +18,9 @@ SOURCES = ["api.cpp", "gemm_f32.hip", "gemm_f64.hip", "gemm_c32.hip", "gemm_c64.
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-COMMON_FLAGS = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option"]
+# -Wno-align-mismatch: C is accessed through element-aligned vector types on purpose (offsets and odd ld).
+COMMON_FLAGS = ["-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
+                "-Wno-align-mismatch"]
 
 
 def _hipcc():
@@ -30,12 +32,34 @@ def _compile(src):
     cmd = [_hipcc()] + COMMON_FLAGS
     if src.endswith(".hip"):
         cmd += DEVICE_FLAGS
+        cmd += ["-Rpass-analysis=kernel-resource-usage"]
     cmd += ["-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # The host pass warns that it does not know the packed-fp32 feature; that is harmless.
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    lines = [l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l]
+    # Resource-usage remarks: a kernel whose accumulators end up in scratch memory still gives
+    # right answers, fifty times slower - refuse to build it.
+    spilled, name = [], "?"
+    for l in lines:
+        if "Function Name:" in l:
+            name = l.split("Function Name:")[1].split("[-Rpass")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in l:
+            if int(l.split("ScratchSize [bytes/lane]:")[1].split()[0]) > 0:
+                spilled.append(name)
+    kept, in_remark = [], False
+    for l in lines:  # drop the remarks together with the source excerpt that follows each of them
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            in_remark = True
+        elif in_remark and (l.lstrip().startswith("|") or l.lstrip().split(" ", 1)[0].isdigit()):
+            pass
+        else:
+            in_remark = False
+            kept.append(l)
+    err = "\n".join(kept)
     if res.returncode != 0:
         raise RuntimeError("compile failed: %s\n%s" % (" ".join(cmd), err))
+    if spilled:
+        raise RuntimeError("%s: kernels use scratch memory (register spills): %s" % (src, ", ".join(spilled)))
     if err.strip():
         sys.stderr.write(err + "\n")
     return obj

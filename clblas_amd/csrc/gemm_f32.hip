@@ -9,8 +9,8 @@ namespace cba {
 //   2:  64x64x16,  wave 32x32, split-K capable (small / deep-K problems)
 static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
-        make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.914),
-        make_tile_entry<float, 128, 128, 16, 64, 64, 2, false, true>(0.919),
+        make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
+        make_tile_entry<float, 128, 128, 16, 64, 64, 2, false, true>(0.920),
         make_tile_entry<float, 64, 64, 16, 32, 32, 2, true, true>(0.83),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

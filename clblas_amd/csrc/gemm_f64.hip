@@ -8,7 +8,7 @@ namespace cba {
 //   1:  64x64x16,  wave 32x32, split-K capable
 static const TileEntry<double> *f64_tiles(int *n) {
     static const TileEntry<double> tab[] = {
-        make_tile_entry<double, 128, 128, 16, 64, 64, 2, false, true>(0.905),
+        make_tile_entry<double, 128, 128, 16, 64, 64, 2, false, true>(0.94),
         make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true>(0.885),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

@@ -189,6 +189,8 @@ template <typename T> struct GemmParams {
     int tiles_m, tiles_n;
     int group_m;      // tile rows walked together (L2 locality)
     int xcd_remap;    // 1: give each XCD a contiguous chunk of the tile list
+    int spread_loads; // 1: issue the loads of the next panel one by one between the MFMA steps of this one
+                      //    instead of all at its top (better when several workgroups share a CU)
     int k_per_split;  // multiple of BK; >= K when the K loop is not split
     T *ws;            // split-K partial sums: ws[split * ws_slice + n * ws_ld + m]
     int64_t ws_ld, ws_slice;
@@ -351,6 +353,12 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
         for (int i = 0; i < PER; ++i)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH), 16,
                                                      (int)voff[i], 0, 0, 0);
+    }
+
+    // One of the PER wave-wide loads of a panel (same arguments as issue()).
+    __device__ __forceinline__ void issue_one(__amdgpu_buffer_rsrc_t r, T *lds, int wave_u, int i) const {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH), 16,
+                                                 (int)voff[i], 0, 0, 0);
     }
 
     // Triangular operand: in the 16 bytes each of this thread's loads delivered, zeroes the
@@ -543,7 +551,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         constexpr int LOADS_PER_PANEL = LA::PER + LB::PER;  // vector-memory instructions per wave and panel
 
         auto stage_ptr = [&](int kp) -> T * { return smem + (kp % NSTAGE) * STAGE; };
-        auto issue_panel = [&](int kp) {
+        auto issue_panel = [&](int kp) __attribute__((always_inline)) {
             const int k0 = k_begin + kp * BK;
             const int64_t ao = a_off(k0), bo = b_off(k0);
             T *dst = stage_ptr(kp);
@@ -552,12 +560,14 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         };
         // Makes panel kp (already requested) readable by the whole workgroup: own loads
         // complete, K tail cleared, barrier.
-        auto publish_panel = [&](int kp, bool newer_in_flight) {
+        // full_depth: the caller knows that the panel is not the last one of its K range, so
+        // it has no tail.
+        auto publish_panel = [&](int kp, bool newer_in_flight, bool full_depth) __attribute__((always_inline)) {
             T *dst = stage_ptr(kp);
             const int k_valid = k_end - (k_begin + kp * BK);
             if (newer_in_flight) __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(LOADS_PER_PANEL));
             else __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0));
-            if (k_valid < BK) {
+            if (!full_depth && k_valid < BK) {
                 la.clear_k_tail(dst, tid, k_valid);
                 lb.clear_k_tail(dst + A_ELEMS, tid, k_valid);
             }
@@ -574,15 +584,43 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 
         issue_panel(0);
         if (DEPTH == 2 && n_panels > 1) issue_panel(1);
-        publish_panel(0, DEPTH == 2 && n_panels > 1);
+        publish_panel(0, DEPTH == 2 && n_panels > 1, false);
 
         const int a_frag = wm * WM + j * VM;
         const int b_frag = wn * WN + j * VN;
         constexpr int STEPS = BK / KS;
 
-        auto do_panel = [&](int kp) {
-            const bool issued = kp + DEPTH < n_panels;
-            if (issued) issue_panel(kp + DEPTH);
+        // steady_tag: panel kp+DEPTH exists and panel kp+1 is not the last one - true for all
+        // but the last few panels, which lets the body run without a single branch.
+        auto do_panel = [&](int kp, auto spread_tag, auto steady_tag) __attribute__((always_inline)) {
+            constexpr bool steady = decltype(steady_tag)::value;
+            const bool issued = steady || kp + DEPTH < n_panels;
+            // The loads of panel kp+DEPTH: all at once here, or - when workgroups share the CU
+            // and cover each other's waits - one at a time behind the MFMAs of the steps below,
+            // where their issue does not hold up this wavefront's MFMAs (8192^3 FP32: +2-4 %;
+            // a workgroup alone on its CU needs the earlier start: -3-6 % there).
+            constexpr bool spread = decltype(spread_tag)::value;
+            __amdgpu_buffer_rsrc_t ra, rb;
+            T *dst_next = stage_ptr(kp + DEPTH);
+            if (issued) {
+                if (spread) {
+                    const int k0n = k_begin + (kp + DEPTH) * BK;
+                    const int64_t ao = a_off(k0n), bo = b_off(k0n);
+                    ra = make_rsrc(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
+                    rb = make_rsrc(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
+                } else {
+                    issue_panel(kp + DEPTH);
+                }
+            }
+            auto issue_behind_step = [&](int s) __attribute__((always_inline)) {
+                constexpr int L = LA::PER + LB::PER;
+#pragma unroll
+                for (int i = 0; i < L; ++i)
+                    if (i * STEPS / L == s) {
+                        if (i < LA::PER) la.issue_one(ra, dst_next, wave_u, i);
+                        else lb.issue_one(rb, dst_next + A_ELEMS, wave_u, i - LA::PER);
+                    }
+            };
 
             const T *As = stage_ptr(kp);
             const T *Bs = As + A_ELEMS;
@@ -688,16 +726,29 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 #pragma unroll
                         for (int bm = 0; bm < TM; ++bm) acc[bn][bm][1] = M::run(bre_x[bn], a_of(bm).im, acc[bn][bm][1]);
                 }
+                if (issued && spread) issue_behind_step(s);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (kp + 1 < n_panels) publish_panel(kp + 1, DEPTH == 2 && issued);
+            if (steady || kp + 1 < n_panels) publish_panel(kp + 1, DEPTH == 2 && issued, steady);
             else __syncthreads();
         };
         // Two panels per trip, so that the stage addresses of each copy are loop-invariant.
-        for (int kp = 0; kp < n_panels; kp += 2) {
-            do_panel(kp);
-            if (kp + 1 < n_panels) do_panel(kp + 1);
-        }
+        // (Both ways of requesting panels are compiled; a branch inside the loop would sit
+        // between the MFMA steps.)
+        // Taken branches cost a wavefront tens of cycles of instruction fetch, which shows as
+        // idle MFMA time when only two wavefronts share a SIMD: the steady part of the loop is
+        // straight-line code, and the last panels (at most DEPTH + 2) run a general copy.
+        auto k_loop = [&](auto spread_tag) __attribute__((always_inline)) {
+            const int n_steady = n_panels - 1 - DEPTH > 0 ? ((n_panels - 1 - DEPTH) & ~1) : 0;
+            int kp = 0;
+            for (; kp < n_steady; kp += 2) {
+                do_panel(kp, spread_tag, std::true_type());
+                do_panel(kp + 1, spread_tag, std::true_type());
+            }
+            for (; kp < n_panels; ++kp) do_panel(kp, spread_tag, std::false_type());
+        };
+        if (p.spread_loads) k_loop(std::true_type());
+        else k_loop(std::false_type());
     }
 
     // ---- epilogue ----

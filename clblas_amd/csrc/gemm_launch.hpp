@@ -198,6 +198,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     if (p.group_m > p.tiles_m) p.group_m = p.tiles_m;
     if (p.group_m < 1) p.group_m = 1;
     p.xcd_remap = debug_env_int("CLBLAS_AMD_GEMM_XCD", 1);
+    p.spread_loads = 0;
     p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
     p.k_per_split = K;
     p.tri_c = p.tri_a = p.tri_b = p.unit_a = p.unit_b = p.rev_m = p.rev_n = p.herm_c = 0;
@@ -254,6 +255,15 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             p.ws = (T *)w;
             fn = e.splitk[idx];
         }
+    }
+    // Workgroups per CU at the start of the launch decide how the K loop requests its panels.
+    {
+        const int forced = debug_env_int("CLBLAS_AMD_GEMM_SPREAD", -1);
+        // Measured at 8192^3 (TFLOP/s, all at once -> spread): FP32 256x128 144.3 -> 148.3, FP64 128x128
+        // 70.5 -> 74.0, complex FP32 145.9 -> 147.0, complex FP64 73.6 -> 73.3 (left as it was); with one
+        // workgroup per CU (2048^3 FP32) 116 -> 112.
+        const bool many = grid_x * (splits > 1 ? splits : 1) >= 2 * 256;
+        p.spread_loads = forced >= 0 ? (forced != 0) : (many && sizeof(T) < 16);
     }
     const size_t smem = e.smem_of[idx];
     if (smem > 64 * 1024) {

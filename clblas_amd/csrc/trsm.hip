@@ -263,25 +263,34 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
         }
     } else {
         constexpr int NLD = CW * (L::NB / 2) / NT;
-        T v0[NLD], v1[NLD];
+        // (kept as real components: arrays of complex structs end up in scratch memory)
+        constexpr int NC = CPLX ? 2 : 1;
+        R v0[NLD][NC], v1[NLD][NC];
+        auto split = [&](T t, R (&out)[NC]) {
+            if constexpr (CPLX) { out[0] = t.re; out[1] = t.im; } else { out[0] = t; }
+        };
+        auto join = [&](const R (&in)[NC]) -> T {
+            if constexpr (CPLX) return T{in[0], in[1]};
+            else return in[0];
+        };
 #pragma unroll
         for (int u = 0; u < NLD; ++u) {
             const int e = tid + u * NT;
             const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-            v0[u] = T();
-            v1[u] = T();
+#pragma unroll
+            for (int q = 0; q < NC; ++q) v0[u][q] = v1[u][q] = (R)0;
             if (j0 + c < nrhs) {
                 const T *src = Bblk + r + (j0 + c) * ldb;
-                if (r < nb) v0[u] = src[0];
-                if (r + 1 < nb) v1[u] = src[1];
+                if (r < nb) split(src[0], v0[u]);
+                if (r + 1 < nb) split(src[1], v1[u]);
             }
         }
 #pragma unroll
         for (int u = 0; u < NLD; ++u) {
             const int e = tid + u * NT;
             const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-            S[c * L::SP + r] = v0[u];
-            S[c * L::SP + r + 1] = v1[u];
+            S[c * L::SP + r] = join(v0[u]);
+            S[c * L::SP + r + 1] = join(v1[u]);
         }
         __syncthreads();
 #pragma unroll
