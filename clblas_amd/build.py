@@ -55,6 +55,8 @@ def _compile(src):
         else:
             in_remark = False
             kept.append(l)
+    if not any("warning" in l or "error" in l for l in kept):
+        kept = []  # only include-stack lines of the dropped remarks are left
     err = "\n".join(kept)
     if res.returncode != 0:
         raise RuntimeError("compile failed: %s\n%s" % (" ".join(cmd), err))
