@@ -189,8 +189,7 @@ template <typename T> struct GemmParams {
     int tiles_m, tiles_n;
     int group_m;      // tile rows walked together (L2 locality)
     int xcd_remap;    // 1: give each XCD a contiguous chunk of the tile list
-    int spread_loads; // 1: issue the loads of the next panel one by one between the MFMA steps of this one
-                      //    instead of all at its top (better when several workgroups share a CU)
+    int stagger;      // 1: every other workgroup of the first round starts late (see the kernel)
     int k_per_split;  // multiple of BK; >= K when the K loop is not split
     T *ws;            // split-K partial sums: ws[split * ws_slice + n * ws_ld + m]
     int64_t ws_ld, ws_slice;
@@ -456,6 +455,23 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     constexpr int NSTAGE = Cfg::NSTAGE, DEPTH = Cfg::DEPTH;
     constexpr bool A_KLAY = Cfg::A_KLAY, B_KLAY = Cfg::B_KLAY;
 
+    // Two workgroups that share a CU from the start run in lockstep and finish together; both
+    // of their slots then go to two later workgroups at once, and at the end of a launch that
+    // is not a whole number of rounds some CUs hold two workgroups while others idle.  So the
+    // workgroups that took the second wave slot of their SIMD in the first round start late,
+    // by about a quarter of the time two of them take for a tile.  (First thing in the kernel:
+    // nothing is live yet.)
+    if (p.stagger && blockIdx.x < 512) {
+        const unsigned slot = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (3 << 11));  // HW_ID.WAVE_ID
+        if (slot & 1) {
+            // MFMA time of one wavefront for one panel, in cycles
+            constexpr int PANEL_CYCLES = Cfg::TM * Cfg::TN * (BK / Cfg::KS) * (Cfg::CPLX ? 4 : 1) * 64;
+            const int panels = (SPLITK ? p.k_per_split : p.K) / BK;
+            const int n = (int)(((int64_t)panels * PANEL_CYCLES / 2) >> 12);
+            for (int i = 0; i < n; ++i) __builtin_amdgcn_s_sleep(64);  // ~4096 cycles each
+        }
+    }
+
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     T *smem = reinterpret_cast<T *>(smem_raw);
 
@@ -592,31 +608,32 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 
         // steady_tag: panel kp+DEPTH exists and panel kp+1 is not the last one - true for all
         // but the last few panels, which lets the body run without a single branch.
-        auto do_panel = [&](int kp, auto spread_tag, auto steady_tag) __attribute__((always_inline)) {
+        auto do_panel = [&](int kp, auto steady_tag) __attribute__((always_inline)) {
             constexpr bool steady = decltype(steady_tag)::value;
             const bool issued = steady || kp + DEPTH < n_panels;
-            // The loads of panel kp+DEPTH: all at once here, or - when workgroups share the CU
-            // and cover each other's waits - one at a time behind the MFMAs of the steps below,
-            // where their issue does not hold up this wavefront's MFMAs (8192^3 FP32: +2-4 %;
-            // a workgroup alone on its CU needs the earlier start: -3-6 % there).
-            constexpr bool spread = decltype(spread_tag)::value;
+            // The loads of panel kp+DEPTH are not issued here, all at once, but one by one behind
+            // the MFMAs of the first steps below, where their issue does not hold up this
+            // wavefront's MFMAs (8192^3: FP32 144 -> 149 TFLOP/s, FP64 70.5 -> 74; 1024^3 FP32
+            // 75 -> 81).  Only the descriptors are made here.
             __amdgpu_buffer_rsrc_t ra, rb;
             T *dst_next = stage_ptr(kp + DEPTH);
             if (issued) {
-                if (spread) {
-                    const int k0n = k_begin + (kp + DEPTH) * BK;
-                    const int64_t ao = a_off(k0n), bo = b_off(k0n);
-                    ra = make_rsrc(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
-                    rb = make_rsrc(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
-                } else {
-                    issue_panel(kp + DEPTH);
-                }
+                const int k0n = k_begin + (kp + DEPTH) * BK;
+                const int64_t ao = a_off(k0n), bo = b_off(k0n);
+                ra = make_rsrc(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
+                rb = make_rsrc(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
             }
+            // (Complex FP64, with two long steps per panel, is the exception: 73.8 TFLOP/s at
+            // 8192^3 with all loads up front, 72.7 with them behind the first step.)
+            constexpr bool LOADS_UP_FRONT = sizeof(T) == 16;
             auto issue_behind_step = [&](int s) __attribute__((always_inline)) {
                 constexpr int L = LA::PER + LB::PER;
+                // over the first quarter of the steps: as good as over all of them where
+                // workgroups share a CU, and the loads keep most of the panel to complete in
+                constexpr int SP = STEPS / 4 > 0 ? STEPS / 4 : 1;
 #pragma unroll
                 for (int i = 0; i < L; ++i)
-                    if (i * STEPS / L == s) {
+                    if ((LOADS_UP_FRONT ? -1 : i * SP / L) == s) {
                         if (i < LA::PER) la.issue_one(ra, dst_next, wave_u, i);
                         else lb.issue_one(rb, dst_next + A_ELEMS, wave_u, i - LA::PER);
                     }
@@ -673,6 +690,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                     for (int e = 0; e < VEC; ++e) bf[bn][e] = Vec<T, VEC>::get(bv, e);
                 }
             };
+            if (LOADS_UP_FRONT && issued) issue_behind_step(-1);
             if constexpr (A_KLAY) read_ak(0, ak[0]); else read_a(0, a[0]);
             if constexpr (B_KLAY) read_bk(0, bk[0]); else read_b(0, b[0]);
 #pragma unroll
@@ -726,29 +744,26 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 #pragma unroll
                         for (int bm = 0; bm < TM; ++bm) acc[bn][bm][1] = M::run(bre_x[bn], a_of(bm).im, acc[bn][bm][1]);
                 }
-                if (issued && spread) issue_behind_step(s);
+                if (!LOADS_UP_FRONT && issued) issue_behind_step(s);
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (steady || kp + 1 < n_panels) publish_panel(kp + 1, DEPTH == 2 && issued, steady);
             else __syncthreads();
         };
         // Two panels per trip, so that the stage addresses of each copy are loop-invariant.
-        // (Both ways of requesting panels are compiled; a branch inside the loop would sit
-        // between the MFMA steps.)
         // Taken branches cost a wavefront tens of cycles of instruction fetch, which shows as
         // idle MFMA time when only two wavefronts share a SIMD: the steady part of the loop is
         // straight-line code, and the last panels (at most DEPTH + 2) run a general copy.
-        auto k_loop = [&](auto spread_tag) __attribute__((always_inline)) {
+        auto k_loop = [&]() __attribute__((always_inline)) {
             const int n_steady = n_panels - 1 - DEPTH > 0 ? ((n_panels - 1 - DEPTH) & ~1) : 0;
             int kp = 0;
             for (; kp < n_steady; kp += 2) {
-                do_panel(kp, spread_tag, std::true_type());
-                do_panel(kp + 1, spread_tag, std::true_type());
+                do_panel(kp, std::true_type());
+                do_panel(kp + 1, std::true_type());
             }
-            for (; kp < n_panels; ++kp) do_panel(kp, spread_tag, std::false_type());
+            for (; kp < n_panels; ++kp) do_panel(kp, std::false_type());
         };
-        if (p.spread_loads) k_loop(std::true_type());
-        else k_loop(std::false_type());
+        k_loop();
     }
 
     // ---- epilogue ----

@@ -198,7 +198,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     if (p.group_m > p.tiles_m) p.group_m = p.tiles_m;
     if (p.group_m < 1) p.group_m = 1;
     p.xcd_remap = debug_env_int("CLBLAS_AMD_GEMM_XCD", 1);
-    p.spread_loads = 0;
+    p.stagger = 0;
     p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
     p.k_per_split = K;
     p.tri_c = p.tri_a = p.tri_b = p.unit_a = p.unit_b = p.rev_m = p.rev_n = p.herm_c = 0;
@@ -256,14 +256,13 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             fn = e.splitk[idx];
         }
     }
-    // Workgroups per CU at the start of the launch decide how the K loop requests its panels.
+    // The late start that keeps the workgroups of a CU out of lockstep when the launch is not a
+    // whole number of rounds of 2 x 256 workgroups (see the kernel; 3584^3 FP64: 54 -> 69 TFLOP/s).
     {
-        const int forced = debug_env_int("CLBLAS_AMD_GEMM_SPREAD", -1);
-        // Measured at 8192^3 (TFLOP/s, all at once -> spread): FP32 256x128 144.3 -> 148.3, FP64 128x128
-        // 70.5 -> 74.0, complex FP32 145.9 -> 147.0, complex FP64 73.6 -> 73.3 (left as it was); with one
-        // workgroup per CU (2048^3 FP32) 116 -> 112.
-        const bool many = grid_x * (splits > 1 ? splits : 1) >= 2 * 256;
-        p.spread_loads = forced >= 0 ? (forced != 0) : (many && sizeof(T) < 16);
+        const int64_t wgs = grid_x * (splits > 1 ? splits : 1);
+        const bool whole_rounds = p.tail_slices <= 1 && wgs % 512 == 0;
+        p.stagger = wgs > 512 && !whole_rounds && !(p.tri_a || p.tri_b) &&
+                    debug_env_int("CLBLAS_AMD_GEMM_STAGGER", 1) != 0;
     }
     const size_t smem = e.smem_of[idx];
     if (smem > 64 * 1024) {
