@@ -30,7 +30,7 @@ PEAK_FP64_MATRIX = 78.6
 # device copy (profiles/bench_8192_counters.md: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
 # Counters cannot be read from inside this process, so the figure is carried as a constant
 # and only reported when the workload is the one it was measured on.
-SGEMM_8192_TRAFFIC_BYTES = 7.69e9
+SGEMM_8192_TRAFFIC_BYTES = 4.95e9
 
 COL, NOTRANS, TRANS = 1, 0, 1
 LEFT, LOWER, NONUNIT = 0, 1, 1

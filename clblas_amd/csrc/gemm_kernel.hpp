@@ -1,5 +1,6 @@
 // MFMA GEMM kernel for gfx950 (CDNA4): FP32, FP64 and their complex counterparts, all
-// transpose / conjugate combinations; the TRI variants also serve SYRK, TRMM and SYMM.
+// transpose / conjugate combinations; the TRI variants also serve SYRK, SYR2K, HERK, HER2K,
+// TRMM, SYMM and HEMM.
 //
 // Computes (column-major, after the host has folded row-major calls)
 //     C(m,n) <- alpha * sum_k opA(m,k) * opB(k,n) + beta * C(m,n)
@@ -16,8 +17,10 @@
 //     bank-conflict free.  Each lane of such a load names its own source address, so the rows
 //     of As[m][k] are stored block by block (all rows of MFMA block 0, then block 1, ...)
 //     while a lane still owns VM consecutive rows of C for its 16-byte stores.
-//   * NSTAGE LDS stages form a ring; the loads of panel p+NSTAGE-1 are issued at the top of
-//     panel p and one barrier per panel publishes the next stage.  Buffer descriptors are
+//   * NSTAGE LDS stages form a ring; the loads of panel p+NSTAGE-1 are issued during panel p,
+//     one at a time behind the MFMAs of its first steps (in front of them they cost several
+//     per cent), and one barrier per panel publishes the next stage.  All but the last few
+//     panels run straight-line code, two panels per loop trip.  Buffer descriptors are
 //     re-based every panel and sized to the exact footprint of the operand, so the hardware
 //     range check turns every access past the end of the matrix into a zero (also on the
 //     LDS path): no extra launch and no per-element branch is needed for M/N remainders or
