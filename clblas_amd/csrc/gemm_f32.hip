@@ -11,7 +11,7 @@ static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, false, true>(0.920),
-        make_tile_entry<float, 64, 64, 16, 32, 32, 2, true, true>(0.83),
+        make_tile_entry<float, 64, 64, 16, 32, 32, 2, true, true>(0.80),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

@@ -9,7 +9,7 @@ namespace cba {
 static const TileEntry<double> *f64_tiles(int *n) {
     static const TileEntry<double> tab[] = {
         make_tile_entry<double, 128, 128, 16, 64, 64, 2, false, true>(0.94),
-        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true>(0.885),
+        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true>(0.84),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

@@ -108,7 +108,7 @@ static inline int tail_slices_for(int64_t t, int K, int bk, bool allowed) {
 
 template <typename T>
 static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, bool need_tri, int tri_c,
-                        bool tail_ok, int *tile_out, int *splits_out) {
+                        bool tri_operand, bool tail_ok, int *tile_out, int *splits_out) {
     const int64_t kCUs = 256;
     int pick = ntab - 1;  // table is ordered large -> small
     if (force >= 0 && force < ntab && (!need_tri || tab[force].tri[0])) {
@@ -122,6 +122,11 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             double rounds = (double)ceil_div64(t, kCUs);
             const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
             if (ts > 1) rounds = (double)(t / kCUs) + 1.0 / ts + 0.05;  // + the reduction pass
+            // A triangular operand makes the tiles differ in depth (half of the full depth on
+            // average, started deepest first): the CUs share the total evenly up to a fraction
+            // of one full-depth tile, fitted to STRMM / DTRMM 4096 and 8192 (STRMM 4096: 256x128
+            // tiles 0.77 ms, 128x128 0.60 ms, 64x64 0.67 ms).
+            if (tri_operand) rounds = (double)t / (2.0 * kCUs) + 0.4;
             double cost = rounds * tab[i].bm * tab[i].bn / tab[i].eff;
             if (t <= kCUs) cost /= 0.85;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             if (!have || cost < best) { best = cost; pick = i; have = true; }
@@ -169,7 +174,8 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     int tile, splits;
     // The tail may be sliced unless tiles differ in depth (triangular operands).
     const bool tail_ok = !(need_tri && (tri->tri_a || tri->tri_b)) && debug_env_int("CLBLAS_AMD_GEMM_TAIL", 1) != 0;
-    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, need_tri ? tri->tri_c : 0, tail_ok, &tile, &splits);
+    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, need_tri ? tri->tri_c : 0,
+                need_tri && (tri->tri_a || tri->tri_b), tail_ok, &tile, &splits);
     const TileEntry<T> &e = tab[tile];
 
     GemmParams<T> p;
