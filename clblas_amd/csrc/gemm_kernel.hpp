@@ -17,7 +17,7 @@
 //     bank-conflict free.  Each lane of such a load names its own source address, so the rows
 //     of As[m][k] are stored block by block (all rows of MFMA block 0, then block 1, ...)
 //     while a lane still owns VM consecutive rows of C for its 16-byte stores.
-//   * NSTAGE LDS stages form a ring; the loads of panel p+NSTAGE-1 are issued during panel p,
+//   * Two LDS stages; the loads of panel p+1 are issued during panel p,
 //     one at a time behind the MFMAs of its first steps (in front of them they cost several
 //     per cent), and one barrier per panel publishes the next stage.  All but the last few
 //     panels run straight-line code, two panels per loop trip.  Buffer descriptors are
@@ -433,11 +433,9 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static constexpr int PITCH_A = LoaderA::LDS_PITCH, PITCH_B = LoaderB::LDS_PITCH;
     static constexpr int A_ELEMS = LoaderA::LDS_ELEMS;
     static constexpr int STAGE = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;  // elements per LDS stage
-    // Two stages: the loads of panel p+1 are issued at the top of panel p.  A third stage
-    // (loads two panels ahead) was measured 1-5 % slower on every tile shape; the kernel
-    // keeps the general ring so that the depth stays a one-line choice.
+    // Two stages: the loads of panel p+1 are issued during panel p.  Deeper rings (three,
+    // four and six stages) were measured slower on large problems and on small ones alike.
     static constexpr int NSTAGE = 2;
-    static constexpr int DEPTH = NSTAGE - 1;
     static constexpr size_t SMEM = (size_t)NSTAGE * STAGE * sizeof(T);
 };
 
@@ -455,7 +453,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     constexpr int TM = Cfg::TM, TN = Cfg::TN, VM = Cfg::VM, VN = Cfg::VN;
     constexpr int PITCH_A = Cfg::PITCH_A, PITCH_B = Cfg::PITCH_B, STAGE = Cfg::STAGE;
     constexpr int VEC = Cfg::VEC, NG = Cfg::NG, A_ELEMS = Cfg::A_ELEMS, VNM = Cfg::VNM;
-    constexpr int NSTAGE = Cfg::NSTAGE, DEPTH = Cfg::DEPTH;
+    constexpr int NSTAGE = Cfg::NSTAGE;
     constexpr bool A_KLAY = Cfg::A_KLAY, B_KLAY = Cfg::B_KLAY;
 
     // Two workgroups that share a CU from the start run in lockstep and finish together; both
@@ -559,15 +557,12 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 for (int v = 0; v < NACC; ++v) acc[bn][bm][pp][v] = (R)0;
 
     if (n_panels > 0) {
-        // Software pipeline over panels: a ring of NSTAGE LDS stages, loads issued DEPTH =
-        // NSTAGE-1 panels ahead.  Panel kp lives in stage kp % NSTAGE.  The loads of panel
-        // kp+DEPTH go out at the top of panel kp into the stage whose last readers finished
+        // Software pipeline over panels: two LDS stages, panel kp lives in stage kp % 2.  The
+        // loads of panel kp+1 go out during panel kp into the stage whose last readers finished
         // before the barrier that ended panel kp-1.  Before the barrier that ends panel kp,
-        // each wave waits for its own loads of panel kp+1 (issued a panel earlier when
-        // DEPTH is 2).
+        // each wave waits for its own loads of panel kp+1.
         typedef typename Cfg::LoaderA LA;
         typedef typename Cfg::LoaderB LB;
-        constexpr int LOADS_PER_PANEL = LA::PER + LB::PER;  // vector-memory instructions per wave and panel
 
         auto stage_ptr = [&](int kp) -> T * { return smem + (kp % NSTAGE) * STAGE; };
         auto issue_panel = [&](int kp) __attribute__((always_inline)) {
@@ -581,11 +576,10 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         // complete, K tail cleared, barrier.
         // full_depth: the caller knows that the panel is not the last one of its K range, so
         // it has no tail.
-        auto publish_panel = [&](int kp, bool newer_in_flight, bool full_depth) __attribute__((always_inline)) {
+        auto publish_panel = [&](int kp, bool full_depth) __attribute__((always_inline)) {
             T *dst = stage_ptr(kp);
             const int k_valid = k_end - (k_begin + kp * BK);
-            if (newer_in_flight) __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(LOADS_PER_PANEL));
-            else __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0));
+            __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0));
             if (!full_depth && k_valid < BK) {
                 la.clear_k_tail(dst, tid, k_valid);
                 lb.clear_k_tail(dst + A_ELEMS, tid, k_valid);
@@ -602,26 +596,25 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         };
 
         issue_panel(0);
-        if (DEPTH == 2 && n_panels > 1) issue_panel(1);
-        publish_panel(0, DEPTH == 2 && n_panels > 1, false);
+        publish_panel(0, false);
 
         const int a_frag = wm * WM + j * VM;
         const int b_frag = wn * WN + j * VN;
         constexpr int STEPS = BK / KS;
 
-        // steady_tag: panel kp+DEPTH exists and panel kp+1 is not the last one - true for all
+        // steady_tag: panel kp+1 exists and is not the last one - true for all
         // but the last few panels, which lets the body run without a single branch.
         auto do_panel = [&](int kp, auto steady_tag) __attribute__((always_inline)) {
             constexpr bool steady = decltype(steady_tag)::value;
-            const bool issued = steady || kp + DEPTH < n_panels;
-            // The loads of panel kp+DEPTH are not issued here, all at once, but one by one behind
+            const bool issued = steady || kp + 1 < n_panels;
+            // The loads of panel kp+1 are not issued here, all at once, but one by one behind
             // the MFMAs of the first steps below, where their issue does not hold up this
             // wavefront's MFMAs (8192^3: FP32 144 -> 149 TFLOP/s, FP64 70.5 -> 74; 1024^3 FP32
             // 75 -> 81).  Only the descriptors are made here.
             __amdgpu_buffer_rsrc_t ra, rb;
-            T *dst_next = stage_ptr(kp + DEPTH);
+            T *dst_next = stage_ptr(kp + 1);
             if (issued) {
-                const int k0n = k_begin + (kp + DEPTH) * BK;
+                const int k0n = k_begin + (kp + 1) * BK;
                 const int64_t ao = a_off(k0n), bo = b_off(k0n);
                 ra = make_rsrc(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
                 rb = make_rsrc(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
@@ -750,15 +743,15 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 if (!LOADS_UP_FRONT && issued) issue_behind_step(s);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (steady || kp + 1 < n_panels) publish_panel(kp + 1, DEPTH == 2 && issued, steady);
+            if (steady || kp + 1 < n_panels) publish_panel(kp + 1, steady);
             else __syncthreads();
         };
         // Two panels per trip, so that the stage addresses of each copy are loop-invariant.
         // Taken branches cost a wavefront tens of cycles of instruction fetch, which shows as
         // idle MFMA time when only two wavefronts share a SIMD: the steady part of the loop is
-        // straight-line code, and the last panels (at most DEPTH + 2) run a general copy.
+        // straight-line code, and the last panels (at most three) run a general copy.
         auto k_loop = [&]() __attribute__((always_inline)) {
-            const int n_steady = n_panels - 1 - DEPTH > 0 ? ((n_panels - 1 - DEPTH) & ~1) : 0;
+            const int n_steady = n_panels > 2 ? ((n_panels - 2) & ~1) : 0;
             int kp = 0;
             for (; kp < n_steady; kp += 2) {
                 do_panel(kp, std::true_type());
