@@ -875,8 +875,18 @@ splitk_reduce_kernel(const T *ws, int64_t ws_ld, int64_t ws_slice, int splits, i
     const int m = (blockIdx.x % m_blocks) * 256 + threadIdx.x;
     const int n = blockIdx.x / m_blocks;
     if (m >= M || n >= N) return;
+    // partials are fetched eight at a time (independent loads) and added in split order
+    const T *w = ws + (int64_t)n * ws_ld + m;
     T s = T();
-    for (int i = 0; i < splits; ++i) s = el_add(s, ws[(int64_t)i * ws_slice + (int64_t)n * ws_ld + m]);
+    int i = 0;
+    for (; i + 8 <= splits; i += 8) {
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = w[(int64_t)(i + u) * ws_slice];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) s = el_add(s, v[u]);
+    }
+    for (; i < splits; ++i) s = el_add(s, w[(int64_t)i * ws_slice]);
     T *c = C + (int64_t)n * ldc + m;
     T r = el_scale(alpha, s);
     if (!el_is_zero(beta)) r = el_axpy(beta, *c, r);
@@ -898,7 +908,15 @@ __global__ void __launch_bounds__(256) tail_reduce_kernel(const GemmParams<T> p,
     if (p.tri_c && (p.tri_c == 1 ? m < n : m > n)) return;
     const T *w = p.ws + (int64_t)r * p.tail_slices * (bm * bn) + e;
     T s = T();
-    for (int i = 0; i < p.tail_slices; ++i) s = el_add(s, w[(int64_t)i * (bm * bn)]);
+    int i = 0;
+    for (; i + 4 <= p.tail_slices; i += 4) {  // four independent loads at a time, added in slice order
+        T v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = w[(int64_t)(i + u) * (bm * bn)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) s = el_add(s, v[u]);
+    }
+    for (; i < p.tail_slices; ++i) s = el_add(s, w[(int64_t)i * (bm * bn)]);
     T *c = p.C + (int64_t)n * p.ldc + m;
     T v = el_scale(p.alpha, s);
     const bool herm_diag = p.herm_c && m == n;
