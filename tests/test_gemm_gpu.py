@@ -280,3 +280,26 @@ def test_sliced_tail_integer_exact(gpu, dtype):
         st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, C, 7, ldc, tile=small_tile)
         assert st == 0
         np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex64, np.complex128])
+def test_many_workgroups_not_whole_rounds_integer_exact(gpu, dtype):
+    """More than 512 workgroups in a launch that is not a whole number of rounds: the launch in
+    which every other workgroup of the first round starts late, with and without a sliced tail.
+    Exact-integer data, smallest tile forced: 31 x 29 = 899 tiles (no slicing: the last round is
+    too full), 30 x 18 = 540 tiles (28 in the last round, sliced)."""
+    cplx = np.dtype(dtype).kind == "c"
+    alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
+    small_tile = {np.float32: 2, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
+    for (M, N, K), (tA, tB) in (((1950, 1830, 150), (NOTRANS, TRANS)), ((1900, 1150, 600), (TRANS, NOTRANS))):
+        lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
+        lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]
+        A = oracle.integers(na, 1, lim, dtype)
+        B = oracle.integers(nb, 2, lim, dtype)
+        C = oracle.integers(nc, 3, 8, dtype)
+        want = C.copy()
+        assert oracle.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, want, 7, ldc) == 0
+        for tile in (small_tile, None):
+            st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, C, 7, ldc, tile=tile)
+            assert st == 0
+            np.testing.assert_array_equal(got, want, err_msg="%dx%dx%d tile %s" % (M, N, K, tile))
