@@ -68,22 +68,24 @@ template <> struct Mma16<float> {
 // (The reference inverts whole 128 x 128 blocks, trtri/*.cpp; inverting only the 16 x 16
 // ones keeps the result much closer to plain substitution.)
 //
-// Leaf kernel: one workgroup = one diagonal block x CW = 32 right-hand sides, 16 wavefronts;
-// wavefront w owns equations [16w, 16w+16) as two 16 x 16 accumulator blocks (lane l:
-// right-hand side l%16 of each block, equations krow(l/16, v)).  Accumulator layout and
+// Leaf kernel: one workgroup = one diagonal block x CW = 16 or 32 right-hand sides, 16
+// wavefronts; wavefront w owns equations [16w, 16w+16) as CW/16 accumulator blocks of 16 x 16
+// (lane l: right-hand side l%16 of each block, equations krow(l/16, v)).  Accumulator layout and
 // MFMA "B" operand layout coincide, so Y_s feeds the MFMAs as it is and X_s goes to the
 // other wavefronts through LDS in the same per-lane order.  Step s: wavefronts w > s subtract
-// L_ws X_s (8 MFMAs each); wavefront s+1 then computes X_(s+1) (8 MFMAs) and publishes it
+// L_ws X_s (4 MFMAs per block); wavefront s+1 then computes X_(s+1) (4 per block) and publishes it
 // while the others are still updating; one barrier per step.
 // For side=left a right-hand side is a column of B; the panel moves between HBM and the
 // accumulator layout through an LDS staging area so that global accesses run along columns.
-template <typename T> struct TrsmLeaf {
+template <typename T, bool RIGHT = false> struct TrsmLeaf {
     typedef typename Elem<T>::Real R;
     static constexpr bool CPLX = Elem<T>::CPLX;
     static constexpr int NB = 256, IB = 16, NBLK = NB / IB, THREADS = 64 * NBLK;
-    // Right-hand sides per workgroup: complex elements cost four MFMAs per product and twice
-    // the staging space, so they take half as many.
-    static constexpr int CW = CPLX ? 16 : 32, NBK = CW / 16;
+    // Right-hand sides per workgroup.  16: two workgroups fit a CU and cover each other's
+    // serial solves (DTRSM left 2048: 0.36 -> 0.31 ms, 4096: 1.36 -> 1.28 ms, 8192 x 512: 1.52 ->
+    // 1.34 ms).  Side = right with real elements keeps 32: its right-hand sides are rows of B,
+    // and 16 of them are too short a run of memory (8192: 0.5 - 1.5 % slower with 16).
+    static constexpr int CW = (RIGHT && !CPLX) ? 32 : 16, NBK = CW / 16;
     static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;  // sub-blocks (bi,bj), bi >= bj, at bi*(bi+1)/2 + bj
     // Packed sub-block: PLANES x 64 lanes x 4 reals.  Real: the values.  Complex: real parts,
     // imaginary parts, negated imaginary parts (so that no sign has to be flipped in the solve).
@@ -197,7 +199,7 @@ template <typename T, bool RIGHT, bool FORWARD>
 __global__ void __launch_bounds__(TrsmLeaf<T>::THREADS)
 trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk,
                  int64_t ldb, int nrhs) {
-    typedef TrsmLeaf<T> L;
+    typedef TrsmLeaf<T, RIGHT> L;
     typedef typename Elem<T>::Real R;
     typedef Mma16<R> M;
     typedef typename M::Acc Acc;
@@ -429,14 +431,13 @@ template <typename T> struct TrsmDriver {
         return hipGetLastError();
     }
 
-    hipError_t leaf(int i0, int nb, T alpha) {
-        const int nrhs = right ? M : N;
-        T *Bblk = right ? B + (int64_t)i0 * ldb : B + i0;
-        typedef TrsmLeaf<T> L;
+    template <bool RIGHT> hipError_t leaf_side(int i0, int nb, T alpha) {
+        typedef TrsmLeaf<T, RIGHT> L;
+        const int nrhs = RIGHT ? M : N;
+        T *Bblk = RIGHT ? B + (int64_t)i0 * ldb : B + i0;
         const R *packed = pack + (int64_t)(i0 / NBL) * L::PACK_REALS;
-        void (*fn)(const R *, int, T, T *, int64_t, int);
-        if (right) fn = forward ? trsm_diag_kernel<T, true, true> : trsm_diag_kernel<T, true, false>;
-        else fn = forward ? trsm_diag_kernel<T, false, true> : trsm_diag_kernel<T, false, false>;
+        void (*fn)(const R *, int, T, T *, int64_t, int) =
+            forward ? trsm_diag_kernel<T, RIGHT, true> : trsm_diag_kernel<T, RIGHT, false>;
         if (L::SMEM > 64 * 1024) {
             hipError_t e = ensure_dynamic_lds((const void *)fn, L::SMEM);
             if (e != hipSuccess) return e;
@@ -445,6 +446,7 @@ template <typename T> struct TrsmDriver {
         hipLaunchKernelGGL(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs);
         return hipGetLastError();
     }
+    hipError_t leaf(int i0, int nb, T alpha) { return right ? leaf_side<true>(i0, nb, alpha) : leaf_side<false>(i0, nb, alpha); }
 
     // Off-diagonal update of the block range `dst` (length nd, start d0) with the solved
     // range `src` (length ns, start s0):   B_dst <- beta * B_dst - coupling * X_src.
