@@ -347,7 +347,6 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     for (int s = 0; s < NBLK; ++s) {
         if (s < nsteps) {  // uniform over the workgroup
             const R *Xs = X + (s & 1) * (NP * NBK * 64 * 4);
-            if (s + RING - 1 <= wave && wave < nsteps) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
             if (wave > s && wave < nsteps) {
                 Acc xb[NP][NBK];
 #pragma unroll
@@ -356,8 +355,11 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                     for (int k = 0; k < NBK; ++k)
                         xb[pp][k] = *reinterpret_cast<const Acc *>(Xs + ((pp * NBK + k) * 64 + lane) * 4);
                 block_mma(ea[s % RING], xb, y);
+                __builtin_amdgcn_sched_barrier(0);
                 if (wave == s + 1) solve_row(s + 1);
             }
+            // requested behind this step's MFMAs, into the ring slot that step s-1 used
+            if (s + RING - 1 <= wave && wave < nsteps) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
             __syncthreads();
         }
     }
