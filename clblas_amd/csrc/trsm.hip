@@ -347,6 +347,11 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     for (int s = 0; s < NBLK; ++s) {
         if (s < nsteps) {  // uniform over the workgroup
             const R *Xs = X + (s & 1) * (NP * NBK * 64 * 4);
+            // Sub-block (wave, s+RING-1) goes into the ring slot that step s-1 used.  With a ring
+            // of two it is the one solve_row(s+1) needs below, so it is requested first; with
+            // three it is requested behind this step's MFMAs.
+            const bool fetch = s + RING - 1 <= wave && wave < nsteps;
+            if (RING == 2 && fetch) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
             if (wave > s && wave < nsteps) {
                 Acc xb[NP][NBK];
 #pragma unroll
@@ -358,8 +363,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                 __builtin_amdgcn_sched_barrier(0);
                 if (wave == s + 1) solve_row(s + 1);
             }
-            // requested behind this step's MFMAs, into the ring slot that step s-1 used
-            if (s + RING - 1 <= wave && wave < nsteps) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
+            if (RING > 2 && fetch) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
             __syncthreads();
         }
     }
