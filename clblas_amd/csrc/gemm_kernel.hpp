@@ -576,7 +576,8 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         // complete, K tail cleared, barrier.
         // full_depth: the caller knows that the panel is not the last one of its K range, so
         // it has no tail.
-        auto publish_panel = [&](int kp, bool full_depth) __attribute__((always_inline)) {
+        // masks: an operand is triangular (TRI kernels only).
+        auto publish_panel = [&](int kp, bool full_depth, bool masks) __attribute__((always_inline)) {
             T *dst = stage_ptr(kp);
             const int k_valid = k_end - (k_begin + kp * BK);
             __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0));
@@ -584,7 +585,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 la.clear_k_tail(dst, tid, k_valid);
                 lb.clear_k_tail(dst + A_ELEMS, tid, k_valid);
             }
-            if (TRI) {
+            if (TRI && masks) {
                 // Only the panels that meet the diagonal (or the zero side of it) need the fix-up.
                 const int k0 = k_begin + kp * BK;
                 if ((p.tri_a == 1 && k0 + BK > m0) || (p.tri_a == 2 && k0 < m0 + BM))
@@ -596,7 +597,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
         };
 
         issue_panel(0);
-        publish_panel(0, false);
+        publish_panel(0, false, true);
 
         const int a_frag = wm * WM + j * VM;
         const int b_frag = wn * WN + j * VN;
@@ -604,8 +605,9 @@ gemm_mfma_kernel(const GemmParams<T> p) {
 
         // steady_tag: panel kp+1 exists and is not the last one - true for all
         // but the last few panels, which lets the body run without a single branch.
-        auto do_panel = [&](int kp, auto steady_tag) __attribute__((always_inline)) {
+        auto do_panel = [&](int kp, auto steady_tag, auto masks_tag) __attribute__((always_inline)) {
             constexpr bool steady = decltype(steady_tag)::value;
+            constexpr bool masks = decltype(masks_tag)::value;
             const bool issued = steady || kp + 1 < n_panels;
             // The loads of panel kp+1 are not issued here, all at once, but one by one behind
             // the MFMAs of the first steps below, where their issue does not hold up this
@@ -743,23 +745,26 @@ gemm_mfma_kernel(const GemmParams<T> p) {
                 if (!LOADS_UP_FRONT && issued) issue_behind_step(s);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (steady || kp + 1 < n_panels) publish_panel(kp + 1, steady);
+            if (steady || kp + 1 < n_panels) publish_panel(kp + 1, steady, masks);
             else __syncthreads();
         };
         // Two panels per trip, so that the stage addresses of each copy are loop-invariant.
         // Taken branches cost a wavefront tens of cycles of instruction fetch, which shows as
         // idle MFMA time when only two wavefronts share a SIMD: the steady part of the loop is
         // straight-line code, and the last panels (at most three) run a general copy.
-        auto k_loop = [&]() __attribute__((always_inline)) {
+        auto k_loop = [&](auto masks_tag) __attribute__((always_inline)) {
             const int n_steady = n_panels > 2 ? ((n_panels - 2) & ~1) : 0;
             int kp = 0;
             for (; kp < n_steady; kp += 2) {
-                do_panel(kp, std::true_type());
-                do_panel(kp + 1, std::true_type());
+                do_panel(kp, std::true_type(), masks_tag);
+                do_panel(kp + 1, std::true_type(), masks_tag);
             }
-            for (; kp < n_panels; ++kp) do_panel(kp, std::false_type());
+            for (; kp < n_panels; ++kp) do_panel(kp, std::false_type(), masks_tag);
         };
-        k_loop();
+        // A triangular operand puts tests (and now and then a fix-up) between the panels; the
+        // other users of the TRI kernels - a triangle of C, sliced tails - keep the straight line.
+        if (TRI && (p.tri_a || p.tri_b)) k_loop(std::true_type());
+        else k_loop(std::false_type());
     }
 
     // ---- epilogue ----
