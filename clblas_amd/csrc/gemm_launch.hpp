@@ -262,13 +262,15 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             fn = e.splitk[idx];
         }
     }
-    // The late start that keeps the workgroups of a CU out of lockstep when the launch is not a
-    // whole number of rounds of 2 x 256 workgroups (see the kernel; 3584^3 FP64: 54 -> 69 TFLOP/s).
+    // The late start that keeps the workgroups of a CU out of lockstep (see the kernel).  Needed when
+    // the launch is not a whole number of rounds of 2 x 256 workgroups (3584^3 FP64: 54 -> 69 TFLOP/s);
+    // with short K ranges it also pays in whole rounds, because the epilogue of one workgroup then
+    // overlaps the K loop of its neighbour (8192 x 8192 x 512 FP64: 66.9 -> 68.2; x 8192: -0.3 %).
     {
         const int64_t wgs = grid_x * (splits > 1 ? splits : 1);
         const bool whole_rounds = p.tail_slices <= 1 && wgs % 512 == 0;
-        p.stagger = wgs > 512 && !whole_rounds && !(p.tri_a || p.tri_b) &&
-                    debug_env_int("CLBLAS_AMD_GEMM_STAGGER", 1) != 0;
+        const int mode = debug_env_int("CLBLAS_AMD_GEMM_STAGGER", 1);  // 0: never
+        p.stagger = mode != 0 && wgs > 512 && !(p.tri_a || p.tri_b) && (!whole_rounds || p.k_per_split <= 2048);
     }
     const size_t smem = e.smem_of[idx];
     if (smem > 64 * 1024) {
