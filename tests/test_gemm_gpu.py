@@ -17,7 +17,7 @@ from helpers import (COL, ROW, NOTRANS, TRANS, CONJ, buf_len, exact_int_limits, 
 pytestmark = pytest.mark.gpu
 
 DT = {"f32": np.float32, "f64": np.float64}
-N_TILES = {np.float32: 3, np.float64: 2}
+N_TILES = {np.float32: 4, np.float64: 2}
 
 
 @pytest.fixture(scope="module")
@@ -268,7 +268,7 @@ def test_sliced_tail_integer_exact(gpu, dtype):
     M, N, K = 1100, 1000, 520
     cplx = np.dtype(dtype).kind == "c"
     alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
-    small_tile = {np.float32: 2, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
+    small_tile = {np.float32: 3, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
     for tA, tB in ((NOTRANS, NOTRANS), (TRANS, CONJ)):
         lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
         lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]
@@ -290,7 +290,7 @@ def test_many_workgroups_not_whole_rounds_integer_exact(gpu, dtype):
     too full), 30 x 18 = 540 tiles (28 in the last round, sliced)."""
     cplx = np.dtype(dtype).kind == "c"
     alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
-    small_tile = {np.float32: 2, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
+    small_tile = {np.float32: 3, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
     for (M, N, K), (tA, tB) in (((1950, 1830, 150), (NOTRANS, TRANS)), ((1900, 1150, 600), (TRANS, NOTRANS))):
         lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
         lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]
