@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
@@ -259,6 +259,44 @@ def main():
             del A, B, B0, C, T
         lv["workload"] = "column-major, lower, left, no transpose, N=M=K=%d, alpha=beta=1 (complex: alpha=1+0.5i)" % n
         extra["level3"] = lv
+
+    # ---- BASELINE configs 1 and 3: SGEMM 1024^3 and the edge-shape sweep (ld = rows + 3, offsets 5/7/11,
+    #      alpha = 0.7, beta = -1.3, all four transposes).  Each against its own bound: MFMA time and HBM time
+    #      of the algorithmic bytes 4 (MK + KN + 2 MN). ----
+    if args.only in ("", "configs"):
+        shapes = {}
+
+        def sgemm_case(M, N, K, tA, tB, alpha, beta, pad, offs):
+            ra, ca = (K, M) if tA else (M, K)   # rows x columns as stored (column-major)
+            rb, cb = (N, K) if tB else (K, N)
+            lda, ldb, ldc = ra + pad, rb + pad, M + pad
+            A = torch.rand(offs[0] + lda * ca, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+            B = torch.rand(offs[1] + ldb * cb, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+            C = torch.rand(offs[2] + ldc * N, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+
+            def call():
+                st = clblas_amd.sgemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2],
+                                      ldc)
+                if st != 0:
+                    raise RuntimeError("clblasSgemm returned %d" % st)
+            reps = 10 if 2.0 * M * N * K > 1e10 else 50
+            wall, ev_ms = timed_calls(torch, call, reps, 3)
+            return ev_ms
+
+        ms = sgemm_case(1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0))
+        shapes["config1 1024x1024x1024 NN"] = {"ms": round(ms, 4), "tflops": round(2.0 * 1024 ** 3 / ms / 1e9, 2)}
+        for (M, N, K) in ((4097, 4095, 1031), (65536, 64, 4096), (64, 65536, 4096), (127, 129, 8192)):
+            flops = 2.0 * M * N * K
+            nbytes = 4.0 * (M * K + K * N + 2.0 * M * N)
+            row = {"mfma_bound_ms": round(flops / (PEAK_FP32_MATRIX * 1e12) * 1e3, 4),
+                   "hbm_bound_ms": round(nbytes / 8e12 * 1e3, 4)}
+            for tA, tB, tag in ((NOTRANS, NOTRANS, "NN"), (NOTRANS, TRANS, "NT"), (TRANS, NOTRANS, "TN"),
+                                (TRANS, TRANS, "TT")):
+                ms = sgemm_case(M, N, K, tA, tB, 0.7, -1.3, 3, (5, 7, 11))
+                row[tag] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2),
+                            "GBps": round(nbytes / ms / 1e6, 1)}
+            shapes["config3 %dx%dx%d" % (M, N, K)] = row
+        extra["sgemm_configs_1_and_3"] = shapes
 
     # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
     cpu = None
