@@ -322,6 +322,11 @@ static_assert(sizeof(FloatComplex) == sizeof(cba::Cx<float>) && sizeof(DoubleCom
               "complex layouts must agree");
 inline cba::Cx<float> cx(FloatComplex z) { return cba::Cx<float>{z.s[0], z.s[1]}; }
 inline cba::Cx<double> cx(DoubleComplex z) { return cba::Cx<double>{z.s[0], z.s[1]}; }
+// Interleaved (re, im) arrays: the same memory seen through the kernels' element type.
+inline const cba::Cx<float> *cx(const FloatComplex *p) { return reinterpret_cast<const cba::Cx<float> *>(p); }
+inline cba::Cx<float> *cx(FloatComplex *p) { return reinterpret_cast<cba::Cx<float> *>(p); }
+inline const cba::Cx<double> *cx(const DoubleComplex *p) { return reinterpret_cast<const cba::Cx<double> *>(p); }
+inline cba::Cx<double> *cx(DoubleComplex *p) { return reinterpret_cast<cba::Cx<double> *>(p); }
 
 template <typename T>
 clblasStatus trsm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
@@ -386,207 +391,216 @@ clblasStatus clblasSetup(void) {
 void clblasTeardown(void) { cba::workspace_release_all(); }
 
 clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
-                         size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B,
-                         size_t offB, size_t ldb, float beta, float *C, size_t offC, size_t ldc,
-                         hipStream_t stream) {
-    return gemm_front<float>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb,
-                             beta, C, offC, ldc, stream);
+                         size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B, size_t offB,
+                         size_t ldb, float beta, float *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return gemm_front<float>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc,
+                             stream);
 }
 
 clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
                          size_t K, double alpha, const double *A, size_t offA, size_t lda, const double *B,
                          size_t offB, size_t ldb, double beta, double *C, size_t offC, size_t ldc,
                          hipStream_t stream) {
-    return gemm_front<double>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB,
-                              ldb, beta, C, offC, ldc, stream);
+    return gemm_front<double>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc,
+                              stream);
 }
 
 clblasStatus clblasCgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
                          size_t K, FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
                          const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta, FloatComplex *C,
                          size_t offC, size_t ldc, hipStream_t stream) {
-    typedef cba::Cx<float> E;
-    return gemm_front<E>(order, transA, transB, M, N, K, cx(alpha),
-                         reinterpret_cast<const E *>(A), offA, lda, reinterpret_cast<const E *>(B), offB, ldb,
-                         cx(beta), reinterpret_cast<E *>(C), offC, ldc, stream);
+    return gemm_front<cba::Cx<float>>(order, transA, transB, M, N, K, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                      cx(beta), cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasZgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
                          size_t K, DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
                          const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta, DoubleComplex *C,
                          size_t offC, size_t ldc, hipStream_t stream) {
-    typedef cba::Cx<double> E;
-    return gemm_front<E>(order, transA, transB, M, N, K, cx(alpha),
-                         reinterpret_cast<const E *>(A), offA, lda, reinterpret_cast<const E *>(B), offB, ldb,
-                         cx(beta), reinterpret_cast<E *>(C), offC, ldc, stream);
+    return gemm_front<cba::Cx<double>>(order, transA, transB, M, N, K, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                       cx(beta), cx(C), offC, ldc, stream);
 }
 
-clblasStatus clblasStrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, float alpha, const float *A, size_t offA, size_t lda,
-                         float *B, size_t offB, size_t ldb, hipStream_t stream) {
-    return trsm_front<float>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
-                             offB, ldb, stream);
+clblasStatus clblasStrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, float alpha, const float *A, size_t offA, size_t lda, float *B,
+                         size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<float>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream);
 }
 
-clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, double alpha, const double *A, size_t offA,
-                         size_t lda, double *B, size_t offB, size_t ldb, hipStream_t stream) {
-    return trsm_front<double>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B,
-                              offB, ldb, stream);
+clblasStatus clblasDtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, double alpha, const double *A, size_t offA, size_t lda, double *B,
+                         size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<double>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream);
 }
 
-clblasStatus clblasCtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, FloatComplex alpha, const FloatComplex *A, size_t offA,
-                         size_t lda, FloatComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
-    return trsm_front<cba::Cx<float>>(order, side, uplo, transA, diag, M, N, cx(alpha),
-                                      reinterpret_cast<const cba::Cx<float> *>(A), offA, lda,
-                                      reinterpret_cast<cba::Cx<float> *>(B), offB, ldb, stream);
+clblasStatus clblasCtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                         FloatComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<cba::Cx<float>>(order, side, uplo, transA, diag, M, N, cx(alpha), cx(A), offA, lda, cx(B), offB,
+                                      ldb, stream);
 }
 
-clblasStatus clblasZtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, DoubleComplex alpha, const DoubleComplex *A, size_t offA,
-                         size_t lda, DoubleComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
-    return trsm_front<cba::Cx<double>>(order, side, uplo, transA, diag, M, N, cx(alpha),
-                                       reinterpret_cast<const cba::Cx<double> *>(A), offA, lda,
-                                       reinterpret_cast<cba::Cx<double> *>(B), offB, ldb, stream);
+clblasStatus clblasZtrsm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                         DoubleComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trsm_front<cba::Cx<double>>(order, side, uplo, transA, diag, M, N, cx(alpha), cx(A), offA, lda, cx(B),
+                                       offB, ldb, stream);
 }
 
-clblasStatus clblasSsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
-                         float alpha, const float *A, size_t offA, size_t lda, float beta, float *C, size_t offC, size_t ldc,
+clblasStatus clblasSsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, float alpha,
+                         const float *A, size_t offA, size_t lda, float beta, float *C, size_t offC, size_t ldc,
                          hipStream_t stream) {
     return syrk_front<float>(order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, stream);
 }
 
-clblasStatus clblasStrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, float alpha, const float *A, size_t offA, size_t lda, float *B,
+clblasStatus clblasStrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, float alpha, const float *A, size_t offA, size_t lda, float *B,
                          size_t offB, size_t ldb, hipStream_t stream) {
     return trmm_front<float>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream);
 }
 
 clblasStatus clblasSsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, float alpha,
-                         const float *A, size_t offA, size_t lda, const float *B, size_t offB, size_t ldb, float beta, float *C,
-                         size_t offC, size_t ldc, hipStream_t stream) {
+                         const float *A, size_t offA, size_t lda, const float *B, size_t offB, size_t ldb, float beta,
+                         float *C, size_t offC, size_t ldc, hipStream_t stream) {
     return symm_front<float>(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
 }
 
-clblasStatus clblasDsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
-                         double alpha, const double *A, size_t offA, size_t lda, double beta, double *C, size_t offC, size_t ldc,
+clblasStatus clblasDsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, double alpha,
+                         const double *A, size_t offA, size_t lda, double beta, double *C, size_t offC, size_t ldc,
                          hipStream_t stream) {
     return syrk_front<double>(order, uplo, transA, N, K, alpha, A, offA, lda, beta, C, offC, ldc, stream);
 }
 
-clblasStatus clblasDtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, double alpha, const double *A, size_t offA, size_t lda, double *B,
+clblasStatus clblasDtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, double alpha, const double *A, size_t offA, size_t lda, double *B,
                          size_t offB, size_t ldb, hipStream_t stream) {
     return trmm_front<double>(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, stream);
 }
 
 clblasStatus clblasDsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, double alpha,
-                         const double *A, size_t offA, size_t lda, const double *B, size_t offB, size_t ldb, double beta, double *C,
-                         size_t offC, size_t ldc, hipStream_t stream) {
+                         const double *A, size_t offA, size_t lda, const double *B, size_t offB, size_t ldb,
+                         double beta, double *C, size_t offC, size_t ldc, hipStream_t stream) {
     return symm_front<double>(order, side, uplo, M, N, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
 }
 
 clblasStatus clblasCsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
-                         FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, FloatComplex beta, FloatComplex *C, size_t offC, size_t ldc,
-                         hipStream_t stream) {
-    return syrk_front<cba::Cx<float>>(order, uplo, transA, N, K, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, cx(beta), reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+                         FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, FloatComplex beta,
+                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syrk_front<cba::Cx<float>>(order, uplo, transA, N, K, cx(alpha), cx(A), offA, lda, cx(beta), cx(C), offC,
+                                      ldc, stream);
 }
 
-clblasStatus clblasCtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, FloatComplex *B,
-                         size_t offB, size_t ldb, hipStream_t stream) {
-    return trmm_front<cba::Cx<float>>(order, side, uplo, transA, diag, M, N, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<cba::Cx<float> *>(B), offB, ldb, stream);
+clblasStatus clblasCtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda,
+                         FloatComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trmm_front<cba::Cx<float>>(order, side, uplo, transA, diag, M, N, cx(alpha), cx(A), offA, lda, cx(B), offB,
+                                      ldb, stream);
 }
 
 clblasStatus clblasCsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, FloatComplex alpha,
-                         const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta, FloatComplex *C,
-                         size_t offC, size_t ldc, hipStream_t stream) {
-    return symm_front<cba::Cx<float>>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+                         const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB,
+                         size_t ldb, FloatComplex beta, FloatComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return symm_front<cba::Cx<float>>(order, side, uplo, M, N, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                      cx(beta), cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasZsyrk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K,
-                         DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, DoubleComplex beta, DoubleComplex *C, size_t offC, size_t ldc,
-                         hipStream_t stream) {
-    return syrk_front<cba::Cx<double>>(order, uplo, transA, N, K, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, cx(beta), reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+                         DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, DoubleComplex beta,
+                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syrk_front<cba::Cx<double>>(order, uplo, transA, N, K, cx(alpha), cx(A), offA, lda, cx(beta), cx(C), offC,
+                                       ldc, stream);
 }
 
-clblasStatus clblasZtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
-                         clblasDiag diag, size_t M, size_t N, DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, DoubleComplex *B,
-                         size_t offB, size_t ldb, hipStream_t stream) {
-    return trmm_front<cba::Cx<double>>(order, side, uplo, transA, diag, M, N, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<cba::Cx<double> *>(B), offB, ldb, stream);
+clblasStatus clblasZtrmm(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA, clblasDiag diag,
+                         size_t M, size_t N, DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                         DoubleComplex *B, size_t offB, size_t ldb, hipStream_t stream) {
+    return trmm_front<cba::Cx<double>>(order, side, uplo, transA, diag, M, N, cx(alpha), cx(A), offA, lda, cx(B),
+                                       offB, ldb, stream);
 }
 
 clblasStatus clblasZsymm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, DoubleComplex alpha,
-                         const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta, DoubleComplex *C,
-                         size_t offC, size_t ldc, hipStream_t stream) {
-    return symm_front<cba::Cx<double>>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+                         const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB,
+                         size_t ldb, DoubleComplex beta, DoubleComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return symm_front<cba::Cx<double>>(order, side, uplo, M, N, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                       cx(beta), cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasSsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
-                          float alpha, const float *A, size_t offA, size_t lda, const float *B, size_t offB, size_t ldb,
-                          float beta, float *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return syr2k_front<float>(order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
+                          float alpha, const float *A, size_t offA, size_t lda, const float *B, size_t offB,
+                          size_t ldb, float beta, float *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syr2k_front<float>(order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc,
+                              stream);
 }
 
 clblasStatus clblasDsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
-                          double alpha, const double *A, size_t offA, size_t lda, const double *B, size_t offB, size_t ldb,
-                          double beta, double *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return syr2k_front<double>(order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream);
+                          double alpha, const double *A, size_t offA, size_t lda, const double *B, size_t offB,
+                          size_t ldb, double beta, double *C, size_t offC, size_t ldc, hipStream_t stream) {
+    return syr2k_front<double>(order, uplo, transAB, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc,
+                               stream);
 }
 
 clblasStatus clblasCsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
-                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb,
-                          FloatComplex beta, FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return syr2k_front<cba::Cx<float>>(order, uplo, transAB, N, K, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B,
+                          size_t offB, size_t ldb, FloatComplex beta, FloatComplex *C, size_t offC, size_t ldc,
+                          hipStream_t stream) {
+    return syr2k_front<cba::Cx<float>>(order, uplo, transAB, N, K, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                       cx(beta), cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasZsyr2k(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K,
-                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb,
-                          DoubleComplex beta, DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return syr2k_front<cba::Cx<double>>(order, uplo, transAB, N, K, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, cx(beta), reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                          const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta, DoubleComplex *C,
+                          size_t offC, size_t ldc, hipStream_t stream) {
+    return syr2k_front<cba::Cx<double>>(order, uplo, transAB, N, K, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                        cx(beta), cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasCherk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, float alpha,
-                         const FloatComplex *A, size_t offA, size_t lda, float beta, FloatComplex *C, size_t offC, size_t ldc,
-                         hipStream_t stream) {
-    return herk_front<float>(false, order, uplo, transA, N, K, cba::Cx<float>{alpha, 0}, reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, nullptr, 0, 0, beta,
-                          reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+                         const FloatComplex *A, size_t offA, size_t lda, float beta, FloatComplex *C, size_t offC,
+                         size_t ldc, hipStream_t stream) {
+    return herk_front<float>(false, order, uplo, transA, N, K, cba::Cx<float>{alpha, 0}, cx(A), offA, lda, nullptr, 0,
+                             0, beta, cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasCher2k(clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
-                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb,
-                          float beta, FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return herk_front<float>(true, order, uplo, trans, N, K, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, beta,
-                          reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+                          FloatComplex alpha, const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B,
+                          size_t offB, size_t ldb, float beta, FloatComplex *C, size_t offC, size_t ldc,
+                          hipStream_t stream) {
+    return herk_front<float>(true, order, uplo, trans, N, K, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb, beta,
+                             cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasChemm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, FloatComplex alpha,
-                         const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB, size_t ldb, FloatComplex beta,
-                         FloatComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return symm_front<cba::Cx<float>, true>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<float> *>(A), offA, lda, reinterpret_cast<const cba::Cx<float> *>(B), offB, ldb, cx(beta),
-                                reinterpret_cast<cba::Cx<float> *>(C), offC, ldc, stream);
+                         const FloatComplex *A, size_t offA, size_t lda, const FloatComplex *B, size_t offB,
+                         size_t ldb, FloatComplex beta, FloatComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return symm_front<cba::Cx<float>, true>(order, side, uplo, M, N, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                            cx(beta), cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasZherk(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, double alpha,
-                         const DoubleComplex *A, size_t offA, size_t lda, double beta, DoubleComplex *C, size_t offC, size_t ldc,
-                         hipStream_t stream) {
-    return herk_front<double>(false, order, uplo, transA, N, K, cba::Cx<double>{alpha, 0}, reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, nullptr, 0, 0, beta,
-                          reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+                         const DoubleComplex *A, size_t offA, size_t lda, double beta, DoubleComplex *C, size_t offC,
+                         size_t ldc, hipStream_t stream) {
+    return herk_front<double>(false, order, uplo, transA, N, K, cba::Cx<double>{alpha, 0}, cx(A), offA, lda, nullptr,
+                              0, 0, beta, cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasZher2k(clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
-                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb,
-                          double beta, DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return herk_front<double>(true, order, uplo, trans, N, K, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, beta,
-                          reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+                          DoubleComplex alpha, const DoubleComplex *A, size_t offA, size_t lda,
+                          const DoubleComplex *B, size_t offB, size_t ldb, double beta, DoubleComplex *C, size_t offC,
+                          size_t ldc, hipStream_t stream) {
+    return herk_front<double>(true, order, uplo, trans, N, K, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb, beta,
+                              cx(C), offC, ldc, stream);
 }
 
 clblasStatus clblasZhemm(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, DoubleComplex alpha,
-                         const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
-                         DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream) {
-    return symm_front<cba::Cx<double>, true>(order, side, uplo, M, N, cx(alpha), reinterpret_cast<const cba::Cx<double> *>(A), offA, lda, reinterpret_cast<const cba::Cx<double> *>(B), offB, ldb, cx(beta),
-                                reinterpret_cast<cba::Cx<double> *>(C), offC, ldc, stream);
+                         const DoubleComplex *A, size_t offA, size_t lda, const DoubleComplex *B, size_t offB,
+                         size_t ldb, DoubleComplex beta, DoubleComplex *C, size_t offC, size_t ldc,
+                         hipStream_t stream) {
+    return symm_front<cba::Cx<double>, true>(order, side, uplo, M, N, cx(alpha), cx(A), offA, lda, cx(B), offB, ldb,
+                                             cx(beta), cx(C), offC, ldc, stream);
 }
 
 }  // extern "C"
