@@ -17,6 +17,7 @@ template <typename T> struct TileEntry {
     size_t smem_of[4];
     bool has_splitk;
     double eff;      // measured fraction of MFMA peak on large problems (tile choice model)
+    double alone;    // further factor when a workgroup has its CU to itself (at most 256 tiles)
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
     void (*plain[4])(const GemmParams<T>);
     void (*splitk[4])(const GemmParams<T>);
@@ -25,10 +26,10 @@ template <typename T> struct TileEntry {
 
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false>
-TileEntry<T> make_tile_entry(double eff) {
+TileEntry<T> make_tile_entry(double eff, double alone = 0.85) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
-    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
     e.smem_of[0] = GemmCfg<T, BM, BN, BK, WM, WN, false, true>::SMEM;
     e.smem_of[1] = GemmCfg<T, BM, BN, BK, WM, WN, false, false>::SMEM;
@@ -128,7 +129,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             // tiles 0.77 ms, 128x128 0.60 ms, 64x64 0.67 ms).
             if (tri_operand) rounds = (double)t / (2.0 * kCUs) + 0.4;
             double cost = rounds * tab[i].bm * tab[i].bn / tab[i].eff;
-            if (t <= kCUs) cost /= 0.85;  // a workgroup alone on its CU cannot keep the MFMA pipes full
+            if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             if (!have || cost < best) { best = cost; pick = i; have = true; }
         }
     }

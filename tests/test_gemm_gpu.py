@@ -17,7 +17,7 @@ from helpers import (COL, ROW, NOTRANS, TRANS, CONJ, buf_len, exact_int_limits, 
 pytestmark = pytest.mark.gpu
 
 DT = {"f32": np.float32, "f64": np.float64}
-N_TILES = {np.float32: 4, np.float64: 2}
+N_TILES = {np.float32: 5, np.float64: 2}
 
 
 @pytest.fixture(scope="module")
@@ -264,11 +264,12 @@ def test_two_streams_and_teardown(gpu):
 def test_sliced_tail_integer_exact(gpu, dtype):
     """More than 256 tiles with a partly filled last round: the tiles of that round are cut into
     K slices and finished by a reduction pass.  Exact-integer data, smallest tile forced so that
-    a modest problem has 18 x 16 = 288 tiles (32 in the last round, 4 slices of K = 520)."""
+    a modest problem has 18 x 16 = 288 tiles (32 in the last round, K = 520 in 2 to 8 slices,
+    by the panel depth of the type's smallest tile)."""
     M, N, K = 1100, 1000, 520
     cplx = np.dtype(dtype).kind == "c"
     alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
-    small_tile = {np.float32: 3, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
+    small_tile = {np.float32: 4, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
     for tA, tB in ((NOTRANS, NOTRANS), (TRANS, CONJ)):
         lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
         lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]
@@ -290,7 +291,7 @@ def test_many_workgroups_not_whole_rounds_integer_exact(gpu, dtype):
     too full), 30 x 18 = 540 tiles (28 in the last round, sliced)."""
     cplx = np.dtype(dtype).kind == "c"
     alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
-    small_tile = {np.float32: 3, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
+    small_tile = {np.float32: 4, np.float64: 1, np.complex64: 1, np.complex128: 1}[dtype]
     for (M, N, K), (tA, tB) in (((1950, 1830, 150), (NOTRANS, TRANS)), ((1900, 1150, 600), (TRANS, NOTRANS))):
         lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
         lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]
