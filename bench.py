@@ -59,6 +59,25 @@ def timed_calls(torch, call, steps, warmup, before_each=None):
     return wall, ev_ms
 
 
+def timed_batch(torch, call, reps, warmup, batches=3):
+    """Mean milliseconds per call of `reps` back-to-back calls between one pair of HIP events (best
+    of `batches`): for launches of tens of microseconds, where an event pair per call would be
+    a good part of what is measured."""
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    best = float("inf")
+    for _ in range(batches):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            call()
+        stop.record()
+        torch.cuda.synchronize()
+        best = min(best, start.elapsed_time(stop) / reps)
+    return best
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -66,8 +85,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm or copy (profiling; copy = a plain "
-                    "1 GiB device copy used to scale the HBM traffic counters)")
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs or copy (profiling; "
+                    "copy = a plain 1 GiB device copy used to scale the HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (one MI355X per box); use --gpus 1")
@@ -279,9 +298,7 @@ def main():
                                       ldc)
                 if st != 0:
                     raise RuntimeError("clblasSgemm returned %d" % st)
-            reps = 10 if 2.0 * M * N * K > 1e10 else 50
-            wall, ev_ms = timed_calls(torch, call, reps, 3)
-            return ev_ms
+            return timed_batch(torch, call, 20 if 2.0 * M * N * K > 1e10 else 100, 5)
 
         ms = sgemm_case(1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0))
         shapes["config1 1024x1024x1024 NN"] = {"ms": round(ms, 4), "tflops": round(2.0 * 1024 ** 3 / ms / 1e9, 2)}
