@@ -11,14 +11,17 @@ namespace cba {
 //      from HBM needs (depth 16: 114.6), and let a workgroup that is alone on its CU run at full rate
 //      (16384 x 128 x 2048: 126 against 117 with depth 16); the larger tiles lose residency with them.
 //   3:  64x128x32, wave 32x64: the mirror image for wide C (64 x 65536 x 4096: 116 against 107)
+//      Tiles 2 and 3 are not offered to products with a triangular operand: the round model for those
+//      was fitted on the square tiles and picks the oblong ones where they lose (STRMM / SSYMM 3072:
+//      7-9 % slower with them).
 //   4:  64x64x32,  wave 32x32, split-K capable (small / deep-K problems; 1024^3: 94 against 86 with
 //      depth 16, 8192 x 64 x 8192: 106-112 against 91-94)
 static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, false, true>(0.920),
-        make_tile_entry<float, 128, 64, 32, 64, 32, 2, false, false>(0.92, 0.97),
-        make_tile_entry<float, 64, 128, 32, 32, 64, 2, false, false>(0.92, 0.97),
+        make_tile_entry<float, 128, 64, 32, 64, 32, 2, false, true>(0.92, 0.97, false),
+        make_tile_entry<float, 64, 128, 32, 32, 64, 2, false, true>(0.92, 0.97, false),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true>(0.84, 0.95),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

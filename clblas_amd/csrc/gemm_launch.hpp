@@ -18,6 +18,7 @@ template <typename T> struct TileEntry {
     bool has_splitk;
     double eff;      // measured fraction of MFMA peak on large problems (tile choice model)
     double alone;    // further factor when a workgroup has its CU to itself (at most 256 tiles)
+    bool tri_operands;  // eligible for products with a triangular A or B (TRMM, SYMM passes)
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
     void (*plain[4])(const GemmParams<T>);
     void (*splitk[4])(const GemmParams<T>);
@@ -26,10 +27,10 @@ template <typename T> struct TileEntry {
 
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false>
-TileEntry<T> make_tile_entry(double eff, double alone = 0.85) {
+TileEntry<T> make_tile_entry(double eff, double alone = 0.85, bool tri_operands = true) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
-    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone; e.tri_operands = tri_operands;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
     e.smem_of[0] = GemmCfg<T, BM, BN, BK, WM, WN, false, true>::SMEM;
     e.smem_of[1] = GemmCfg<T, BM, BN, BK, WM, WN, false, false>::SMEM;
@@ -119,6 +120,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         bool have = false;
         for (int i = 0; i < ntab; ++i) {
             if (need_tri && !tab[i].tri[0]) continue;
+            if (tri_operand && !tab[i].tri_operands) continue;
             const int64_t t = active_tiles(M, N, tab[i].bm, tab[i].bn, tri_c);
             double rounds = (double)ceil_div64(t, kCUs);
             const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
