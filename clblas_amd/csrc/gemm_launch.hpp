@@ -16,7 +16,11 @@ template <typename T> struct TileEntry {
     size_t smem;     // largest of the four variants (for the residency estimate)
     size_t smem_of[4];
     bool has_splitk;
-    double eff;      // measured fraction of MFMA peak on large problems (tile choice model)
+    // Tile choice model: fraction of MFMA peak the tile is credited with.  Fitted to the choices that
+    // measure best at 1000..5000, where the short K loops cost the small tiles more than at 8192^3
+    // (there the five FP32 tiles run at .953 / .943 / .93 / .915 / .88; crediting them with those
+    // figures moved 3000 x 1500 x 1000 from 105 to 98 TFLOP/s and 4097 x 4095 x 1031 from 125 to 122).
+    double eff;
     double alone;    // further factor when a workgroup has its CU to itself (at most 256 tiles)
     bool tri_operands;  // eligible for products with a triangular A or B (TRMM, SYMM passes)
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
