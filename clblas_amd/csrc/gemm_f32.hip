@@ -20,8 +20,8 @@ static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, false, true>(0.920),
-        make_tile_entry<float, 128, 64, 32, 64, 32, 2, false, true>(0.92, 0.97, false),
-        make_tile_entry<float, 64, 128, 32, 32, 64, 2, false, true>(0.92, 0.97, false),
+        make_tile_entry<float, 128, 64, 32, 64, 32, 2, false, true>(0.92, 0.97, 0.0),
+        make_tile_entry<float, 64, 128, 32, 32, 64, 2, false, true>(0.92, 0.97, 0.0),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true>(0.84, 0.95),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

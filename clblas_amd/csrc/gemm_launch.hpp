@@ -22,7 +22,7 @@ template <typename T> struct TileEntry {
     // figures moved 3000 x 1500 x 1000 from 105 to 98 TFLOP/s and 4097 x 4095 x 1031 from 125 to 122).
     double eff;
     double alone;    // further factor when a workgroup has its CU to itself (at most 256 tiles)
-    bool tri_operands;  // eligible for products with a triangular A or B (TRMM, SYMM passes)
+    double eff_tri;  // `eff` for products with a triangular A or B (TRMM, SYMM passes); 0: not offered
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
     void (*plain[4])(const GemmParams<T>);
     void (*splitk[4])(const GemmParams<T>);
@@ -31,10 +31,10 @@ template <typename T> struct TileEntry {
 
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false>
-TileEntry<T> make_tile_entry(double eff, double alone = 0.85, bool tri_operands = true) {
+TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -1.0) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
-    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone; e.tri_operands = tri_operands;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
     e.smem_of[0] = GemmCfg<T, BM, BN, BK, WM, WN, false, true>::SMEM;
     e.smem_of[1] = GemmCfg<T, BM, BN, BK, WM, WN, false, false>::SMEM;
@@ -124,7 +124,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         bool have = false;
         for (int i = 0; i < ntab; ++i) {
             if (need_tri && !tab[i].tri[0]) continue;
-            if (tri_operand && !tab[i].tri_operands) continue;
+            if (tri_operand && tab[i].eff_tri <= 0) continue;
             const int64_t t = active_tiles(M, N, tab[i].bm, tab[i].bn, tri_c);
             double rounds = (double)ceil_div64(t, kCUs);
             const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
@@ -134,7 +134,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             // of one full-depth tile, fitted to STRMM / DTRMM 4096 and 8192 (STRMM 4096: 256x128
             // tiles 0.77 ms, 128x128 0.60 ms, 64x64 0.67 ms).
             if (tri_operand) rounds = (double)t / (2.0 * kCUs) + 0.4;
-            double cost = rounds * tab[i].bm * tab[i].bn / tab[i].eff;
+            double cost = rounds * tab[i].bm * tab[i].bn / (tri_operand ? tab[i].eff_tri : tab[i].eff);
             if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             if (!have || cost < best) { best = cost; pick = i; have = true; }
         }
