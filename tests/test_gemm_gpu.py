@@ -161,6 +161,30 @@ def test_config3_sgemm_edge_sweep(gpu, M, N, K):
         assert not np.array_equal(got[mask], C[mask])
 
 
+VECTOR_LIKE_SHAPES = [(8192, 1, 2048), (1, 8192, 2048), (5000, 3, 7), (3, 2000, 20000), (1, 1, 100000),
+                      (70000, 2, 1), (33, 70000, 5), (4099, 61, 4099)]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("M,N,K", VECTOR_LIKE_SHAPES)
+def test_vector_like_and_degenerate_shapes(gpu, dtype, M, N, K):
+    """Matrix-vector, outer-product and dot-product shaped calls (one dimension of 1..3, another in
+    the tens of thousands), all four transposes, padded leading dimensions and offsets: sampled
+    elements against the exact product, surroundings of C untouched."""
+    alpha, beta = 0.75, -0.5
+    offs = (3, 9, 1)
+    for tA, tB in itertools.product([NOTRANS, TRANS], [NOTRANS, TRANS]):
+        lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 5, offs)
+        A, B, C = oracle.uniform(na, 4, dtype), oracle.uniform(nb, 5, dtype), oracle.uniform(nc, 6, dtype)
+        st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc)
+        assert st == 0
+        _check_sampled(dtype, tA != NOTRANS, tB != NOTRANS, M, N, K, alpha, beta, A[offs[0]:], lda, B[offs[1]:], ldb,
+                       C[offs[2]:], got[offs[2]:], ldc, nsamp=500)
+        mask = np.zeros(nc, dtype=bool)
+        logical_view(mask, COL, NOTRANS, M, N, offs[2], ldc)[:] = True
+        np.testing.assert_array_equal(got[~mask], C[~mask])
+
+
 def _freivalds(torch, dA, dB, dC0, dC, tA, tB, n, alpha, beta):
     """C v == alpha opA (opB v) + beta C0 v in fp64 on the device; returns the relative defect."""
     v = torch.randn(n, dtype=torch.float64, device="cuda")
