@@ -69,7 +69,8 @@ def backward_error(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B0, X
 
 
 VARIANTS = list(itertools.product([LEFT, RIGHT], [UPPER, LOWER], [NOTRANS, TRANS], [UNIT, NONUNIT]))
-SIZES = [(1, 1), (5, 3), (37, 29), (130, 17), (23, 300), (257, 64), (300, 520), (512, 33), (513, 40), (48, 1030)]
+SIZES = [(1, 1), (5, 3), (37, 29), (130, 17), (23, 300), (257, 64), (300, 520), (512, 33), (513, 40), (48, 1030),
+         (3000, 1), (1, 3000), (2049, 2), (2, 2049)]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
