@@ -234,6 +234,48 @@ def test_level3_matches_gemm_on_explicit_operands_4096(gpu, dtype):
     assert (C - Cg).abs().max().item() <= tol
 
 
+@pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("order", [ROW, COL])
+def test_long_thin_shapes_integer_exact(gpu, dtype, order):
+    """Triangles of a few thousand rows against one to three columns (and the reverse): SYRK with
+    K = 1 and N = 1, TRMM and SYMM with a single right-hand side on either side.  Exact-integer
+    data, poisoned triangles, default tile choice."""
+    alpha, beta = scalars(dtype)
+    for si, (N, K) in enumerate([(3000, 1), (1, 3000), (2049, 3)]):
+        for uplo, trans in itertools.product([UPPER, LOWER], [NOTRANS, TRANS]):
+            rows, cols = (N, K) if trans == NOTRANS else (K, N)
+            A, lda = matrix(order, rows, cols, 5, 3, 110 + si, dtype, True, limit=4)
+            C, ldc = matrix(order, N, N, 7, 2, 120 + si, dtype, True)
+            logical_view(C, order, NOTRANS, N, N, 7, ldc)[~tri_mask(N, uplo == LOWER)] = nan_of(dtype)
+            want = C.copy()
+            assert oracle.syrk(order, uplo, trans, N, K, alpha, A, 5, lda, beta, want, 7, ldc) == 0
+            st, got = gpu.syrk(order, uplo, trans, N, K, alpha, A, 5, lda, beta, C, 7, ldc)
+            assert st == 0
+            np.testing.assert_array_equal(got.view(np.uint8), want.view(np.uint8), err_msg="syrk N=%d K=%d" % (N, K))
+    for si, (M, N) in enumerate([(3000, 1), (1, 3000), (2049, 2), (2, 2049)]):
+        for side, uplo in itertools.product([LEFT, RIGHT], [UPPER, LOWER]):
+            n = M if side == LEFT else N
+            A0, lda = matrix(order, n, n, 5, 3, 130 + si, dtype, True, limit=2)
+            B, ldb = matrix(order, M, N, 7, 2, 140 + si, dtype, True, limit=2)
+            C, ldc = matrix(order, M, N, 11, 1, 150 + si, dtype, True)
+            A = A0.copy()
+            poison_triangle(A, order, n, 5, lda, uplo)
+            want = C.copy()
+            assert oracle.symm(order, side, uplo, M, N, alpha, A, 5, lda, B, 7, ldb, beta, want, 11, ldc) == 0
+            st, got = gpu.symm(order, side, uplo, M, N, alpha, A, 5, lda, B, 7, ldb, beta, C, 11, ldc)
+            assert st == 0
+            np.testing.assert_array_equal(got, want, err_msg="symm M=%d N=%d" % (M, N))
+            for trans, diag in itertools.product([NOTRANS, CONJ], [UNIT, NONUNIT]):
+                A = A0.copy()
+                poison_triangle(A, order, n, 5, lda, uplo, unit=diag == UNIT)
+                want = B.copy()
+                assert oracle.trmm(order, side, uplo, trans, diag, M, N, alpha, A, 5, lda, want, 7, ldb) == 0
+                st, got = gpu.trmm(order, side, uplo, trans, diag, M, N, alpha, A, 5, lda, B, 7, ldb)
+                assert st == 0
+                assert not np.isnan(got[7:]).any()
+                np.testing.assert_array_equal(got, want, err_msg="trmm M=%d N=%d" % (M, N))
+
+
 def test_validation_codes(gpu):
     import clblas_amd
     import torch
