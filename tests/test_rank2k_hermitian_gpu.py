@@ -105,6 +105,34 @@ def test_hemm_integer_exact_all_tiles(gpu, dtype, order, side, uplo):
             np.testing.assert_array_equal(got, want, err_msg="M=%d N=%d tile %s" % (M, N, tile))
 
 
+@pytest.mark.parametrize("kind,dtype,order,uplo,trans", rank2k_variants())
+def test_rank2k_long_thin_integer_exact(gpu, kind, dtype, order, uplo, trans):
+    """Rank-1 / rank-3 updates of a triangle of a few thousand rows, and a 1 x 1 result from
+    operands 3000 deep: exact-integer data, default tile choice."""
+    alpha, beta = rank2k_scalars(kind, dtype, True)
+    for si, (N, K) in enumerate([(3000, 1), (1, 3000), (2049, 3)]):
+        A, lda, B, ldb, C, ldc, keep = rank2k_case(kind, dtype, order, uplo, trans, N, K, 210 + 3 * si, True)
+        want = C.copy()
+        assert call_rank2k(oracle, kind, order, uplo, trans, N, K, alpha, A, 5, lda, B, 3, ldb, beta, want, 7, ldc) == 0
+        st, got = getattr(gpu, kind)(*((order, uplo, trans, N, K, alpha, A, 5, lda) +
+                                       (() if kind == "herk" else (B, 3, ldb)) + (beta, C, 7, ldc)))
+        assert st == 0
+        np.testing.assert_array_equal(got, want, err_msg="%s N=%d K=%d" % (kind, N, K))
+
+
+@pytest.mark.parametrize("dtype", CPLX)
+@pytest.mark.parametrize("order,side,uplo", list(itertools.product([ROW, COL], [LEFT, RIGHT], [UPPER, LOWER])))
+def test_hemm_long_thin_integer_exact(gpu, dtype, order, side, uplo):
+    alpha, beta = scalars(dtype)
+    for si, (M, N) in enumerate([(3000, 1), (1, 3000), (2049, 2), (2, 2049)]):
+        A, lda, B, ldb, C, ldc = hemm_case(dtype, order, side, uplo, M, N, 250 + 3 * si, True)
+        want = C.copy()
+        assert oracle.hemm(order, side, uplo, M, N, alpha, A, 5, lda, B, 7, ldb, beta, want, 11, ldc) == 0
+        st, got = gpu.hemm(order, side, uplo, M, N, alpha, A, 5, lda, B, 7, ldb, beta, C, 11, ldc)
+        assert st == 0
+        np.testing.assert_array_equal(got, want, err_msg="M=%d N=%d" % (M, N))
+
+
 @pytest.mark.parametrize("dtype", CPLX)
 @pytest.mark.parametrize("side,uplo", list(itertools.product([LEFT, RIGHT], [UPPER, LOWER])))
 def test_hemm_uniform_data(gpu, dtype, side, uplo):
