@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import (COL, ROW, NOTRANS, TRANS, CONJ, buf_len, exact_int_limits, gemm_bound, golden_cases,
+from helpers import (COL, ROW, NOTRANS, TRANS, CONJ, LEFT, LOWER, NONUNIT, buf_len, exact_int_limits, gemm_bound, golden_cases,
                      logical_view, mem_dims)
 
 pytestmark = pytest.mark.gpu
@@ -282,6 +282,57 @@ def test_two_streams_and_teardown(gpu):
         np.testing.assert_array_equal(d[5].cpu().numpy(), w2)
         clblas_amd.teardown()          # second pass runs after the scratch was released
     assert clblas_amd.setup() == 0
+
+
+def test_host_threads_on_their_own_streams(gpu):
+    """Four host threads call the library at the same time, each on its own stream (ctypes
+    releases the interpreter lock during a call): split-K SGEMM, whose scratch buffer is looked up
+    per stream under the library's lock, and DTRSM with its packing buffer.  Exact-integer GEMM
+    data, so every result must equal the oracle's."""
+    import threading
+    import torch
+    import clblas_amd
+    M, N, K = 100, 90, 4096
+    la, _ = exact_int_limits(K, 1.0, 1.0, np.float32)
+    n = 300
+    jobs = []
+    for t in range(4):
+        A, B, C = (oracle.integers(sz, 10 * t + i, la, np.float32) for i, sz in enumerate((M * K, K * N, M * N)))
+        want = C.copy()
+        oracle.gemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, want, 0, M)
+        T = oracle.triangular(n, n, True, 50 + t, np.float64)
+        X = oracle.uniform(n * 64, 60 + t, np.float64)
+        wx = X.copy()
+        assert oracle.trsm_naive(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, 64, 1.0, T, 0, n, wx, 0, n) == 0
+        jobs.append(dict(d=[torch.from_numpy(x).cuda() for x in (A, B, C, T, X)], C0=C, X0=X, want=want, wx=wx,
+                         stream=torch.cuda.Stream(), err=None))
+    torch.cuda.synchronize()
+
+    def work(j):
+        try:
+            dA, dB, dC, dT, dX = j["d"]
+            for _ in range(20):
+                dC.copy_(torch.from_numpy(j["C0"]), non_blocking=False)
+                dX.copy_(torch.from_numpy(j["X0"]), non_blocking=False)
+                with torch.cuda.stream(j["stream"]):
+                    st1 = clblas_amd.sgemm(COL, NOTRANS, NOTRANS, M, N, K, 1.0, dA, 0, M, dB, 0, K, 1.0, dC, 0, M)
+                    st2 = clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, 64, 1.0, dT, 0, n, dX, 0, n)
+                j["stream"].synchronize()
+                assert st1 == 0 and st2 == 0
+                np.testing.assert_array_equal(dC.cpu().numpy(), j["want"])
+                got = dX.cpu().numpy()
+                assert np.abs(got - j["wx"]).max() <= 32 * n * np.finfo(np.float64).eps * np.abs(j["wx"]).max()
+        except BaseException as e:  # reported by the main thread
+            j["err"] = e
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    for j in jobs:
+        if j["err"] is not None:
+            raise j["err"]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex64, np.complex128])
