@@ -313,6 +313,13 @@ def main():
                 row[tag] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2),
                             "GBps": round(nbytes / ms / 1e6, 1)}
             shapes["config3 %dx%dx%d" % (M, N, K)] = row
+        # What the memory system gives a plain streaming kernel on this box (1 GiB read + 1 GiB written):
+        # the yardstick for the HBM-side figures of the skinny shapes above.
+        src = torch.empty(1 << 28, device="cuda", dtype=torch.float32)
+        dst = torch.empty_like(src)
+        copy_ms = timed_batch(torch, lambda: dst.copy_(src), 5, 2)
+        shapes["plain_device_copy_GBps"] = round(2 * 2 ** 30 / copy_ms / 1e6, 1)
+        del src, dst
         extra["sgemm_configs_1_and_3"] = shapes
 
     # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
