@@ -53,11 +53,18 @@ void *workspace_get(hipStream_t stream, size_t bytes, int kind) {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     WsSlot &slot = g_ws[std::make_pair(std::make_pair(dev, kind), stream)];
     if (slot.bytes >= bytes && slot.ptr) return slot.ptr;
+    // Outgrown buffers stay allocated until teardown (kernels already enqueued may still use them), so
+    // grow by at least half: the retired ones then add up to at most twice the current size.
     size_t want = bytes < (size_t)(1 << 20) ? (size_t)(1 << 20) : bytes;
+    if (want < slot.bytes + slot.bytes / 2) want = slot.bytes + slot.bytes / 2;
     void *p = nullptr;
     if (hipMalloc(&p, want) != hipSuccess) {
         (void)hipGetLastError();
-        return nullptr;
+        want = bytes;  // no room for the margin: try the size that is needed
+        if (hipMalloc(&p, want) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
     }
     if (slot.ptr) g_ws_retired.push_back(std::make_pair(dev, slot.ptr));
     slot.ptr = p;
