@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|vendor]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
@@ -85,7 +85,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs or copy (profiling; "
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, vendor or copy (profiling; "
                     "copy = a plain 1 GiB device copy used to scale the HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -321,6 +321,33 @@ def main():
         shapes["plain_device_copy_GBps"] = round(2 * 2 ** 30 / copy_ms / 1e6, 1)
         del src, dst
         extra["sgemm_configs_1_and_3"] = shapes
+
+    # ---- Yardstick: the vendor BLAS that torch calls (rocBLAS / hipBLASLt) on the same box, same sizes.
+    #      Not the reference and not a target of the parity tests: it shows what the part gives a
+    #      tuned library.  FP32 without TF32-style shortcuts. ----
+    if args.only in ("", "vendor"):
+        torch.backends.cuda.matmul.allow_tf32 = False
+        vy = {}
+        for name, dt, fl in (("sgemm", torch.float32, 2.0), ("dgemm", torch.float64, 2.0),
+                             ("cgemm", torch.complex64, 8.0), ("zgemm", torch.complex128, 8.0)):
+            real = torch.float32 if dt in (torch.float32, torch.complex64) else torch.float64
+            shape = (n, n, 2) if dt.is_complex else (n, n)
+            mk = lambda: torch.rand(shape, device="cuda", dtype=real, generator=gen) * 2 - 1
+            A, B = mk(), mk()
+            if dt.is_complex:
+                A, B = torch.view_as_complex(A), torch.view_as_complex(B)
+            C = torch.empty(n, n, device="cuda", dtype=dt)
+            ms = timed_batch(torch, lambda: torch.mm(A, B, out=C), 5, 2)
+            vy["torch_mm_" + name] = {"tflops": round(fl * n ** 3 / ms / 1e9, 2), "ms": round(ms, 3)}
+            del A, B, C
+        T = torch.tril(torch.rand(n, n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1) / n
+        T.diagonal().copy_(torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) + 1)
+        Bt = torch.randn(n, n, device="cuda", dtype=torch.float64, generator=gen)
+        ms = timed_batch(torch, lambda: torch.linalg.solve_triangular(T, Bt, upper=False), 3, 1)
+        vy["torch_solve_triangular_f64"] = {"tflops": round(float(n) * (n + 1) * n / ms / 1e9, 2), "ms": round(ms, 3)}
+        vy["workload"] = "square, N=%d, row-major torch tensors, no transposes, beta=0" % n
+        del T, Bt
+        extra["vendor_yardstick"] = vy
 
     # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
     cpu = None
