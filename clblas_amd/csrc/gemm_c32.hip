@@ -6,12 +6,13 @@ namespace cba {
 // Ordered from the largest tile to the smallest.  A complex element carries four times the
 // flops of a real one for twice the bytes, so these tiles match the real 256x128 / 128x128
 // ones in arithmetic intensity.
-//   0: 128x128x16, wave 64x64 (2 workgroups of 4 waves per CU)
+//   0: 128x128x16, wave 64x64 (2 workgroups of 4 waves per CU), split-K capable for small C with deep K
+//      (1024 x 1024 x 8192: 116 -> 139 TFLOP/s, 1280 x 1280 x 16384 105 -> 142)
 //   1:  64x64x8,  wave 32x32, split-K capable (credited with .90; .84 where an operand is triangular:
 //      3328^3 127 -> 135 TFLOP/s, 3000 x 1500 x 1000 120 -> 126, CSYRK 6144 130 -> 139 against .84 for all)
 static const TileEntry<Cx<float>> *c32_tiles(int *n) {
     static const TileEntry<Cx<float>> tab[] = {
-        make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, false, true>(0.93),
+        make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, true, true>(0.93),
         make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true, true>(0.90, 0.85, 0.84),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

@@ -4,11 +4,12 @@
 namespace cba {
 
 // Ordered from the largest tile to the smallest.
-//   0: 128x64x8, wave 64x32 (2 workgroups of 4 waves per CU)
+//   0: 128x64x8, wave 64x32 (2 workgroups of 4 waves per CU), split-K capable for small C with deep K
+//      (1024 x 1024 x 8192: 64 -> 71 TFLOP/s, 768 x 768 x 16384 59 -> 70)
 //   1:  64x64x8, wave 32x32, split-K capable
 static const TileEntry<Cx<double>> *c64_tiles(int *n) {
     static const TileEntry<Cx<double>> tab[] = {
-        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, false, true>(0.93),
+        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, true, true>(0.93),
         make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true>(0.86),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

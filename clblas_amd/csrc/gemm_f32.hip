@@ -5,12 +5,15 @@ namespace cba {
 
 // Ordered from the largest tile to the smallest.
 //   0: 256x128x16, wave 128x64 (2 workgroups of 4 waves per CU)
-//   1: 128x128x16, wave 64x64
+//   1: 128x128x16, wave 64x64, split-K capable
 //   2: 128x64x32,  wave 64x32 (narrow C: 65536 x 64 x 4096 runs at 119 TFLOP/s with it, 107 with 64x64).
 //      Panels of depth 32 keep twice the bytes in flight, which is what a product that streams A
 //      from HBM needs (depth 16: 114.6), and let a workgroup that is alone on its CU run at full rate
 //      (16384 x 128 x 2048: 126 against 117 with depth 16); the larger tiles lose residency with them.
 //   3:  64x128x32, wave 32x64: the mirror image for wide C (64 x 65536 x 4096: 116 against 107)
+//      Tiles 1 to 3 are split-K capable for small C with deep K, where the 64x64 tile (split or not) loses to
+//      them: 1024 x 1024 x 65536 98 -> 141 TFLOP/s, 1280 x 1280 x 8192 108 -> 125, 768 x 768 x 16384 109 -> 128,
+//      3000 x 200 x 6000 72 -> 87.
 //      Tiles 2 and 3 are not offered to products with a triangular operand: the round model for those
 //      was fitted on the square tiles and picks the oblong ones where they lose (STRMM / SSYMM 3072:
 //      7-9 % slower with them).
@@ -19,9 +22,9 @@ namespace cba {
 static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
-        make_tile_entry<float, 128, 128, 16, 64, 64, 2, false, true>(0.920),
-        make_tile_entry<float, 128, 64, 32, 64, 32, 2, false, true>(0.92, 0.97, 0.0),
-        make_tile_entry<float, 64, 128, 32, 32, 64, 2, false, true>(0.92, 0.97, 0.0),
+        make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920),
+        make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0),
+        make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.97, 0.0),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true>(0.84, 0.95),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

@@ -4,13 +4,14 @@
 namespace cba {
 
 // Ordered from the largest tile to the smallest.
-//   0: 128x128x16, wave 64x64 (2 workgroups of 4 waves per CU)
+//   0: 128x128x16, wave 64x64 (2 workgroups of 4 waves per CU), split-K capable for small C with deep K
+//      (1024 x 1024 x 16384: 50 -> 69 TFLOP/s, 1280 x 1280 x 8192 54 -> 66, 256 x 4096 x 8192 46 -> 66)
 //   1:  64x64x16,  wave 32x32, split-K capable.  Credited with .90 for plain and triangular-C
 //      products (2304^3 64.7 -> 67.9 TFLOP/s, 3328^3 64.5 -> 68.6, 3000 x 1500 x 1000 56.6 -> 61.1 against
 //      .84) and with .84 where an operand is triangular (DTRMM / DSYMM 6144 lose 2-3 % with .90).
 static const TileEntry<double> *f64_tiles(int *n) {
     static const TileEntry<double> tab[] = {
-        make_tile_entry<double, 128, 128, 16, 64, 64, 2, false, true>(0.94),
+        make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94),
         make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true>(0.90, 0.85, 0.84),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

@@ -112,15 +112,47 @@ static inline int tail_slices_for(int64_t t, int K, int bk, bool allowed) {
     return s < 2 ? 1 : (int)s;
 }
 
+// K split of a tile shape that cannot give every CU a workgroup: about two workgroups per CU,
+// at least four panels per range.
+static inline int splits_for(int64_t t, int K, int bk) {
+    const int64_t kCUs = 256;
+    if (t >= kCUs || K < 8 * bk) return 1;
+    int64_t want = (2 * kCUs) / t;
+    const int64_t max_by_k = K / (4 * bk);
+    if (want > max_by_k) want = max_by_k;
+    if (want > 64) want = 64;
+    return want < 1 ? 1 : (int)want;
+}
+
+// Cost of the pass that adds up the K ranges, in the tile model's unit (elements of C per CU at
+// the MFMA peak over the whole depth K): a dependent launch of about 8 us plus the partial sums
+// written and read back at about 4 TB/s (1024 x 1024 x 8192 FP32 in 4 ranges: 12 us measured).
+template <typename T> static double split_overhead_cost(int M, int N, int K, int splits) {
+    const double peak_per_cu = (sizeof(typename Elem<T>::Real) == 4 ? 157.3e12 : 78.6e12) / 256.0;
+    const double flops_per_step = Elem<T>::CPLX ? 8.0 : 2.0;
+    const double seconds = 8e-6 + (double)(splits + 1) * M * N * sizeof(T) / 4e12;
+    return seconds * peak_per_cu / (flops_per_step * K);
+}
+
 template <typename T>
 static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, bool need_tri, int tri_c,
                         bool tri_operand, bool tail_ok, int *tile_out, int *splits_out) {
     const int64_t kCUs = 256;
     int pick = ntab - 1;  // table is ordered large -> small
+    bool pick_split = true;
     if (force >= 0 && force < ntab && (!need_tri || tab[force].tri[0])) {
         pick = force;
     } else {
-        double best = 0;
+        // Cost of tile i with its depth cut into s ranges: the ranges fill the CUs that the tiles
+        // alone leave idle, at the price of the pass that adds them up.
+        auto split_cost = [&](int i, int64_t t, int s) {
+            const double alone = t * s <= kCUs ? tab[i].alone : 1.0;
+            return (double)ceil_div64(t * s, kCUs) * tab[i].bm * tab[i].bn / (s * tab[i].eff * alone) +
+                   split_overhead_cost<T>(M, N, K, s);
+        };
+        const bool split_model = debug_env_int("CLBLAS_AMD_GEMM_SPLIT_MODEL", 1) != 0 && !need_tri;
+        double best = 0, best_split = 0;
+        int pick_of_split = -1;
         bool have = false;
         for (int i = 0; i < ntab; ++i) {
             if (need_tri && !tab[i].tri[0]) continue;
@@ -137,19 +169,31 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             double cost = rounds * tab[i].bm * tab[i].bn / (tri_operand ? tab[i].eff_tri : tab[i].eff);
             if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             if (!have || cost < best) { best = cost; pick = i; have = true; }
+            // Small C, deep K: the larger tiles with a K split, ranges of at least 512 and 32 panels.
+            if (split_model && tab[i].has_splitk && i != ntab - 1) {
+                const int s = splits_for(t, K, tab[i].bk);
+                if (s > 1 && K / s >= 512 && K / s >= 32 * tab[i].bk) {
+                    const double c = split_cost(i, t, s);
+                    if (pick_of_split < 0 || c < best_split) { best_split = c; pick_of_split = i; }
+                }
+            }
         }
+        // The smallest tile adds a K split whenever even it cannot give every CU a workgroup; a larger
+        // tile is split only where the model puts it 3 % ahead of what would run otherwise.
+        if (pick_of_split >= 0) {
+            if (pick == ntab - 1 && tab[pick].has_splitk) {
+                const int64_t t = active_tiles(M, N, tab[pick].bm, tab[pick].bn, 0);
+                const int s = splits_for(t, K, tab[pick].bk);
+                if (s > 1) best = split_cost(pick, t, s);
+            }
+            if (best_split * 1.03 < best) pick = pick_of_split;
+            else pick_of_split = -1;
+        }
+        pick_split = pick == ntab - 1 || pick == pick_of_split;
     }
     int splits = 1;
-    if (tab[pick].has_splitk && !need_tri) {
-        int64_t t = ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn);
-        if (t < kCUs && K >= 8 * tab[pick].bk) {
-            int64_t want = (2 * kCUs) / t;              // aim for ~2 workgroups per CU
-            int64_t max_by_k = K / (4 * tab[pick].bk);  // at least 4 panels per split
-            splits = (int)(want < max_by_k ? want : max_by_k);
-            if (splits < 1) splits = 1;
-            if (splits > 64) splits = 64;
-        }
-    }
+    if (pick_split && tab[pick].has_splitk && !need_tri)
+        splits = splits_for(ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn), K, tab[pick].bk);
     *tile_out = pick;
     *splits_out = splits;
 }

@@ -379,3 +379,25 @@ def test_many_workgroups_not_whole_rounds_integer_exact(gpu, dtype):
             st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, C, 7, ldc, tile=tile)
             assert st == 0
             np.testing.assert_array_equal(got, want, err_msg="%dx%dx%d tile %s" % (M, N, K, tile))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.complex64, np.complex128])
+def test_small_c_deep_k_integer_exact(gpu, dtype):
+    """Small C, deep K: too few tiles for the 256 CUs, so the tile choice cuts K into ranges for one of
+    the larger tiles (partial sums in the workspace, added up by a second pass).  Exact-integer data,
+    default tile choice and every tile forced; odd offsets and leading dimensions."""
+    cplx = np.dtype(dtype).kind == "c"
+    alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
+    n_tiles = 2 if dtype != np.float32 else 5
+    for (M, N, K), (tA, tB) in (((640, 520, 6000), (NOTRANS, NOTRANS)), ((300, 900, 5000), (TRANS, CONJ))):
+        lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
+        lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]
+        A = oracle.integers(na, 1, lim, dtype)
+        B = oracle.integers(nb, 2, lim, dtype)
+        C = oracle.integers(nc, 3, 8, dtype)
+        want = C.copy()
+        assert oracle.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, want, 7, ldc) == 0
+        for tile in [None] + list(range(n_tiles)):
+            st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, 3, lda, B, 5, ldb, beta, C, 7, ldc, tile=tile)
+            assert st == 0
+            np.testing.assert_array_equal(got, want, err_msg="%dx%dx%d tile %s" % (M, N, K, tile))
