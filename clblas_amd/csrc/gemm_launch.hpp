@@ -125,12 +125,14 @@ static inline int splits_for(int64_t t, int K, int bk) {
 }
 
 // Cost of the pass that adds up the K ranges, in the tile model's unit (elements of C per CU at
-// the MFMA peak over the whole depth K): a dependent launch of about 8 us plus the partial sums
-// written and read back at about 4 TB/s (1024 x 1024 x 8192 FP32 in 4 ranges: 12 us measured).
+// the MFMA peak over the whole depth K): a dependent launch of about 5 us plus the partial sums
+// written and read back at about 4 TB/s.  Fitted to FP64 with 64x64 tiles, us by ranges (model):
+// 512^3 1: 21 (22), 4: 15 (16), 8: 18 (17.5); 960 x 960 x 256 1: 14 (13), 2: 22 (22); 640 x 640 x 512
+// 1: 20.9 (21.9), 5: 19.1 (20), each with 4 us for the first launch.
 template <typename T> static double split_overhead_cost(int M, int N, int K, int splits) {
     const double peak_per_cu = (sizeof(typename Elem<T>::Real) == 4 ? 157.3e12 : 78.6e12) / 256.0;
     const double flops_per_step = Elem<T>::CPLX ? 8.0 : 2.0;
-    const double seconds = 8e-6 + (double)(splits + 1) * M * N * sizeof(T) / 4e12;
+    const double seconds = 5e-6 + (double)(splits + 1) * M * N * sizeof(T) / 4e12;
     return seconds * peak_per_cu / (flops_per_step * K);
 }
 
@@ -178,22 +180,46 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
                 }
             }
         }
-        // The smallest tile adds a K split whenever even it cannot give every CU a workgroup; a larger
-        // tile is split only where the model puts it 3 % ahead of what would run otherwise.
-        if (pick_of_split >= 0) {
-            if (pick == ntab - 1 && tab[pick].has_splitk) {
-                const int64_t t = active_tiles(M, N, tab[pick].bm, tab[pick].bn, 0);
-                const int s = splits_for(t, K, tab[pick].bk);
-                if (s > 1) best = split_cost(pick, t, s);
+        // The smallest tile, when even it cannot give every CU a workgroup, takes the number of ranges
+        // that the same model prices lowest, one range included (short K: the pass that adds the
+        // ranges up costs more than the idle CUs; 960 x 960 x 256 FP64 22 -> 14 us, 512^3 18 -> 15 us).
+        // A larger tile is split only where the model puts it 3 % ahead of what would run otherwise.
+        const int last = ntab - 1;
+        int last_splits = -1;  // -1: the rule without the model
+        if (split_model && pick == last && tab[last].has_splitk) {
+            const int64_t t = active_tiles(M, N, tab[last].bm, tab[last].bn, 0);
+            const int s_max = splits_for(t, K, tab[last].bk);
+            if (s_max > 1) {
+                static const int kCand[] = {2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 40, 48, 64};
+                last_splits = 1;  // `best` is the cost of one range
+                for (int s : kCand) {
+                    if (s >= s_max) break;
+                    const double c = split_cost(last, t, s);
+                    if (c < best) { best = c; last_splits = s; }
+                }
+                const double c = split_cost(last, t, s_max);
+                if (c < best) { best = c; last_splits = s_max; }
             }
+        }
+        if (pick_of_split >= 0) {
             if (best_split * 1.03 < best) pick = pick_of_split;
             else pick_of_split = -1;
         }
-        pick_split = pick == ntab - 1 || pick == pick_of_split;
+        if (pick == last && last_splits >= 0) {
+            *tile_out = pick;
+            *splits_out = last_splits;
+            const int forced_s = debug_env_int("CLBLAS_AMD_GEMM_SPLITS", 0);
+            if (forced_s <= 0) return;
+        }
+        pick_split = pick == last || pick == pick_of_split;
     }
     int splits = 1;
     if (pick_split && tab[pick].has_splitk && !need_tri)
         splits = splits_for(ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn), K, tab[pick].bk);
+    if (tab[pick].has_splitk && !need_tri) {  // debug: number of K ranges (clamped to 4 panels per range)
+        const int forced = debug_env_int("CLBLAS_AMD_GEMM_SPLITS", 0);
+        if (forced > 0) splits = forced > K / (4 * tab[pick].bk) ? (K / (4 * tab[pick].bk) > 0 ? K / (4 * tab[pick].bk) : 1) : forced;
+    }
     *tile_out = pick;
     *splits_out = splits;
 }
