@@ -142,6 +142,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
     const int64_t kCUs = 256;
     int pick = ntab - 1;  // table is ordered large -> small
     bool pick_split = true;
+    int model_splits = -1;  // ranges chosen by the cost model for the smallest tile (-1: none)
     if (force >= 0 && force < ntab && (!need_tri || tab[force].tri[0])) {
         pick = force;
     } else {
@@ -205,20 +206,17 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             if (best_split * 1.03 < best) pick = pick_of_split;
             else pick_of_split = -1;
         }
-        if (pick == last && last_splits >= 0) {
-            *tile_out = pick;
-            *splits_out = last_splits;
-            const int forced_s = debug_env_int("CLBLAS_AMD_GEMM_SPLITS", 0);
-            if (forced_s <= 0) return;
-        }
         pick_split = pick == last || pick == pick_of_split;
+        if (pick == last) model_splits = last_splits;
     }
     int splits = 1;
-    if (pick_split && tab[pick].has_splitk && !need_tri)
-        splits = splits_for(ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn), K, tab[pick].bk);
-    if (tab[pick].has_splitk && !need_tri) {  // debug: number of K ranges (clamped to 4 panels per range)
-        const int forced = debug_env_int("CLBLAS_AMD_GEMM_SPLITS", 0);
-        if (forced > 0) splits = forced > K / (4 * tab[pick].bk) ? (K / (4 * tab[pick].bk) > 0 ? K / (4 * tab[pick].bk) : 1) : forced;
+    if (tab[pick].has_splitk && !need_tri) {
+        const int by_rule = splits_for(ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn), K, tab[pick].bk);
+        if (model_splits >= 0) splits = model_splits;
+        else if (pick_split) splits = by_rule;
+        const int forced = debug_env_int("CLBLAS_AMD_GEMM_SPLITS", 0);  // debug: number of K ranges
+        const int most = K / (4 * tab[pick].bk) > 0 ? K / (4 * tab[pick].bk) : 1;  // 4 panels per range
+        if (forced > 0) splits = forced < most ? forced : most;
     }
     *tile_out = pick;
     *splits_out = splits;
