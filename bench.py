@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|vendor]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|vendor]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
@@ -85,7 +85,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, vendor or copy (profiling; "
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, vendor or copy (profiling; "
                     "copy = a plain 1 GiB device copy used to scale the HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -321,6 +321,30 @@ def main():
         shapes["plain_device_copy_GBps"] = round(2 * 2 ** 30 / copy_ms / 1e6, 1)
         del src, dst
         extra["sgemm_configs_1_and_3"] = shapes
+
+    # ---- Small C, deep K: fewer tiles than CUs, so the tile choice cuts K into ranges (column-major NN,
+    #      alpha = beta = 1); the vendor BLAS behind torch.mm on the same product beside it. ----
+    if args.only in ("", "deepk"):
+        dk = {}
+        for name, dt, fn, peak in (("sgemm", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX),
+                                   ("dgemm", torch.float64, clblas_amd.dgemm, PEAK_FP64_MATRIX)):
+            for (M, N, K) in ((1024, 1024, 16384), (768, 768, 16384), (3000, 200, 6000)):
+                A = torch.rand(K, M, device="cuda", dtype=dt, generator=gen) * 2 - 1   # column-major M x K
+                B = torch.rand(N, K, device="cuda", dtype=dt, generator=gen) * 2 - 1   # column-major K x N
+                C = torch.zeros(N, M, device="cuda", dtype=dt)
+
+                def call():
+                    st = fn(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, C, 0, M)
+                    if st != 0:
+                        raise RuntimeError("clblas %s returned %d" % (name, st))
+                ms = timed_batch(torch, call, 20, 3)
+                vendor_ms = timed_batch(torch, lambda: torch.mm(B, A, out=C), 20, 3)   # C^T = B^T A^T, row-major
+                tf = 2.0 * M * N * K / ms / 1e9
+                dk["%s %dx%dx%d" % (name, M, N, K)] = {
+                    "ms": round(ms, 4), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
+                    "torch_mm_tflops": round(2.0 * M * N * K / vendor_ms / 1e9, 2)}
+                del A, B, C
+        extra["small_c_deep_k"] = dk
 
     # ---- Yardstick: the vendor BLAS that torch calls (rocBLAS / hipBLASLt) on the same box, same sizes.
     #      Not the reference and not a target of the parity tests: it shows what the part gives a
