@@ -23,6 +23,12 @@ template <typename T> struct TileEntry {
     double eff;
     double alone;    // further factor when a workgroup has its CU to itself (at most 256 tiles)
     double eff_tri;  // `eff` for products with a triangular A or B (TRMM, SYMM passes); 0: not offered
+    // Fixed time of a workgroup (first loads, write-back of C) as a depth: the cost of a tile is taken
+    // times (1 + k0 / K).  On large C with short K the write-back is what bounds the rate, and the
+    // small tiles, more of them per CU, overlap it better (8192 x 8192 x 64 FP64: 35.7 TFLOP/s with 64x64 tiles,
+    // 31.6 with 128x128; rates over K fit T(K) = T_inf K / (K + k0) with k0 = 68 and 95).  0: no such term.
+    double k0;
+    double tail_extra;  // rounds that a sliced tail adds on top of 1 / slices (reduction pass, uneven slices)
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
     void (*plain[4])(const GemmParams<T>);
     void (*splitk[4])(const GemmParams<T>);
@@ -31,10 +37,11 @@ template <typename T> struct TileEntry {
 
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false>
-TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -1.0) {
+TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -1.0, double k0 = 0.0,
+                             double tail_extra = 0.05) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
-    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri; e.k0 = k0; e.tail_extra = tail_extra;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
     e.smem_of[0] = GemmCfg<T, BM, BN, BK, WM, WN, false, true>::SMEM;
     e.smem_of[1] = GemmCfg<T, BM, BN, BK, WM, WN, false, false>::SMEM;
@@ -163,7 +170,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             const int64_t t = active_tiles(M, N, tab[i].bm, tab[i].bn, tri_c);
             double rounds = (double)ceil_div64(t, kCUs);
             const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
-            if (ts > 1) rounds = (double)(t / kCUs) + 1.0 / ts + 0.05;  // + the reduction pass
+            if (ts > 1) rounds = (double)(t / kCUs) + 1.0 / ts + tab[i].tail_extra;
             // A triangular operand makes the tiles differ in depth (half of the full depth on
             // average, started deepest first): the CUs share the total evenly up to a fraction
             // of one full-depth tile, fitted to STRMM / DTRMM 4096 and 8192 (STRMM 4096: 256x128
@@ -171,6 +178,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             if (tri_operand) rounds = (double)t / (2.0 * kCUs) + 0.4;
             double cost = rounds * tab[i].bm * tab[i].bn / (tri_operand ? tab[i].eff_tri : tab[i].eff);
             if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
+            cost *= 1.0 + tab[i].k0 / K;
             if (!have || cost < best) { best = cost; pick = i; have = true; }
             // Small C, deep K: the larger tiles with a K split, ranges of at least 512 and 32 panels.
             if (split_model && tab[i].has_splitk && i != ntab - 1) {
