@@ -27,6 +27,7 @@ template <typename T> struct TileEntry {
     // times (1 + k0 / K).  On large C with short K the write-back is what bounds the rate, and the
     // small tiles, more of them per CU, overlap it better (8192 x 8192 x 64 FP64: 35.7 TFLOP/s with 64x64 tiles,
     // 31.6 with 128x128; rates over K fit T(K) = T_inf K / (K + k0) with k0 = 68 and 95).  0: no such term.
+    double eff_tri_c;  // `eff` for products that store one triangle of C (SYRK, HERK, ...); default: eff
     double k0;
     double tail_extra;  // rounds that a sliced tail adds on top of 1 / slices (reduction pass, uneven slices)
     // index: (transA ? 2 : 0) | (transB ? 1 : 0)
@@ -38,10 +39,12 @@ template <typename T> struct TileEntry {
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false>
 TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -1.0, double k0 = 0.0,
-                             double tail_extra = 0.05) {
+                             double tail_extra = 0.05, double eff_tri_c = -1.0) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
-    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK; e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri; e.k0 = k0; e.tail_extra = tail_extra;
+    e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK;
+    e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri; e.k0 = k0; e.tail_extra = tail_extra;
+    e.eff_tri_c = eff_tri_c < 0 ? eff : eff_tri_c;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
     e.smem_of[0] = GemmCfg<T, BM, BN, BK, WM, WN, false, true>::SMEM;
     e.smem_of[1] = GemmCfg<T, BM, BN, BK, WM, WN, false, false>::SMEM;
@@ -176,7 +179,8 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             // of one full-depth tile, fitted to STRMM / DTRMM 4096 and 8192 (STRMM 4096: 256x128
             // tiles 0.77 ms, 128x128 0.60 ms, 64x64 0.67 ms).
             if (tri_operand) rounds = (double)t / (2.0 * kCUs) + 0.4;
-            double cost = rounds * tab[i].bm * tab[i].bn / (tri_operand ? tab[i].eff_tri : tab[i].eff);
+            const double eff = tri_operand ? tab[i].eff_tri : tri_c ? tab[i].eff_tri_c : tab[i].eff;
+            double cost = rounds * tab[i].bm * tab[i].bn / eff;
             if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             cost *= 1.0 + tab[i].k0 / K;
             if (!have || cost < best) { best = cost; pick = i; have = true; }
