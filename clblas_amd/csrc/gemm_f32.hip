@@ -5,7 +5,9 @@ namespace cba {
 
 // Ordered from the largest tile to the smallest.
 //   0: 256x128x16, wave 128x64 (2 workgroups of 4 waves per CU)
-//   1: 128x128x16, wave 64x64, split-K capable
+//   1: 128x128x16, wave 64x64, split-K capable; its sliced tail is priced at 0.12 rounds (2304^3, 324 tiles with 68
+//      in the tail round: 119 TFLOP/s, where the 64x64 tiles reach 127; 3700^3 stays with this tile, 137.8
+//      against 134.5)
 //   2: 128x64x32,  wave 64x32 (narrow C: 65536 x 64 x 4096 runs at 119 TFLOP/s with it, 107 with 64x64).
 //      Panels of depth 32 keep twice the bytes in flight, which is what a product that streams A
 //      from HBM needs (depth 16: 114.6), and let a workgroup that is alone on its CU run at full rate
@@ -22,7 +24,7 @@ namespace cba {
 static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
-        make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920),
+        make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.12),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0),
         make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.97, 0.0),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true>(0.84, 0.95),
