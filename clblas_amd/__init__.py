@@ -76,7 +76,9 @@ EXPORTED_SYMBOLS = (
     "clblasCtrsm",
     "clblasZtrsm",
 ) + tuple("clblas%s%s" % (t, f) for f in ("syrk", "trmm", "symm", "syr2k") for t in "SDCZ") + tuple(
-    "clblas%s%s" % (t, f) for f in ("herk", "her2k", "hemm") for t in "CZ")
+    "clblas%s%s" % (t, f) for f in ("herk", "her2k", "hemm") for t in "CZ") + (
+    "clblasAmdReleaseStream", "clblasAmdReserveWorkspace", "clblasAmdWorkspaceStats", "clblasAmdLastDispatch",
+    "clblasAmdReloadDebugEnv")
 
 _lib = None
 
@@ -139,6 +141,16 @@ def _declare(lib):
     lib.clblasTeardown.argtypes = []
     lib.clblasGetVersion.restype = i
     lib.clblasGetVersion.argtypes = [ctypes.POINTER(ctypes.c_uint)] * 3
+    lib.clblasAmdReleaseStream.restype = i
+    lib.clblasAmdReleaseStream.argtypes = [vp]
+    lib.clblasAmdReserveWorkspace.restype = i
+    lib.clblasAmdReserveWorkspace.argtypes = [vp, sz, sz, sz]
+    lib.clblasAmdWorkspaceStats.restype = None
+    lib.clblasAmdWorkspaceStats.argtypes = [ctypes.POINTER(sz), ctypes.POINTER(sz)]
+    lib.clblasAmdLastDispatch.restype = sz
+    lib.clblasAmdLastDispatch.argtypes = [ctypes.c_char_p, sz]
+    lib.clblasAmdReloadDebugEnv.restype = None
+    lib.clblasAmdReloadDebugEnv.argtypes = []
 
 
 def load_library(path=None):
@@ -181,6 +193,34 @@ def setup():
 
 def teardown():
     load_library().clblasTeardown()
+
+
+def release_stream(stream=None):
+    """Frees the library's scratch buffers of `stream` (its work must have completed)."""
+    return load_library().clblasAmdReleaseStream(_stream(stream))
+
+
+def reserve_workspace(gemm_bytes=0, trmm_bytes=0, trsm_bytes=0, stream=None):
+    return load_library().clblasAmdReserveWorkspace(_stream(stream), gemm_bytes, trmm_bytes, trsm_bytes)
+
+
+def workspace_stats():
+    """(streams that hold scratch buffers, bytes of their current buffers)."""
+    a, b = ctypes.c_size_t(), ctypes.c_size_t()
+    load_library().clblasAmdWorkspaceStats(ctypes.byref(a), ctypes.byref(b))
+    return a.value, b.value
+
+
+def last_dispatch():
+    """(description of the last GEMM kernel this thread launched, launches issued so far)."""
+    buf = ctypes.create_string_buffer(512)
+    n = load_library().clblasAmdLastDispatch(buf, 512)
+    return buf.value.decode(), n
+
+
+def reload_debug_env():
+    """Makes the library read its CLBLAS_AMD_* debugging variables again (it reads them once)."""
+    load_library().clblasAmdReloadDebugEnv()
 
 
 def get_version():

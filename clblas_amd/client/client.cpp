@@ -194,7 +194,7 @@ template <typename T, typename... Rest> clblasStatus hemm(clblasOrder, clblasSid
 
 enum Fn { FN_GEMM, FN_TRSM, FN_TRMM, FN_SYRK, FN_SYMM, FN_SYR2K, FN_HERK, FN_HER2K, FN_HEMM, FN_COUNT };
 
-template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t n, size_t k, bool &ok) {
+template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t n, size_t k, hipStream_t stream, bool &ok) {
     typedef typename Type<T>::Real R;
     const int NC = Type<T>::NC;
     const bool tri = fn == FN_TRSM || fn == FN_TRMM;    // A triangular, B in place
@@ -228,8 +228,6 @@ template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t 
     HIP_OK(hipMemcpy(da, ha.data(), na * sizeof(T), hipMemcpyHostToDevice));
     HIP_OK(hipMemcpy(db, hb.data(), nb * sizeof(T), hipMemcpyHostToDevice));
     HIP_OK(hipMemcpy(dc, hc.data(), nc * sizeof(T), hipMemcpyHostToDevice));
-    hipStream_t stream;
-    HIP_OK(hipStreamCreate(&stream));
     hipEvent_t e0, e1;
     HIP_OK(hipEventCreate(&e0));
     HIP_OK(hipEventCreate(&e1));
@@ -293,7 +291,6 @@ template <typename T> double run_case(const Options &o, Fn fn, size_t m, size_t 
     }
     HIP_OK(hipEventDestroy(e0));
     HIP_OK(hipEventDestroy(e1));
-    HIP_OK(hipStreamDestroy(stream));
     HIP_OK(hipFree(da));
     HIP_OK(hipFree(db));
     HIP_OK(hipFree(dc));
@@ -329,14 +326,16 @@ int main(int argc, char **argv) {
                   "library,numQueues,label,GFLOPS");
     const size_t count = sizes.empty() ? 1 : sizes.size();
     int rc = 0;
+    hipStream_t stream;  // one stream for the whole run: the library keeps its scratch buffers per stream
+    HIP_OK(hipStreamCreate(&stream));
     for (size_t i = 0; i < count; ++i) {
         const size_t m = sizes.empty() ? o.m : sizes[i], n = sizes.empty() ? o.n : sizes[i], k = sizes.empty() ? o.k : sizes[i];
         bool ok = true;
         double g;
-        if (o.precision == "s") g = run_case<float>(o, (Fn)fn, m, n, k, ok);
-        else if (o.precision == "d") g = run_case<double>(o, (Fn)fn, m, n, k, ok);
-        else if (o.precision == "c") g = run_case<FloatComplex>(o, (Fn)fn, m, n, k, ok);
-        else g = run_case<DoubleComplex>(o, (Fn)fn, m, n, k, ok);
+        if (o.precision == "s") g = run_case<float>(o, (Fn)fn, m, n, k, stream, ok);
+        else if (o.precision == "d") g = run_case<double>(o, (Fn)fn, m, n, k, stream, ok);
+        else if (o.precision == "c") g = run_case<FloatComplex>(o, (Fn)fn, m, n, k, stream, ok);
+        else g = run_case<DoubleComplex>(o, (Fn)fn, m, n, k, stream, ok);
         if (!ok) { rc = 1; continue; }
         std::printf("%zu,%zu,%zu,%zu,%zu,%zu,%zu,%zu,%zu,%g,%g,%s,%s,%s,%s,%s,%s,%s%s,gpu,clblas_amd,1,%s,%g\n", m, n, k,
                     o.lda, o.ldb, o.ldc, o.offA, o.offBX, o.offCY, o.alpha, o.beta, o.order ? "column" : "row",
@@ -344,6 +343,9 @@ int main(int argc, char **argv) {
                     o.diag ? "nonunit" : "unit", o.precision.c_str(), o.function.c_str(), o.label.c_str(), g);
         std::fflush(stdout);
     }
+    HIP_OK(hipStreamSynchronize(stream));
+    clblasAmdReleaseStream(stream);
+    HIP_OK(hipStreamDestroy(stream));
     clblasTeardown();
     return rc;
 }

@@ -12,10 +12,14 @@
 //   src/library/blas/init.c:33-263 (GetVersion / Setup / Teardown).
 #include "../../include/clblas_amd.h"
 #include "internal.h"
+#include "workspace.hpp"
 
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
+#include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <utility>
@@ -23,72 +27,108 @@
 
 namespace cba {
 
-int forced_gemm_tile() {
-    const char *s = std::getenv("CLBLAS_AMD_GEMM_TILE");
-    if (!s || !*s) return -1;
-    return std::atoi(s);
-}
+namespace {
+DebugKnobs g_knobs;
+std::once_flag g_knobs_once;
 
-int debug_env_int(const char *name, int dflt) {
+int env_int(const char *name, int dflt) {
     const char *s = std::getenv(name);
     if (!s || !*s) return dflt;
     return std::atoi(s);
 }
 
+void read_knobs() {
+    DebugKnobs k;
+    k.gemm_tile = env_int("CLBLAS_AMD_GEMM_TILE", -1);
+    k.split_model = env_int("CLBLAS_AMD_GEMM_SPLIT_MODEL", 1);
+    k.splits = env_int("CLBLAS_AMD_GEMM_SPLITS", 0);
+    k.tail = env_int("CLBLAS_AMD_GEMM_TAIL", 1);
+    k.group_m = env_int("CLBLAS_AMD_GEMM_GROUP_M", 0);
+    k.xcd = env_int("CLBLAS_AMD_GEMM_XCD", 1);
+    k.stagger = env_int("CLBLAS_AMD_GEMM_STAGGER", 1);
+    k.fused_reduce = env_int("CLBLAS_AMD_GEMM_FUSED_REDUCE", 1);
+    k.log = env_int("CLBLAS_AMD_LOG", 0);
+    g_knobs = k;
+}
+}  // namespace
+
+const DebugKnobs &knobs() {
+    std::call_once(g_knobs_once, read_knobs);
+    return g_knobs;
+}
+
+// Debugging only: must not run while another thread is inside a library call.
+void reload_knobs() {
+    std::call_once(g_knobs_once, read_knobs);
+    read_knobs();
+}
+
+DispatchRecord &dispatch_record() {
+    static thread_local DispatchRecord rec;
+    return rec;
+}
+
 namespace {
-struct WsSlot {
-    void *ptr = nullptr;
-    size_t bytes = 0;
-};
-std::mutex g_ws_mutex;
-std::map<std::pair<std::pair<int, int>, hipStream_t>, WsSlot> g_ws;  // ((device, kind), stream) -> current buffer
-std::vector<std::pair<int, void *>> g_ws_retired;    // outgrown buffers, freed at teardown
+void *hip_ws_alloc(int device, size_t bytes) {
+    int cur = 0;
+    if (hipGetDevice(&cur) != hipSuccess) return nullptr;
+    if (cur != device && hipSetDevice(device) != hipSuccess) return nullptr;
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes) != hipSuccess) {
+        (void)hipGetLastError();  // the failed allocation is reported through the return value
+        p = nullptr;
+    }
+    if (cur != device) (void)hipSetDevice(cur);
+    return p;
+}
+void hip_ws_release(int device, void *ptr) {
+    int cur = 0;
+    (void)hipGetDevice(&cur);
+    if (cur != device) (void)hipSetDevice(device);
+    (void)hipFree(ptr);
+    if (cur != device) (void)hipSetDevice(cur);
+}
+void hip_ws_sync(int device) {
+    int cur = 0;
+    (void)hipGetDevice(&cur);
+    if (cur != device) (void)hipSetDevice(device);
+    (void)hipDeviceSynchronize();
+    if (cur != device) (void)hipSetDevice(cur);
+}
+WorkspaceCache &ws_cache() {
+    static WorkspaceCache cache(WorkspaceAllocator{hip_ws_alloc, hip_ws_release, hip_ws_sync});
+    return cache;
+}
 std::mutex g_lds_mutex;
 std::map<std::pair<int, const void *>, size_t> g_lds_limit;
 }  // namespace
 
-void *workspace_get(hipStream_t stream, size_t bytes, int kind) {
+hipError_t workspace_get(hipStream_t stream, size_t bytes, int kind, void **out) {
+    *out = nullptr;
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    WsSlot &slot = g_ws[std::make_pair(std::make_pair(dev, kind), stream)];
-    if (slot.bytes >= bytes && slot.ptr) return slot.ptr;
-    // Outgrown buffers stay allocated until teardown (kernels already enqueued may still use them), so
-    // grow by at least half: the retired ones then add up to at most twice the current size.
-    size_t want = bytes < (size_t)(1 << 20) ? (size_t)(1 << 20) : bytes;
-    if (want < slot.bytes + slot.bytes / 2) want = slot.bytes + slot.bytes / 2;
-    void *p = nullptr;
-    if (hipMalloc(&p, want) != hipSuccess) {
-        (void)hipGetLastError();
-        want = bytes;  // no room for the margin: try the size that is needed
-        if (hipMalloc(&p, want) != hipSuccess) {
-            (void)hipGetLastError();
-            return nullptr;
-        }
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    WorkspaceError why = WS_OK;
+    // Fast path: the buffer exists (no question about capture needed).
+    void *p = ws_cache().get(dev, (const void *)stream, kind, bytes, false, &why);
+    if (!p) {
+        // It has to be allocated: not on a stream that is being captured into a graph (hipMalloc
+        // there would fail and invalidate the capture).
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) cap = hipStreamCaptureStatusNone;
+        if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
+        p = ws_cache().get(dev, (const void *)stream, kind, bytes, true, &why);
+        if (!p) return hipErrorOutOfMemory;
     }
-    if (slot.ptr) g_ws_retired.push_back(std::make_pair(dev, slot.ptr));
-    slot.ptr = p;
-    slot.bytes = want;
-    return p;
+    *out = p;
+    return hipSuccess;
 }
 
-void workspace_release_all() {
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    int cur = 0;
-    (void)hipGetDevice(&cur);
-    for (auto &kv : g_ws) {
-        if (kv.second.ptr) {
-            (void)hipSetDevice(kv.first.first.first);
-            (void)hipFree(kv.second.ptr);
-        }
-    }
-    for (auto &r : g_ws_retired) {
-        (void)hipSetDevice(r.first);
-        (void)hipFree(r.second);
-    }
-    g_ws.clear();
-    g_ws_retired.clear();
-    (void)hipSetDevice(cur);
+void workspace_release_all() { ws_cache().release_all(); }
+void ws_release_stream(int device, hipStream_t stream) { ws_cache().release_stream(device, (const void *)stream); }
+void ws_stats(size_t *streams, size_t *bytes) {
+    if (streams) *streams = ws_cache().stream_count();
+    if (bytes) *bytes = ws_cache().bytes_held();
 }
 
 hipError_t ensure_dynamic_lds(const void *fn, size_t bytes) {
@@ -136,10 +176,14 @@ clblasStatus map_hip_error(hipError_t e) {
     if (e == hipErrorOutOfMemory) return clblasOutOfResources;
     if (e == hipErrorInvalidValue) return clblasInvalidValue;
     if (e == hipErrorNotSupported) return clblasNotImplemented;
+    if (e == hipErrorStreamCaptureUnsupported) return clblasInvalidOperation;  // would have had to allocate under capture
     return clblasOutOfResources;
 }
 
-const size_t kMaxDim = 0x7fffffff;  // kernels index tiles with 32-bit ints (reference: cl_uint, xgemm.cc:362-372)
+// Kernels index rows and columns with 32-bit ints (reference: cl_uint, xgemm.cc:362-372); the largest
+// index they form is a dimension rounded up to a whole tile (edge 256) plus one vector, so dimensions
+// stop one tile short of 2^31.
+const size_t kMaxDim = 0x7fffffff - 512;
 
 template <typename T>
 clblasStatus gemm_front(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M,
@@ -396,6 +440,45 @@ clblasStatus clblasSetup(void) {
 }
 
 void clblasTeardown(void) { cba::workspace_release_all(); }
+
+void clblasAmdReloadDebugEnv(void) { cba::reload_knobs(); }
+
+size_t clblasAmdLastDispatch(char *text, size_t size) {
+    const cba::DispatchRecord &r = cba::dispatch_record();
+    if (text && size) {
+        if (r.launches == 0)
+            std::snprintf(text, size, "none");
+        else
+            std::snprintf(text, size, "%s<%c,%dx%dx%d,%d threads> %c%c M=%d N=%d K=%d grid=(%u,%u) splits=%d%s tail_slices=%d%s",
+                          r.kernel, r.type, r.bm, r.bn, r.bk, r.threads, r.trans_a ? 'T' : 'N', r.trans_b ? 'T' : 'N',
+                          r.M, r.N, r.K, r.grid_x, r.grid_y, r.splits, r.fused_reduce ? " (summed in the same launch)" : "",
+                          r.tail_slices, r.tri ? " tri" : "");
+    }
+    return (size_t)r.launches;
+}
+
+clblasStatus clblasAmdReleaseStream(hipStream_t stream) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError();
+        return clblasInvalidDevice;
+    }
+    cba::ws_release_stream(dev, stream);
+    return clblasSuccess;
+}
+
+clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, size_t trmm_bytes, size_t trsm_bytes) {
+    const size_t want[3] = {gemm_bytes, trmm_bytes, trsm_bytes};
+    for (int kind = 0; kind < 3; ++kind) {
+        if (!want[kind]) continue;
+        void *p = nullptr;
+        hipError_t e = cba::workspace_get(stream, want[kind], kind, &p);
+        if (e != hipSuccess) return map_hip_error(e);
+    }
+    return clblasSuccess;
+}
+
+void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes) { cba::ws_stats(streams, bytes); }
 
 clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
                          size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B, size_t offB,

@@ -34,10 +34,11 @@ static const TileEntry<float> *f32_tiles(int *n) {
 }
 
 hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float alpha, const float *A, int64_t lda,
-                          const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream, const GemmTri *tri) {
+                          const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream, const GemmTri *tri,
+                          const FixedScratch *fixed) {
     int n;
     const TileEntry<float> *tab = f32_tiles(&n);
-    return run_gemm_colmajor<float>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, tri);
+    return run_gemm_colmajor<float>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, tri, fixed);
 }
 
 }  // namespace cba

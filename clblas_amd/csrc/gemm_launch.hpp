@@ -6,6 +6,8 @@
 // compiled ahead of time, so "selection" is only a table lookup.
 #pragma once
 
+#include <cstdio>
+
 #include "gemm_kernel.hpp"
 #include "internal.h"
 
@@ -77,6 +79,44 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
 }
 
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// 1-D grids are built from 64-bit products; HIP takes 32-bit block counts.
+static const int64_t kMaxGrid = 0x7fffffffLL;
+
+template <typename T> static char type_letter() {
+    return Elem<T>::CPLX ? (sizeof(T) == 8 ? 'c' : 'z') : (sizeof(T) == 4 ? 's' : 'd');
+}
+
+// Records the launch for clblasAmdLastDispatch and, with CLBLAS_AMD_LOG=1, prints it.
+template <typename T>
+static DispatchRecord &note_launch(const char *kernel, int bm, int bn, int bk, int threads, bool tA, bool tB, int M,
+                                   int N, int K, unsigned gx, unsigned gy) {
+    DispatchRecord &r = dispatch_record();
+    r.type = type_letter<T>(); r.kernel = kernel;
+    r.bm = bm; r.bn = bn; r.bk = bk; r.threads = threads;
+    r.trans_a = tA; r.trans_b = tB; r.M = M; r.N = N; r.K = K;
+    r.splits = 1; r.tail_slices = 1; r.tri = 0; r.fused_reduce = 0;
+    r.grid_x = gx; r.grid_y = gy;
+    r.launches++;
+    return r;
+}
+static inline void log_dispatch(const DispatchRecord &r) {
+    if (knobs().log)
+        fprintf(stderr, "clblas_amd: %s<%c,%dx%dx%d> %c%c M=%d N=%d K=%d grid=(%u,%u) block=%d splits=%d tail_slices=%d tri=%d\n",
+                r.kernel, r.type, r.bm, r.bn, r.bk, r.trans_a ? 'T' : 'N', r.trans_b ? 'T' : 'N', r.M, r.N, r.K, r.grid_x,
+                r.grid_y, r.threads, r.splits, r.tail_slices, r.tri);
+}
+
+// Scratch for this call: the caller's fixed buffer if there is one, else the per-stream cache.
+static inline hipError_t scratch_for(hipStream_t stream, size_t bytes, const FixedScratch *fixed, void **out) {
+    if (fixed) {
+        *out = nullptr;
+        if (bytes > fixed->bytes) return hipErrorOutOfMemory;
+        *out = fixed->ptr;
+        return hipSuccess;
+    }
+    return workspace_get(stream, bytes, 0, out);
+}
 
 // Chooses tile and split count.  The reference keys its choice on M*N brackets and
 // divisibility (AutoGemmParameters.py:8-55); here remainders are handled in-kernel, so the
@@ -163,7 +203,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             return (double)ceil_div64(t * s, kCUs) * tab[i].bm * tab[i].bn / (s * tab[i].eff * alone) +
                    split_overhead_cost<T>(M, N, K, s);
         };
-        const bool split_model = debug_env_int("CLBLAS_AMD_GEMM_SPLIT_MODEL", 1) != 0 && !need_tri;
+        const bool split_model = knobs().split_model != 0 && !need_tri;
         double best = 0, best_split = 0;
         int pick_of_split = -1;
         bool have = false;
@@ -226,7 +266,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         const int by_rule = splits_for(ceil_div64(M, tab[pick].bm) * ceil_div64(N, tab[pick].bn), K, tab[pick].bk);
         if (model_splits >= 0) splits = model_splits;
         else if (pick_split) splits = by_rule;
-        const int forced = debug_env_int("CLBLAS_AMD_GEMM_SPLITS", 0);  // debug: number of K ranges
+        const int forced = knobs().splits;  // debug: number of K ranges
         const int most = K / (4 * tab[pick].bk) > 0 ? K / (4 * tab[pick].bk) : 1;  // 4 panels per range
         if (forced > 0) splits = forced < most ? forced : most;
     }
@@ -237,14 +277,16 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
 template <typename T>
 static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, bool tB, bool cA, bool cB, int M,
                                     int N, int K, T alpha, const T *A, int64_t lda, const T *B, int64_t ldb,
-                                    T beta, T *C, int64_t ldc, hipStream_t stream, const GemmTri *tri = nullptr) {
+                                    T beta, T *C, int64_t ldc, hipStream_t stream, const GemmTri *tri = nullptr,
+                                    const FixedScratch *fixed = nullptr) {
     const bool need_tri = tri && tri->any();
     if (need_tri && K == 0) return hipErrorInvalidValue;  // callers reject empty products earlier
     if (K == 0) {
         int mb = (int)ceil_div64(M, 256);
-        hipLaunchKernelGGL(scale_c_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
-                           beta, C, ldc);
-        return hipGetLastError();
+        if ((int64_t)mb * N > kMaxGrid) return hipErrorInvalidValue;
+        log_dispatch(note_launch<T>("scale_c_kernel", 0, 0, 0, 256, tA, tB, M, N, K, (unsigned)((int64_t)mb * N), 1));
+        return launch_kernel(scale_c_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
+                             beta, C, ldc);
     }
     // 32-bit panel offsets: (tile edge or panel depth) * ld * sizeof(T) must stay < 2^31.
     const int64_t max_edge = 256;
@@ -252,16 +294,17 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     if (lda > ld_limit || ldb > ld_limit) {
         if (need_tri) return hipErrorNotSupported;
         int mb = (int)ceil_div64(M, 256);
-        hipLaunchKernelGGL(gemm_wide_ld_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream,
-                           tA ? 1 : 0, tB ? 1 : 0, cA ? 1 : 0, cB ? 1 : 0, M, N, K, mb, alpha, A, lda, B, ldb, beta, C,
-                           ldc);
-        return hipGetLastError();
+        if ((int64_t)mb * N > kMaxGrid) return hipErrorInvalidValue;
+        log_dispatch(note_launch<T>("gemm_wide_ld_kernel", 0, 0, 0, 256, tA, tB, M, N, K, (unsigned)((int64_t)mb * N), 1));
+        return launch_kernel(gemm_wide_ld_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream,
+                             tA ? 1 : 0, tB ? 1 : 0, cA ? 1 : 0, cB ? 1 : 0, M, N, K, mb, alpha, A, lda, B, ldb, beta,
+                             C, ldc);
     }
 
     int tile, splits;
     // The tail may be sliced unless tiles differ in depth (triangular operands).
-    const bool tail_ok = !(need_tri && (tri->tri_a || tri->tri_b)) && debug_env_int("CLBLAS_AMD_GEMM_TAIL", 1) != 0;
-    choose_tile(tab, ntab, M, N, K, forced_gemm_tile(), need_tri, need_tri ? tri->tri_c : 0,
+    const bool tail_ok = !(need_tri && (tri->tri_a || tri->tri_b)) && knobs().tail != 0;
+    choose_tile(tab, ntab, M, N, K, knobs().gemm_tile, need_tri, need_tri ? tri->tri_c : 0,
                 need_tri && (tri->tri_a || tri->tri_b), tail_ok, &tile, &splits);
     const TileEntry<T> &e = tab[tile];
 
@@ -287,10 +330,10 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         const double resident = e.smem_of[0] > 40 * 1024 ? 64.0 : 128.0;
         while ((double)(2 * gm_default) * (2 * gm_default) <= resident * e.bn / e.bm && gm_default < 16) gm_default *= 2;
     }
-    p.group_m = debug_env_int("CLBLAS_AMD_GEMM_GROUP_M", gm_default);
+    p.group_m = knobs().group_m > 0 ? knobs().group_m : gm_default;
     if (p.group_m > p.tiles_m) p.group_m = p.tiles_m;
     if (p.group_m < 1) p.group_m = 1;
-    p.xcd_remap = debug_env_int("CLBLAS_AMD_GEMM_XCD", 1);
+    p.xcd_remap = knobs().xcd;
     p.stagger = 0;
     p.ws = nullptr; p.ws_ld = 0; p.ws_slice = 0;
     p.k_per_split = K;
@@ -325,8 +368,16 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             const int64_t kps = ceil_div64(ceil_div64(K, ts), e.bk) * e.bk;
             const int slices = (int)ceil_div64(K, kps);
             const int64_t r = ntiles % 256;
-            void *w = workspace_get(stream, (size_t)(r * slices) * e.bm * e.bn * sizeof(T));
-            if (slices > 1 && w) {  // without workspace the plain schedule still works
+            void *w = nullptr;
+            const size_t need = (size_t)(r * slices) * e.bm * e.bn * sizeof(T);
+            if (slices > 1) {
+                hipError_t we = scratch_for(stream, need, fixed, &w);
+                // A caller that must not allocate gets an error rather than another schedule (its
+                // results then never depend on what happens to be allocated); so does a stream
+                // under capture.  Plain out-of-memory falls back to the unsliced schedule.
+                if (we != hipSuccess && (fixed || we != hipErrorOutOfMemory)) return we;
+            }
+            if (slices > 1 && w) {
                 fn = e.tri[idx];
                 p.tail_first = (int)(ntiles - r);
                 p.tail_slices = slices;
@@ -343,8 +394,9 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             p.k_per_split = (int)kps;
             p.ws_ld = ((int64_t)M + 63) / 64 * 64;
             p.ws_slice = p.ws_ld * N;
-            void *w = workspace_get(stream, (size_t)(p.ws_slice * splits) * sizeof(T));
-            if (!w) return hipErrorOutOfMemory;
+            void *w = nullptr;
+            hipError_t we = scratch_for(stream, (size_t)(p.ws_slice * splits) * sizeof(T), fixed, &w);
+            if (we != hipSuccess) return we;
             p.ws = (T *)w;
             fn = e.splitk[idx];
         }
@@ -356,7 +408,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     {
         const int64_t wgs = grid_x * (splits > 1 ? splits : 1);
         const bool whole_rounds = p.tail_slices <= 1 && wgs % 512 == 0;
-        const int mode = debug_env_int("CLBLAS_AMD_GEMM_STAGGER", 1);  // 0: never
+        const int mode = knobs().stagger;  // 0: never
         p.stagger = mode != 0 && wgs > 512 && !(p.tri_a || p.tri_b) && (!whole_rounds || p.k_per_split <= 2048);
     }
     const size_t smem = e.smem_of[idx];
@@ -364,21 +416,28 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         hipError_t err = ensure_dynamic_lds((const void *)fn, smem);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(fn, dim3((unsigned)grid_x, (unsigned)splits), dim3(e.threads), smem, stream, p);
-    hipError_t err = hipGetLastError();
+    if (grid_x > kMaxGrid) return hipErrorInvalidValue;
+    {
+        DispatchRecord &rec = note_launch<T>("gemm_mfma_kernel", e.bm, e.bn, e.bk, e.threads, tA, tB, M, N, K,
+                                             (unsigned)grid_x, (unsigned)splits);
+        rec.splits = splits; rec.tail_slices = p.tail_slices; rec.tri = need_tri ? 1 : 0;
+        log_dispatch(rec);
+    }
+    hipError_t err = launch_kernel(fn, dim3((unsigned)grid_x, (unsigned)splits), dim3(e.threads), smem, stream, p);
     if (err != hipSuccess) return err;
     if (p.tail_slices > 1) {
         const int64_t r = ntiles - p.tail_first;
-        hipLaunchKernelGGL(tail_reduce_kernel<T>, dim3((unsigned)ceil_div64((int64_t)e.bm * e.bn, 256), (unsigned)r),
-                           dim3(256), 0, stream, p, e.bm, e.bn);
-        err = hipGetLastError();
+        dispatch_record().launches++;
+        err = launch_kernel(tail_reduce_kernel<T>, dim3((unsigned)ceil_div64((int64_t)e.bm * e.bn, 256), (unsigned)r),
+                            dim3(256), 0, stream, p, e.bm, e.bn);
         if (err != hipSuccess) return err;
     }
     if (splits > 1) {
         int mb = (int)ceil_div64(M, 256);
-        hipLaunchKernelGGL(splitk_reduce_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, p.ws,
-                           p.ws_ld, p.ws_slice, splits, M, N, mb, alpha, beta, C, ldc);
-        err = hipGetLastError();
+        if ((int64_t)mb * N > kMaxGrid) return hipErrorInvalidValue;
+        dispatch_record().launches++;
+        err = launch_kernel(splitk_reduce_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, p.ws,
+                            p.ws_ld, p.ws_slice, splits, M, N, mb, alpha, beta, C, ldc);
     }
     return err;
 }

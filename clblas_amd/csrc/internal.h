@@ -6,26 +6,72 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 namespace cba {
+
+// Launches `fn` and returns the status of THIS launch.  (The <<<>>> form reports through the
+// thread's sticky error, which would also pick up - and clear - an error that unrelated code of
+// the caller left there.)
+template <typename... KArgs, size_t... I>
+inline hipError_t launch_kernel_impl(void (*fn)(KArgs...), dim3 grid, dim3 block, size_t smem, hipStream_t stream,
+                                     std::tuple<KArgs...> &args, std::index_sequence<I...>) {
+    void *ptrs[] = {(void *)&std::get<I>(args)..., nullptr};
+    return hipLaunchKernel((const void *)fn, grid, block, ptrs, smem, stream);
+}
+template <typename... KArgs, typename... Args>
+inline hipError_t launch_kernel(void (*fn)(KArgs...), dim3 grid, dim3 block, size_t smem, hipStream_t stream,
+                                Args &&...args) {
+    static_assert(sizeof...(KArgs) == sizeof...(Args), "argument count");
+    std::tuple<KArgs...> t(static_cast<KArgs>(args)...);
+    return launch_kernel_impl(fn, grid, block, smem, stream, t, std::index_sequence_for<KArgs...>());
+}
 
 // Complex element, laid out as the reference's FloatComplex / DoubleComplex (cl_float2 /
 // cl_double2, src/clBLAS-complex.h:25-26: real part first).
 template <typename R> struct Cx { R re, im; };
 
-// Debug-only override of the GEMM tile choice: index into the per-type tile table taken
-// from the environment variable CLBLAS_AMD_GEMM_TILE, or -1.
-int forced_gemm_tile();
+// Debug switches, read from the environment once (first use) and again only when
+// clblasAmdReloadDebugEnv() is called: the launch path itself never calls getenv.
+//   CLBLAS_AMD_GEMM_TILE (index into the per-type tile table, -1: model's choice), _SPLIT_MODEL,
+//   _SPLITS, _TAIL, _GROUP_M (0: default), _XCD, _STAGGER: see the tile choice in gemm_launch.hpp;
+//   CLBLAS_AMD_LOG=1: one line per kernel launch on stderr.
+struct DebugKnobs {
+    int gemm_tile = -1, split_model = 1, splits = 0, tail = 1, group_m = 0, xcd = 1, stagger = 1, log = 0;
+    int fused_reduce = 1;  // CLBLAS_AMD_GEMM_FUSED_REDUCE=0: K ranges are added up by a second launch
+};
+const DebugKnobs &knobs();
+void reload_knobs();
 
-// Debug-only integer knob from the environment (tile walk order experiments), or `dflt`.
-int debug_env_int(const char *name, int dflt);
+// What the last GEMM launch of the calling thread was (diagnostics: clblasAmdLastDispatch).
+struct DispatchRecord {
+    char type = '?';           // s, d, c, z
+    int bm = 0, bn = 0, bk = 0, threads = 0;
+    int trans_a = 0, trans_b = 0;
+    int M = 0, N = 0, K = 0;
+    int splits = 1, tail_slices = 1, tri = 0, fused_reduce = 0;
+    unsigned grid_x = 0, grid_y = 0;
+    unsigned long long launches = 0;  // kernel launches by this thread since the library was loaded
+    const char *kernel = "";          // kernel family ("gemm_mfma_kernel", "gemm_wide_ld_kernel", ...)
+};
+DispatchRecord &dispatch_record();  // thread-local
 
-// Library-owned device scratch for `stream` on the current device, at least `bytes` long.
-// Grown on demand; earlier, smaller buffers stay alive until clblasTeardown so that work
-// already enqueued on them remains valid.  Returns nullptr if the allocation fails.
-// `kind` separates buffers that are alive at the same time (0: split-K partial sums,
-// 1: the operand copy of an in-place routine).
-void *workspace_get(hipStream_t stream, size_t bytes, int kind = 0);
+// Library-owned device scratch for `stream` on the current device, at least `bytes` long
+// (kinds: workspace.hpp).  Grown on demand; see workspace.hpp for the lifetime rules.
+// hipErrorOutOfMemory if the allocation fails; hipErrorStreamCaptureUnsupported if `stream`
+// is being captured into a graph and the buffer would have to be allocated now.
+hipError_t workspace_get(hipStream_t stream, size_t bytes, int kind, void **out);
 void workspace_release_all();
+void ws_release_stream(int device, hipStream_t stream);
+void ws_stats(size_t *streams, size_t *bytes);
+
+// Caller-supplied scratch that replaces workspace_get for one call (the entry point that
+// must not allocate): requests beyond `bytes` fail with hipErrorOutOfMemory.
+struct FixedScratch {
+    void *ptr;
+    size_t bytes;
+};
 
 // Raises a kernel's dynamic LDS limit (needed above 64 KiB); cached per function.
 hipError_t ensure_dynamic_lds(const void *fn, size_t bytes);
@@ -46,7 +92,7 @@ struct GemmTri {
 // major; pointers already include their element offsets.
 hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float alpha, const float *A, int64_t lda,
                           const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream,
-                          const GemmTri *tri = nullptr);
+                          const GemmTri *tri = nullptr, const FixedScratch *fixed = nullptr);
 hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double alpha, const double *A,
                           int64_t lda, const double *B, int64_t ldb, double beta, double *C, int64_t ldc,
                           hipStream_t stream, const GemmTri *tri = nullptr);

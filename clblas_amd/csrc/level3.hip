@@ -67,13 +67,15 @@ template <typename T>
 hipError_t trmm_colmajor(bool right, bool lower, bool trans, bool conj, bool unit, int M, int N, T alpha, const T *A,
                          int64_t lda, T *B, int64_t ldb, hipStream_t stream) {
     const int64_t ldw = ((int64_t)M + 63) / 64 * 64;
-    T *W = (T *)workspace_get(stream, (size_t)ldw * N * sizeof(T), 1);
-    if (!W) return hipErrorOutOfMemory;
+    void *wv = nullptr;
+    hipError_t err = workspace_get(stream, (size_t)ldw * N * sizeof(T), 1, &wv);
+    if (err != hipSuccess) return err;
+    T *W = (T *)wv;
     const int mb = (M + 255) / 256;
     if ((int64_t)mb * N > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(copy_matrix_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
-                       (const T *)B, ldb, W, ldw);
-    hipError_t err = hipGetLastError();
+    dispatch_record().launches++;
+    err = launch_kernel(copy_matrix_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
+                        (const T *)B, ldb, W, ldw);
     if (err != hipSuccess) return err;
     GemmTri tri;
     const bool op_lower = lower != trans;  // op(A) is lower triangular

@@ -425,16 +425,17 @@ template <typename T> struct TrsmDriver {
         typedef TrsmLeaf<T> L;
         const int n = right ? N : M;
         const int nblk = (n + NBL - 1) / NBL;
-        R *w = (R *)workspace_get(stream, (size_t)nblk * L::PACK_REALS * sizeof(R), 2);
-        if (!w) return hipErrorOutOfMemory;
+        void *wv = nullptr;
+        hipError_t we = workspace_get(stream, (size_t)nblk * L::PACK_REALS * sizeof(R), 2, &wv);
+        if (we != hipSuccess) return we;
+        R *w = (R *)wv;
         pack = w;
+        dispatch_record().launches++;
         if (forward)
-            hipLaunchKernelGGL((trsm_pack_kernel<T, true>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
-                               conj, unit, w);
-        else
-            hipLaunchKernelGGL((trsm_pack_kernel<T, false>), dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
-                               conj, unit, w);
-        return hipGetLastError();
+            return launch_kernel(trsm_pack_kernel<T, true>, dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
+                                 conj, unit, w);
+        return launch_kernel(trsm_pack_kernel<T, false>, dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
+                             conj, unit, w);
     }
 
     template <bool RIGHT> hipError_t leaf_side(int i0, int nb, T alpha) {
@@ -449,8 +450,8 @@ template <typename T> struct TrsmDriver {
             if (e != hipSuccess) return e;
         }
         dim3 grid((unsigned)((nrhs + L::CW - 1) / L::CW)), block(L::THREADS);
-        hipLaunchKernelGGL(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs);
-        return hipGetLastError();
+        dispatch_record().launches++;
+        return launch_kernel(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs);
     }
     hipError_t leaf(int i0, int nb, T alpha) { return right ? leaf_side<true>(i0, nb, alpha) : leaf_side<false>(i0, nb, alpha); }
 

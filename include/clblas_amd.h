@@ -297,6 +297,41 @@ clblasStatus clblasZhemm(clblasOrder order, clblasSide side, clblasUplo uplo, si
                          const DoubleComplex *B, size_t offB, size_t ldb, DoubleComplex beta,
                          DoubleComplex *C, size_t offC, size_t ldc, hipStream_t stream); /* src/clBLAS.h:9305-9326 */
 
+/* ---- Workspace and diagnostics.  These four have no counterpart in the reference: clBLAS allocates
+ * and frees its temporaries inside every call (src/library/blas/xtrsm.cc:1186-1207, 1499-1500) and
+ * logs nothing; this library keeps scratch buffers per (device, stream) and lets the caller
+ * manage them. ---- */
+
+/* Frees the scratch buffers kept for `stream` on the current device.  Call it after the stream's
+ * work has completed and before destroying the stream.  Without it a process still holds a
+ * bounded amount: at most 32 streams per device keep buffers, the least recently used one is
+ * evicted (after a device synchronisation) when another appears. */
+clblasStatus clblasAmdReleaseStream(hipStream_t stream);
+
+/* Makes sure the scratch buffers of `stream` on the current device are at least this large
+ * (bytes; 0 leaves a buffer alone): gemm_bytes for GEMM-shaped calls that cut K into ranges
+ * (ranges x M x N elements, M rounded up to 64) or slice their last round of tiles (at most 256
+ * tiles of 256 x 128 elements), trmm_bytes for TRMM's copy of B (M x N elements), trsm_bytes
+ * for TRSM's packed diagonal blocks (about 35 000 elements per 256 rows of the triangle; three
+ * times that for complex types).  A later call on the stream whose needs fit allocates nothing,
+ * so it can be the first thing recorded into a HIP graph.  A call that would have to allocate
+ * while its stream is being captured returns clblasInvalidOperation and leaves the capture valid. */
+clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, size_t trmm_bytes, size_t trsm_bytes);
+
+/* Number of streams that hold scratch buffers, and the bytes of their current buffers. */
+void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes);
+
+/* Describes the last GEMM kernel the calling thread launched (kernel family, tile, transposes,
+ * sizes, grid, K ranges), as text; returns the number of kernel launches the thread has issued
+ * through this library.  With CLBLAS_AMD_LOG=1 in the environment every launch also prints
+ * such a line on stderr. */
+size_t clblasAmdLastDispatch(char *text, size_t size);
+
+/* The library reads its debugging environment variables (CLBLAS_AMD_*) once, at first use.
+ * This reads them again.  Debugging only: not to be called while another thread is inside a
+ * library call. */
+void clblasAmdReloadDebugEnv(void);
+
 #ifdef __cplusplus
 }
 #endif

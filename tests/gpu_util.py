@@ -16,13 +16,9 @@ def gemm(order, tA, tB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, off
     fn = {np.dtype(np.float32): clblas_amd.sgemm, np.dtype(np.float64): clblas_amd.dgemm,
           np.dtype(np.complex64): clblas_amd.cgemm, np.dtype(np.complex128): clblas_amd.zgemm}[C.dtype]
     dA, dB, dC = _dev(A), _dev(B), _dev(C)
-    if tile is not None:
-        os.environ["CLBLAS_AMD_GEMM_TILE"] = str(tile)
-    try:
+    with _forced_tile(tile):
         st = fn(order, tA, tB, M, N, K, alpha, dA, offA, lda, dB, offB, ldb, beta, dC, offC, ldc)
         torch.cuda.synchronize()
-    finally:
-        os.environ.pop("CLBLAS_AMD_GEMM_TILE", None)
     return st, dC.cpu().numpy()
 
 
@@ -35,15 +31,27 @@ def trsm(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B, offB, ldb):
     return st, dB.cpu().numpy()
 
 
-def _forced_tile(tile):
-    class _Ctx:
-        def __enter__(self):
-            if tile is not None:
-                os.environ["CLBLAS_AMD_GEMM_TILE"] = str(tile)
+class debug_env:
+    """Sets CLBLAS_AMD_* debugging variables for the calls inside the block.  The library reads
+    its environment once, so it is told to read it again on the way in and on the way out."""
 
-        def __exit__(self, *a):
-            os.environ.pop("CLBLAS_AMD_GEMM_TILE", None)
-    return _Ctx()
+    def __init__(self, **kv):
+        self.kv = {k: str(v) for k, v in kv.items() if v is not None}
+
+    def __enter__(self):
+        if self.kv:
+            os.environ.update(self.kv)
+            clblas_amd.reload_debug_env()
+
+    def __exit__(self, *a):
+        if self.kv:
+            for k in self.kv:
+                os.environ.pop(k, None)
+            clblas_amd.reload_debug_env()
+
+
+def _forced_tile(tile):
+    return debug_env(CLBLAS_AMD_GEMM_TILE=tile)
 
 
 _PREFIX = {np.dtype(np.float32): "S", np.dtype(np.float64): "D", np.dtype(np.complex64): "C",
