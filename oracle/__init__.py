@@ -335,6 +335,45 @@ def ref_trsm(order, side, uplo, transA, diag, M, N, alpha, A, lda, B, ldb):
     f(int(order), int(side), int(uplo), int(transA), int(diag), M, N, alpha, _p(A), lda, _p(B), ldb)
 
 
+_TYPE_CODE = {np.dtype(np.float32): 0, np.dtype(np.float64): 1, np.dtype(np.complex64): 2, np.dtype(np.complex128): 3}
+
+
+def trsm_ref_inputs(dtype, order, side, uplo, diag, M, N, alpha, offA, lda, offB, ldb, seed):
+    """(A, B) buffers of the reference TRSM test's input family (oracle_trsm_ref_inputs): NaN in
+    every element the routine must not read, B already divided by alpha where |alpha| != 1."""
+    dtype = np.dtype(dtype)
+    limA = M if side == 0 else N
+    rows_b, cols_b = (M, N) if order == 1 else (N, M)   # (contiguous extent, strides) of B in memory
+    lenA = offA + lda * limA
+    lenB = offB + ldb * cols_b
+    assert lda >= limA and ldb >= rows_b
+    A = np.empty(lenA, dtype=dtype)
+    B = np.empty(lenB, dtype=dtype)
+    al = np.array([complex(alpha).real, complex(alpha).imag], dtype=np.float64)
+    f = lib().oracle_trsm_ref_inputs
+    f.restype = None
+    f.argtypes = [_i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp, _sz, _sz, _sz, _u64]
+    f(_TYPE_CODE[dtype], int(order), int(side), int(uplo), int(diag), M, N, _p(al), _p(A), offA, lda, lenA, _p(B), offB,
+      ldb, lenB, seed)
+    return A, B
+
+
+def trsm_hp(order, side, uplo, transA, diag, M, N, alpha, A, offA, lda, B, offB, ldb, rhs):
+    """Solutions of the right-hand sides `rhs` (columns of B for side left, rows for right) by
+    substitution in long double, rounded to double: array (len(rhs), n), float64 or complex128."""
+    n = M if side == 0 else N
+    rhs = np.ascontiguousarray(rhs, dtype=np.uintp)
+    X = np.empty((len(rhs), n), dtype=np.complex128)
+    al = np.array([complex(alpha).real, complex(alpha).imag], dtype=np.float64)
+    f = lib().oracle_trsm_hp
+    f.restype = _i
+    f.argtypes = [_i, _i, _i, _i, _i, _i, _sz, _sz, _vp, _vp, _sz, _sz, _vp, _sz, _sz, _vp, _sz, _vp]
+    st = f(_TYPE_CODE[np.dtype(B.dtype)], int(order), int(side), int(uplo), int(transA), int(diag), M, N, _p(al), _p(A),
+           offA, lda, _p(B), offB, ldb, _p(rhs), len(rhs), _p(X))
+    assert st == 0, st
+    return X if _is_complex(B) else np.ascontiguousarray(X.real)
+
+
 # ---- seeded generators -------------------------------------------------------------------
 
 def uniform(n, seed, dtype=np.float32):

@@ -47,6 +47,8 @@
  *                             reference's own naive syr2k (oracle/_ref); HEMM against oracle
  *                             GEMM on the explicitly formed Hermitian matrix; HER2K with B == A
  *                             against HERK.  (The reference has no naive herk / her2k / hemm.)
+ *   oracle_trsm_ref_inputs, oracle_trsm_hp (trsm_reftest.inc)
+ *                           - see the header of that file (tests/test_oracle_trsm_reftest.py).
  *   oracle_check_*          - expectations of src/tests/functional/func-error.cpp:58-104 and
  *                             the branch table of generic/common.c:585-688.
  *   Bit-for-bit output of the OpenCL kernels (implementation-defined `mad` contraction,
@@ -677,3 +679,8 @@ void oracle_fill_int_f64(double *x, size_t n, uint64_t seed, uint32_t limit) {
     }
 FILL_TRI(oracle_fill_tri_f32, float)
 FILL_TRI(oracle_fill_tri_f64, double)
+
+/* ------------------------------------------------------------------------------------ */
+/* The reference TRSM test's input family and a long double solver to judge against       */
+/* ------------------------------------------------------------------------------------ */
+#include "trsm_reftest.inc"

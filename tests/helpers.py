@@ -89,3 +89,99 @@ def golden_array(values, dtype):
 
 def golden_scalar(v):
     return complex(v[0], v[1]) if isinstance(v, list) else v
+
+
+# ---- the reference's own yardstick for TRSM --------------------------------------------------
+
+TRSM_DELTA_0 = {np.dtype(np.float32): 2.0 ** -20, np.dtype(np.float64): 2.0 ** -50,
+                np.dtype(np.complex64): 2.0 ** -20, np.dtype(np.complex128): 2.0 ** -50}
+
+
+def trsm_ref_delta(dtype, side, uplo, transA, diag, alpha, abs_diag, abs_b):
+    """Per-element bound of the reference's TRSM correctness test, trsmDelta
+    (src/tests/correctness/trsm-delta.h:44-240), for selected right-hand sides.
+
+    abs_diag: |a_pp|, length n (n = M for side left, N for right).  abs_b: |b| of the ORIGINAL
+    right-hand sides, shape (nsel, n) (columns of B for left, rows for right).  Returns the bound
+    in the same shape; the reference applies it to |reference BLAS result - clBLAS result|
+    (complex: to the real and to the imaginary part, src/tests/include/matrix.h:372-400).
+
+    Restated: s_p = |b_p / a_pp| * DELTA_0 * |alpha| (no division for a unit diagonal), summed
+    along the direction of the substitution ("Gauss' method" part), plus a part for the block
+    algorithm with block size 32 (16 for double complex): weights z = 1, 2, ... over the
+    same-offset elements of the blocks the substitution has passed, times the block size.  For
+    side right with a lower effective triangle the reference's block loop runs from block k/bs to
+    (k + bs - 1)/bs, i.e. over at most one block (:216-218); that is kept as it is."""
+    dtype = np.dtype(dtype)
+    n = abs_b.shape[1]
+    bs = 16 if dtype == np.dtype(np.complex128) else 32
+    is_upper = (uplo == UPPER) == (transA == NOTRANS)
+    forward = (side == LEFT) != is_upper
+    s = abs_b.astype(np.float64)
+    if diag == NONUNIT:
+        s = s / abs_diag[None, :]
+    s = s * (TRSM_DELTA_0[dtype] * abs(alpha))
+    if not forward:
+        s = s[:, ::-1]
+    gauss = np.cumsum(s, axis=1)
+    if not forward:
+        gauss = gauss[:, ::-1]
+    nb = (n + bs - 1) // bs
+    g = np.zeros((abs_b.shape[0], nb * bs))
+    g[:, :n] = gauss
+    g = g.reshape(-1, nb, bs)
+    if forward:
+        blk = np.cumsum(np.cumsum(g, axis=1), axis=1)               # sum_{j<=pb} (pb+1-j) g[j]
+    elif side == LEFT:
+        blk = np.cumsum(np.cumsum(g[:, ::-1], axis=1), axis=1)[:, ::-1]   # sum_{j>=pb} (j-pb+1) g[j]
+    else:
+        blk = g.copy()
+        blk[:, :, 0] = 0.0                                          # empty block range when k % bs == 0
+    blk = blk.reshape(-1, nb * bs)[:, :n]
+    return gauss + bs * blk
+
+
+def trsm_ref_delta_loops(dtype, side, uplo, transA, diag, alpha, abs_diag, abs_b):
+    """The same bound written as the reference's loops (one right-hand side at a time); used only
+    to check the vectorised form above."""
+    dtype = np.dtype(dtype)
+    nsel, n = abs_b.shape
+    bs = 16 if dtype == np.dtype(np.complex128) else 32
+    is_upper = (uplo == UPPER) == (transA == NOTRANS)
+    d0 = TRSM_DELTA_0[dtype]
+    out = np.zeros((nsel, n))
+    for q in range(nsel):
+        delta = np.zeros(n)
+        s = [(abs_b[q, p] / abs_diag[p] if diag == NONUNIT else abs_b[q, p]) * d0 * abs(alpha) for p in range(n)]
+        if side == LEFT:
+            order = range(n - 1, -1, -1) if is_upper else range(n)
+        else:
+            order = range(n) if is_upper else range(n - 1, -1, -1)
+        prev = None
+        for p in order:
+            delta[p] = s[p] + (delta[prev] if prev is not None else 0.0)
+            prev = p
+        cl = np.zeros(n)
+        for p in range(n):
+            if side == LEFT:
+                if is_upper:
+                    j0, j1, z, zinc = p // bs, (n + bs - 1) // bs, 1, 1
+                else:
+                    j0, j1 = 0, p // bs + 1
+                    z, zinc = j1 - j0, -1
+            else:
+                if is_upper:
+                    j0, j1 = 0, p // bs + 1
+                    z, zinc = j1 - j0, -1
+                else:
+                    j0, j1, z, zinc = p // bs, (p + bs - 1) // bs, 1, 1
+            acc = 0.0
+            for j in range(j0, j1):
+                idx = j * bs + p % bs
+                if idx >= n:
+                    continue
+                acc += z * delta[idx]
+                z += zinc
+            cl[p] = acc * bs
+        out[q] = delta + cl
+    return out
