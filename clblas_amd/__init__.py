@@ -68,6 +68,7 @@ EXPORTED_SYMBOLS = (
     "clblasSetup",
     "clblasTeardown",
     "clblasSgemm",
+    "clblasSgemmNoAlloc",
     "clblasDgemm",
     "clblasCgemm",
     "clblasZgemm",
@@ -95,7 +96,8 @@ class DoubleComplex(ctypes.Structure):
 
 def _declare(lib):
     sz, vp, i = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_int
-    for name, real in (("clblasSgemm", ctypes.c_float), ("clblasDgemm", ctypes.c_double)):
+    for name, real in (("clblasSgemm", ctypes.c_float), ("clblasSgemmNoAlloc", ctypes.c_float),
+                       ("clblasDgemm", ctypes.c_double)):
         fn = getattr(lib, name)
         fn.restype = i
         fn.argtypes = [i, i, i, sz, sz, sz, real, vp, sz, sz, vp, sz, sz, real, vp, sz, sz, vp]
@@ -232,6 +234,12 @@ def get_version():
 def sgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
     return load_library().clblasSgemm(int(order), int(transA), int(transB), M, N, K, alpha, _ptr(A), offA, lda,
                                       _ptr(B), offB, ldb, beta, _ptr(C), offC, ldc, _stream(stream))
+
+
+def sgemm_noalloc(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):
+    """clblasSgemmNoAlloc: clblasSgemm on the library's fixed scratch array (allocates nothing)."""
+    return load_library().clblasSgemmNoAlloc(int(order), int(transA), int(transB), M, N, K, alpha, _ptr(A), offA, lda,
+                                             _ptr(B), offB, ldb, beta, _ptr(C), offC, ldc, _stream(stream))
 
 
 def dgemm(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc, stream=None):

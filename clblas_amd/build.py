@@ -14,7 +14,7 @@ OBJ_DIR = os.path.join(HERE, "build")
 LIB_PATH = os.path.join(HERE, "libclblas_amd.so")
 CLIENT_PATH = os.path.join(HERE, "client", "clblas_amd-client")
 
-SOURCES = ["api.cpp", "gemm_f32.hip", "gemm_f64.hip", "gemm_c32.hip", "gemm_c64.hip", "level3.hip", "trsm.hip"]
+SOURCES = ["api.cpp", "gemm_f32.hip", "gemm_f64.hip", "gemm_c32.hip", "gemm_c64.hip", "level3.hip", "trsm.hip", "noalloc.hip"]
 
 # -packed-fp32-ops: keep the compiler from forming v_pk_*_f32 out of scalar float code.
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -185,7 +185,7 @@ clblasStatus map_hip_error(hipError_t e) {
 // stop one tile short of 2^31.
 const size_t kMaxDim = 0x7fffffff - 512;
 
-template <typename T>
+template <typename T, bool NOALLOC = false>
 clblasStatus gemm_front(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M,
                         size_t N, size_t K, T alpha, const T *A, size_t offA, size_t lda, const T *B, size_t offB,
                         size_t ldb, T beta, T *C, size_t offC, size_t ldc, hipStream_t stream) {
@@ -216,8 +216,12 @@ clblasStatus gemm_front(clblasOrder order, clblasTranspose transA, clblasTranspo
         std::swap(lda, ldb);
         std::swap(pa, pb);
     }
-    return map_hip_error(cba::launch_gemm<T>(tA, tB, cA, cB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb,
-                                             (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+    if constexpr (NOALLOC)
+        return map_hip_error(cba::sgemm_colmajor_noalloc(tA, tB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb,
+                                                         (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+    else
+        return map_hip_error(cba::launch_gemm<T>(tA, tB, cA, cB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb,
+                                                 (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
 }
 
 template <typename T> struct IsComplex { static const bool value = false; };
@@ -436,6 +440,13 @@ clblasStatus clblasSetup(void) {
     const char want[] = "gfx950";
     for (int i = 0; i < 6; ++i)
         if (arch[i] != want[i]) return clblasInvalidDevice;
+    // Address of this GPU's fixed scratch array, for clblasSgemmNoAlloc (which also looks it up
+    // itself on its first call per device if Setup was not called).
+    void *scratch = nullptr;
+    if (cba::noalloc_scratch(&scratch) != hipSuccess) {
+        (void)hipGetLastError();
+        return clblasOutOfResources;
+    }
     return clblasSuccess;
 }
 
@@ -485,6 +496,14 @@ clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          size_t ldb, float beta, float *C, size_t offC, size_t ldc, hipStream_t stream) {
     return gemm_front<float>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC, ldc,
                              stream);
+}
+
+clblasStatus clblasSgemmNoAlloc(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
+                                size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B,
+                                size_t offB, size_t ldb, float beta, float *C, size_t offC, size_t ldc,
+                                hipStream_t stream) {
+    return gemm_front<float, true>(order, transA, transB, M, N, K, alpha, A, offA, lda, B, offB, ldb, beta, C, offC,
+                                   ldc, stream);
 }
 
 clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,

@@ -93,6 +93,13 @@ struct GemmTri {
 hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float alpha, const float *A, int64_t lda,
                           const float *B, int64_t ldb, float beta, float *C, int64_t ldc, hipStream_t stream,
                           const GemmTri *tri = nullptr, const FixedScratch *fixed = nullptr);
+// SGEMM with the fixed per-GPU scratch array instead of the per-stream buffers (noalloc.hip):
+// allocates nothing; hipErrorOutOfMemory when the call needs more scratch than the array holds.
+hipError_t sgemm_colmajor_noalloc(bool transA, bool transB, int M, int N, int K, float alpha, const float *A,
+                                  int64_t lda, const float *B, int64_t ldb, float beta, float *C, int64_t ldc,
+                                  hipStream_t stream);
+// Device address of the current GPU's fixed scratch array (looked up once per device).
+hipError_t noalloc_scratch(void **ptr);
 hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double alpha, const double *A,
                           int64_t lda, const double *B, int64_t ldb, double beta, double *C, int64_t ldc,
                           hipStream_t stream, const GemmTri *tri = nullptr);

@@ -118,6 +118,23 @@ clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTransp
                          const float *B, size_t offB, size_t ldb, float beta,
                          float *C, size_t offC, size_t ldc, hipStream_t stream);
 
+/* clblasSgemm for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, validation, kernels and results (bit for bit) as clblasSgemm, but
+ * the partial sums of a K split or of a sliced last round of tiles go to a fixed array of
+ * CLBLAS_AMD_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process
+ * ends, instead of to a per-stream buffer allocated on first use: the call allocates nothing.
+ * A call that would need more scratch than that (small C with very deep K: K ranges x N x M
+ * rounded up to 64, x 4 bytes) returns clblasOutOfResources and enqueues nothing; calls that
+ * need no scratch (the large ones) have no size limit.  All calls on one GPU share the array:
+ * calls in order on one stream are safe, calls that overlap in time on one GPU race. */
+#define CLBLAS_AMD_NOALLOC_SCRATCH_BYTES (32u << 20)
+clblasStatus clblasSgemmNoAlloc(clblasOrder order, clblasTranspose transA, clblasTranspose transB,
+                                size_t M, size_t N, size_t K, float alpha,
+                                const float *A, size_t offA, size_t lda,
+                                const float *B, size_t offB, size_t ldb, float beta,
+                                float *C, size_t offC, size_t ldc, hipStream_t stream);
+
 /* Replaces clblasDgemm (src/clBLAS.h:7463-7486, src/library/blas/xgemm.cc:728-783). */
 clblasStatus clblasDgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB,
                          size_t M, size_t N, size_t K, double alpha,
