@@ -78,6 +78,58 @@ def timed_batch(torch, call, reps, warmup, batches=3):
     return best
 
 
+def run_tiles_set(torch, clblas_amd, gen, reps):
+    """The launches that profiles/tiles_counters.md reports on, each `reps` times, in a fixed order:
+    config 1, the four config-3 shapes (NN and TN), a K split, a sliced tail, DTRSM at 8192 and 2048.
+    Prints one JSON line with, per case, the number of kernels the library launched for it, so that a
+    rocprofv3 counter file of the same run can be cut into cases by dispatch order."""
+    cases = []
+
+    def sgemm_case(name, M, N, K, tA, tB, alpha, beta, pad, offs):
+        ra, ca = (K, M) if tA else (M, K)
+        rb, cb = (N, K) if tB else (K, N)
+        lda, ldb, ldc = ra + pad, rb + pad, M + pad
+        A = torch.rand(offs[0] + lda * ca, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+        B = torch.rand(offs[1] + ldb * cb, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+        C = torch.rand(offs[2] + ldc * N, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+        torch.cuda.synchronize()
+        n0 = clblas_amd.last_dispatch()[1]
+        for _ in range(reps):
+            st = clblas_amd.sgemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc)
+            if st != 0:
+                raise RuntimeError("clblasSgemm returned %d" % st)
+        torch.cuda.synchronize()
+        desc, n1 = clblas_amd.last_dispatch()
+        cases.append({"name": name, "calls": reps, "launches": n1 - n0, "flops_per_call": 2.0 * M * N * K,
+                      "bytes_per_call": 4.0 * (M * K + K * N + M * N * (2 if beta != 0 else 1)), "last_gemm": desc})
+
+    sgemm_case("config1 sgemm 1024x1024x1024 NN", 1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0))
+    for (M, N, K) in ((4097, 4095, 1031), (65536, 64, 4096), (64, 65536, 4096), (127, 129, 8192)):
+        for tA, tag in ((NOTRANS, "NN"), (TRANS, "TN")):
+            sgemm_case("config3 sgemm %dx%dx%d %s" % (M, N, K, tag), M, N, K, tA, NOTRANS, 0.7, -1.3, 3, (5, 7, 11))
+    sgemm_case("K split: sgemm 1024x1024x8192 NN", 1024, 1024, 8192, NOTRANS, NOTRANS, 1.0, 1.0, 0, (0, 0, 0))
+    sgemm_case("sliced tail: sgemm 2304x2304x2304 NN", 2304, 2304, 2304, NOTRANS, NOTRANS, 1.0, 1.0, 0, (0, 0, 0))
+    for n in (8192, 2048):
+        A = torch.rand(n * n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1
+        A /= n
+        A.view(n, n).diagonal().copy_(torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) + 1)
+        B0 = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
+        B = B0.clone()
+        torch.cuda.synchronize()
+        n0 = clblas_amd.last_dispatch()[1]
+        for _ in range(reps):
+            B.copy_(B0)
+            st = clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, A, 0, n, B, 0, n)
+            if st != 0:
+                raise RuntimeError("clblasDtrsm returned %d" % st)
+        torch.cuda.synchronize()
+        cases.append({"name": "dtrsm %d left lower notrans nonunit" % n, "calls": reps,
+                      "launches": clblas_amd.last_dispatch()[1] - n0, "flops_per_call": float(n) * (n + 1) * n,
+                      "bytes_per_call": 8.0 * (n * (n + 1) / 2 + 2.0 * n * n)})
+        del A, B, B0
+    print(json.dumps({"metric": "tile set for the counter profile", "reps": reps, "cases": cases}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -85,8 +137,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, vendor or copy (profiling; "
-                    "copy = a plain 1 GiB device copy used to scale the HBM traffic counters)")
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, vendor, tiles or copy "
+                    "(profiling; copy = a plain 1 GiB device copy used to scale the HBM traffic counters; tiles = every tile "
+                    "the five configurations use, --steps times each, for the counter profile)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (one MI355X per box); use --gpus 1")
@@ -105,6 +158,10 @@ def main():
     gen.manual_seed(1234)
     extra = {}
     result = None
+
+    if args.only == "tiles":
+        run_tiles_set(torch, clblas_amd, gen, max(1, min(args.steps, 5)))
+        return
 
     if args.only == "copy":
         src = torch.rand(1 << 28, device="cuda", dtype=torch.float32, generator=gen)  # 1 GiB

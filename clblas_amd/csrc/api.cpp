@@ -46,7 +46,7 @@ void read_knobs() {
     k.group_m = env_int("CLBLAS_AMD_GEMM_GROUP_M", 0);
     k.xcd = env_int("CLBLAS_AMD_GEMM_XCD", 1);
     k.stagger = env_int("CLBLAS_AMD_GEMM_STAGGER", 1);
-    k.fused_reduce = env_int("CLBLAS_AMD_GEMM_FUSED_REDUCE", 1);
+    k.deep_panels = env_int("CLBLAS_AMD_GEMM_DEEP", 1);
     k.log = env_int("CLBLAS_AMD_LOG", 0);
     g_knobs = k;
 }
@@ -460,10 +460,9 @@ size_t clblasAmdLastDispatch(char *text, size_t size) {
         if (r.launches == 0)
             std::snprintf(text, size, "none");
         else
-            std::snprintf(text, size, "%s<%c,%dx%dx%d,%d threads> %c%c M=%d N=%d K=%d grid=(%u,%u) splits=%d%s tail_slices=%d%s",
+            std::snprintf(text, size, "%s<%c,%dx%dx%d,%d threads> %c%c M=%d N=%d K=%d grid=(%u,%u) splits=%d tail_slices=%d%s",
                           r.kernel, r.type, r.bm, r.bn, r.bk, r.threads, r.trans_a ? 'T' : 'N', r.trans_b ? 'T' : 'N',
-                          r.M, r.N, r.K, r.grid_x, r.grid_y, r.splits, r.fused_reduce ? " (summed in the same launch)" : "",
-                          r.tail_slices, r.tri ? " tri" : "");
+                          r.M, r.N, r.K, r.grid_x, r.grid_y, r.splits, r.tail_slices, r.tri ? " tri" : "");
     }
     return (size_t)r.launches;
 }

@@ -20,14 +20,16 @@ namespace cba {
 //      was fitted on the square tiles and picks the oblong ones where they lose (STRMM / SSYMM 3072:
 //      7-9 % slower with them).
 //   4:  64x64x32,  wave 32x32, split-K capable (small / deep-K problems; 1024^3: 94 against 86 with
-//      depth 16, 8192 x 64 x 8192: 106-112 against 91-94)
+//      depth 16, 8192 x 64 x 8192: 106-112 against 91-94); with panels of depth 64 where a workgroup's K
+//      range is at least 1024 (1024^3 95.4 -> 99.0 TFLOP/s, 1024 x 1024 x 2048 109 -> 115, 960 x 960 x 2048
+//      96 -> 101, 512 x 512 x 4096 85 -> 90)
 static const TileEntry<float> *f32_tiles(int *n) {
     static const TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.12),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0),
         make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.97, 0.0),
-        make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true>(0.84, 0.95),
+        make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64>(0.84, 0.95),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

@@ -9,12 +9,14 @@ namespace cba {
 //   1:  64x64x16,  wave 32x32, split-K capable.  Credited with .90 for plain and triangular-C
 //      products (2304^3 64.7 -> 67.9 TFLOP/s, 3328^3 64.5 -> 68.6, 3000 x 1500 x 1000 56.6 -> 61.1 against
 //      .84) and with .84 where an operand is triangular (DTRMM / DSYMM 6144 lose 2-3 % with .90).
+//      With panels of depth 32 where a workgroup's K range is at least 1024 (1024^3 54.9 -> 58.5 TFLOP/s,
+//      1024 x 1024 x 2048 59.8 -> 64.2, 960 x 960 x 2048 50.9 -> 53.4).
 //   Short K on large C goes to the 64x64 tiles through the fixed-time term (k0 = 95 and 68):
 //   4096 x 4096 x 64 31.9 -> 38.9 TFLOP/s, x 128 45.5 -> 52.2, x 256 57.5 -> 61.6, 3000 x 3000 x 640 59.2 -> 64.3.
 static const TileEntry<double> *f64_tiles(int *n) {
     static const TileEntry<double> tab[] = {
         make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 95.0),
-        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true>(0.90, 0.85, 0.84, 68.0),
+        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32>(0.90, 0.85, 0.84, 68.0),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

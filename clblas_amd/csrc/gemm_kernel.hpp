@@ -898,6 +898,44 @@ splitk_reduce_kernel(const T *ws, int64_t ws_ld, int64_t ws_slice, int splits, i
     *c = r;
 }
 
+// The same for many K ranges over a small C (deep K, few tiles), where the pass above is a chain of
+// dependent load batches on too few threads: 8 threads share an element, thread part l fetches ranges
+// l, l + 8, l + 16, ... at once (up to 8 independent loads) and adds them in that order, and the
+// 8 part sums are added in part order.  A fixed order, so the result is reproducible bit for bit;
+// it differs from the order of the pass above only in which roundings happen.
+// Block b covers rows [32 * (b % m_blocks), +32) of column b / m_blocks; thread t: part t / 32, row t % 32.
+template <typename T>
+__global__ void __launch_bounds__(256)
+splitk_reduce_wide_kernel(const T *ws, int64_t ws_ld, int64_t ws_slice, int splits, int M, int N, int m_blocks,
+                          T alpha, T beta, T *C, int64_t ldc) {
+    __shared__ T part_sum[8][33];
+    const int part = threadIdx.x >> 5, row = threadIdx.x & 31;
+    const int m = (blockIdx.x % m_blocks) * 32 + row;
+    const int n = blockIdx.x / m_blocks;
+    T s = T();
+    if (m < M) {
+        const T *w = ws + (int64_t)n * ws_ld + m;
+        T v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (part + 8 * u < splits) v[u] = w[(int64_t)(part + 8 * u) * ws_slice];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (part + 8 * u < splits) s = u == 0 ? v[0] : el_add(s, v[u]);
+    }
+    part_sum[part][row] = s;
+    __syncthreads();
+    if (part == 0 && m < M) {
+        T t = part_sum[0][row];
+        const int parts = splits < 8 ? splits : 8;
+        for (int l = 1; l < parts; ++l) t = el_add(t, part_sum[l][row]);
+        T *c = C + (int64_t)n * ldc + m;
+        T r = el_scale(alpha, t);
+        if (!el_is_zero(beta)) r = el_axpy(beta, *c, r);
+        *c = r;
+    }
+}
+
 // Finishes the tiles whose K range was cut into slices (see GemmParams::tail_*): sums the
 // slices in a fixed order, applies alpha / beta once and honours tri_c.  Block (x, r) covers
 // elements [256 x, 256 x + 256) of sliced tile r (tile-local, column-major, pitch bm).

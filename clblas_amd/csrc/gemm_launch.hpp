@@ -15,6 +15,14 @@ namespace cba {
 
 template <typename T> struct TileEntry {
     int bm, bn, bk, threads;
+    // The same tile with deeper panels (bk_deep; 0: none), for workgroups with a long K range: half
+    // the barriers and loop overhead per flop (FP32 64x64 with depth 64 instead of 32: 1024 x 1024 x 4096
+    // 70.6 -> 66.5 us, 960 x 960 x 2048 38.0 -> 35.8, 1024^3 22.3 -> 21.7), but a first panel twice as
+    // long to fetch before the first MFMA (512^3: 11.4 -> 12.9 us), so only from 1024 deep.
+    int bk_deep;
+    size_t smem_deep[4];
+    void (*plain_deep[4])(const GemmParams<T>);
+    void (*splitk_deep[4])(const GemmParams<T>);
     size_t smem;     // largest of the four variants (for the residency estimate)
     size_t smem_of[4];
     bool has_splitk;
@@ -39,7 +47,7 @@ template <typename T> struct TileEntry {
 };
 
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false, int BK_DEEP = 0>
 TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -1.0, double k0 = 0.0,
                              double tail_extra = 0.05, double eff_tri_c = -1.0) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
@@ -66,6 +74,29 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
         e.splitk[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, true, MINW>;
     } else {
         for (int i = 0; i < 4; ++i) e.splitk[i] = nullptr;
+    }
+    // The same tile with panels of depth BK_DEEP (see TileEntry::bk_deep).
+    if constexpr (BK_DEEP > 0) {
+        e.bk_deep = BK_DEEP;
+        e.smem_deep[0] = GemmCfg<T, BM, BN, BK_DEEP, WM, WN, false, true>::SMEM;
+        e.smem_deep[1] = GemmCfg<T, BM, BN, BK_DEEP, WM, WN, false, false>::SMEM;
+        e.smem_deep[2] = GemmCfg<T, BM, BN, BK_DEEP, WM, WN, true, true>::SMEM;
+        e.smem_deep[3] = GemmCfg<T, BM, BN, BK_DEEP, WM, WN, true, false>::SMEM;
+        e.plain_deep[0] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, false, true, false, MINW>;
+        e.plain_deep[1] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, false, false, false, MINW>;
+        e.plain_deep[2] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, true, true, false, MINW>;
+        e.plain_deep[3] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, true, false, false, MINW>;
+        if constexpr (WITH_SPLITK) {
+            e.splitk_deep[0] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, false, true, true, MINW>;
+            e.splitk_deep[1] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, false, false, true, MINW>;
+            e.splitk_deep[2] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, true, true, true, MINW>;
+            e.splitk_deep[3] = gemm_mfma_kernel<T, BM, BN, BK_DEEP, WM, WN, true, false, true, MINW>;
+        } else {
+            for (int i = 0; i < 4; ++i) e.splitk_deep[i] = nullptr;
+        }
+    } else {
+        e.bk_deep = 0;
+        for (int i = 0; i < 4; ++i) { e.smem_deep[i] = 0; e.plain_deep[i] = nullptr; e.splitk_deep[i] = nullptr; }
     }
     if constexpr (WITH_TRI) {
         e.tri[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, false, MINW, true>;
@@ -95,7 +126,7 @@ static DispatchRecord &note_launch(const char *kernel, int bm, int bn, int bk, i
     r.type = type_letter<T>(); r.kernel = kernel;
     r.bm = bm; r.bn = bn; r.bk = bk; r.threads = threads;
     r.trans_a = tA; r.trans_b = tB; r.M = M; r.N = N; r.K = K;
-    r.splits = 1; r.tail_slices = 1; r.tri = 0; r.fused_reduce = 0;
+    r.splits = 1; r.tail_slices = 1; r.tri = 0;
     r.grid_x = gx; r.grid_y = gy;
     r.launches++;
     return r;
@@ -344,6 +375,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     if (ntiles > 0x7fffffffLL) return hipErrorInvalidValue;
 
     auto fn = e.plain[idx];
+    int bk_used = e.bk;
     if (need_tri) {
         if (!e.tri[idx]) return hipErrorNotSupported;
         fn = e.tri[idx];
@@ -411,19 +443,30 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         const int mode = knobs().stagger;  // 0: never
         p.stagger = mode != 0 && wgs > 512 && !(p.tri_a || p.tri_b) && (!whole_rounds || p.k_per_split <= 2048);
     }
-    const size_t smem = e.smem_of[idx];
+    size_t smem = e.smem_of[idx];
+    const int threads = e.threads;
+    if (e.bk_deep > 0 && !need_tri && p.tail_slices <= 1 && knobs().deep_panels != 0) {
+        // A long K range per workgroup: the variant with deeper panels (K ranges are cut at multiples
+        // of the tile's own depth, so they have to be multiples of the deeper one too).
+        const int krange = splits > 1 ? p.k_per_split : K;
+        if ((krange >= 1024 || knobs().deep_panels > 1) && (splits <= 1 || p.k_per_split % e.bk_deep == 0)) {
+            fn = splits > 1 ? e.splitk_deep[idx] : e.plain_deep[idx];
+            smem = e.smem_deep[idx];
+            bk_used = e.bk_deep;
+        }
+    }
     if (smem > 64 * 1024) {
         hipError_t err = ensure_dynamic_lds((const void *)fn, smem);
         if (err != hipSuccess) return err;
     }
     if (grid_x > kMaxGrid) return hipErrorInvalidValue;
     {
-        DispatchRecord &rec = note_launch<T>("gemm_mfma_kernel", e.bm, e.bn, e.bk, e.threads, tA, tB, M, N, K,
+        DispatchRecord &rec = note_launch<T>("gemm_mfma_kernel", e.bm, e.bn, bk_used, threads, tA, tB, M, N, K,
                                              (unsigned)grid_x, (unsigned)splits);
         rec.splits = splits; rec.tail_slices = p.tail_slices; rec.tri = need_tri ? 1 : 0;
         log_dispatch(rec);
     }
-    hipError_t err = launch_kernel(fn, dim3((unsigned)grid_x, (unsigned)splits), dim3(e.threads), smem, stream, p);
+    hipError_t err = launch_kernel(fn, dim3((unsigned)grid_x, (unsigned)splits), dim3(threads), smem, stream, p);
     if (err != hipSuccess) return err;
     if (p.tail_slices > 1) {
         const int64_t r = ntiles - p.tail_first;
@@ -433,11 +476,20 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         if (err != hipSuccess) return err;
     }
     if (splits > 1) {
-        int mb = (int)ceil_div64(M, 256);
-        if ((int64_t)mb * N > kMaxGrid) return hipErrorInvalidValue;
         dispatch_record().launches++;
-        err = launch_kernel(splitk_reduce_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, p.ws,
-                            p.ws_ld, p.ws_slice, splits, M, N, mb, alpha, beta, C, ldc);
+        // Many ranges over a small C: the pass with eight threads per element (all loads of an element in
+        // flight at once; SGEMM 127 x 129 x 8192 in 37 ranges: 13.7 -> 12.4 us per call); otherwise one
+        // thread per element.
+        if (splits > 8 && splits <= 64 && (int64_t)M * N <= (1 << 20)) {
+            int mb = (int)ceil_div64(M, 32);
+            err = launch_kernel(splitk_reduce_wide_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream,
+                                p.ws, p.ws_ld, p.ws_slice, splits, M, N, mb, alpha, beta, C, ldc);
+        } else {
+            int mb = (int)ceil_div64(M, 256);
+            if ((int64_t)mb * N > kMaxGrid) return hipErrorInvalidValue;
+            err = launch_kernel(splitk_reduce_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, p.ws,
+                                p.ws_ld, p.ws_slice, splits, M, N, mb, alpha, beta, C, ldc);
+        }
     }
     return err;
 }

@@ -39,7 +39,7 @@ template <typename R> struct Cx { R re, im; };
 //   CLBLAS_AMD_LOG=1: one line per kernel launch on stderr.
 struct DebugKnobs {
     int gemm_tile = -1, split_model = 1, splits = 0, tail = 1, group_m = 0, xcd = 1, stagger = 1, log = 0;
-    int fused_reduce = 1;  // CLBLAS_AMD_GEMM_FUSED_REDUCE=0: K ranges are added up by a second launch
+    int deep_panels = 1;   // CLBLAS_AMD_GEMM_DEEP: 0 never the deep-panel variant of a tile, 1 by the rule, 2 wherever built
 };
 const DebugKnobs &knobs();
 void reload_knobs();
@@ -50,7 +50,7 @@ struct DispatchRecord {
     int bm = 0, bn = 0, bk = 0, threads = 0;
     int trans_a = 0, trans_b = 0;
     int M = 0, N = 0, K = 0;
-    int splits = 1, tail_slices = 1, tri = 0, fused_reduce = 0;
+    int splits = 1, tail_slices = 1, tri = 0;
     unsigned grid_x = 0, grid_y = 0;
     unsigned long long launches = 0;  // kernel launches by this thread since the library was loaded
     const char *kernel = "";          // kernel family ("gemm_mfma_kernel", "gemm_wide_ld_kernel", ...)

@@ -79,6 +79,34 @@ def test_integer_exact_all_tiles(gpu, dtype, order, tA, tB):
             np.testing.assert_array_equal(got, want, err_msg="shape %s tile %s" % ((M, N, K), tile))
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("tA,tB", list(itertools.product([NOTRANS, TRANS], [NOTRANS, TRANS])))
+def test_integer_exact_deep_panel_variant(gpu, dtype, tA, tB):
+    """The smallest tile has a second form with panels twice as deep, used where a workgroup's K
+    range is long.  Here it is switched on for every depth (CLBLAS_AMD_GEMM_DEEP=2), with and without a
+    K split, on depths that are and are not multiples of the panel depth."""
+    import clblas_amd
+    small = N_TILES[dtype] - 1
+    shapes = INT_SHAPES + [(200, 150, 1100), (100, 90, 4096), (250, 130, 2050)]
+    for si, (M, N, K) in enumerate(shapes):
+        alpha, beta = 3.0, -2.0
+        la, lc = exact_int_limits(K, alpha, beta, dtype)
+        offs = (5, 7, 11)
+        lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 3, offs)
+        A = oracle.integers(na, 400 + si, la, dtype)
+        B = oracle.integers(nb, 500 + si, la, dtype)
+        C = oracle.integers(nc, 600 + si, lc, dtype)
+        want = C.copy()
+        assert oracle.gemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, want, offs[2], ldc) == 0
+        with gpu.debug_env(CLBLAS_AMD_GEMM_DEEP=2, CLBLAS_AMD_GEMM_TILE=small):
+            st, got = gpu.gemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc)
+            what = clblas_amd.last_dispatch()[0]
+        assert st == 0
+        deep = "64x64x64" if dtype == np.float32 else "64x64x32"
+        assert deep in what or "splits=1 " not in what, what   # a K split whose ranges are not multiples of the depth keeps the plain form
+        np.testing.assert_array_equal(got, want, err_msg="shape %s: %s" % ((M, N, K), what))
+
+
 def _check_sampled(dtype, tA, tB, M, N, K, alpha, beta, A, lda, B, ldb, C0, got, ldc, nsamp=3000, seed=0):
     """Column-major buffers starting at element (0,0).  Checks sampled elements (all four
     borders plus random interior points) against the high-precision oracle."""
