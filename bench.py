@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|vendor]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|tilemodel|vendor|tiles|copy]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
@@ -25,12 +25,35 @@ if ROOT not in sys.path:
 PEAK_FP32_MATRIX = 157.3  # TFLOP/s, MI355X dense MFMA
 PEAK_FP64_MATRIX = 78.6
 
-# HBM-side bytes per launch of the SGEMM 8192^3 kernel, from two rocprofv3 --pmc runs
-# (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a plain 1 GiB
-# device copy (profiles/bench_8192_counters.md: FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).
-# Counters cannot be read from inside this process, so the figure is carried as a constant
-# and only reported when the workload is the one it was measured on.
-SGEMM_8192_TRAFFIC_BYTES = 4.95e9
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_8192_counters.md")
+
+
+def profiled_sgemm_traffic(dispatch):
+    """HBM-side bytes per launch of the SGEMM 8192^3 kernel, read from the tracked rocprofv3 summary
+    (two --pmc runs, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain
+    1 GiB device copy).  Counters cannot be read from inside this process, so the figure is the
+    profile's - and it is only reported when the kernel that ran here (`dispatch`, the library's own
+    description of its last launch) is the kernel the profile measured: same tile, one launch per call.
+    Returns (bytes or None, note)."""
+    import re
+    m = re.search(r"<s,(\d+)x(\d+)x(\d+),", dispatch)
+    if not m or "splits=1 " not in dispatch + " " or "tail_slices=1" not in dispatch:
+        return None, "the launch is not a single plain GEMM kernel"
+    tile = "gemm_mfma_kernel<float, %s, %s, %s," % m.groups()
+    total, seen = 0.0, set()
+    try:
+        for line in open(TRAFFIC_PROFILE):
+            cells = [c.strip() for c in line.split("|")]
+            if len(cells) >= 6 and cells[1] == "sgemm" and cells[3] in ("FETCH_SIZE", "WRITE_SIZE"):
+                if tile not in cells[2]:
+                    return None, "profiles/bench_8192_counters.md was measured on %s, this run used %s" % (cells[2], tile)
+                total += float(cells[5].split()[0]) * 1e9
+                seen.add(cells[3])
+    except OSError as e:
+        return None, "no traffic profile: %s" % e
+    if seen != {"FETCH_SIZE", "WRITE_SIZE"}:
+        return None, "profiles/bench_8192_counters.md has no sgemm FETCH_SIZE / WRITE_SIZE rows"
+    return total, "profiles/bench_8192_counters.md, kernel %s...>" % tile
 
 COL, NOTRANS, TRANS = 1, 0, 1
 LEFT, LOWER, NONUNIT = 0, 1, 1
@@ -76,6 +99,63 @@ def timed_batch(torch, call, reps, warmup, batches=3):
         torch.cuda.synchronize()
         best = min(best, start.elapsed_time(stop) / reps)
     return best
+
+
+TILE_MODEL_SHAPES = (
+    (768, 768, 768), (1000, 1000, 1000), (1280, 1280, 1280), (1500, 1500, 1500), (1792, 1792, 1792), (2000, 2000, 2000),
+    (2304, 2304, 2304), (2560, 2560, 2560), (3000, 3000, 3000), (3328, 3328, 3328), (3584, 3584, 3584), (3700, 3700, 3700),
+    (4097, 4095, 1031), (5000, 1000, 1000), (1800, 2200, 2600), (4200, 1700, 900), (6000, 6000, 640), (4480, 4480, 2000),
+    (3000, 1500, 1000), (1000, 3000, 1500), (5000, 5000, 700), (2500, 7000, 1200), (7000, 2500, 300), (1100, 1000, 520),
+    (640, 520, 6000), (300, 900, 5000), (1024, 1024, 8192), (768, 768, 16384), (3000, 200, 6000), (200, 3000, 6000),
+    (16384, 128, 2048), (128, 16384, 2048), (4096, 4096, 64), (4096, 4096, 256), (8192, 8192, 128), (6144, 6144, 6144),
+    (5120, 5120, 5120), (2048, 2048, 2048), (4096, 4096, 4096), (1536, 1536, 1536),
+)
+
+
+def tile_model_block(torch, clblas_amd, gen):
+    """Default tile choice against every forced tile (debug switch CLBLAS_AMD_GEMM_TILE), SGEMM and DGEMM,
+    column-major NN, alpha = beta = 1.  Per shape: [default TFLOP/s, default tile, best forced TFLOP/s, best
+    tile]; `mispicks` lists the shapes where the default runs more than 3 % behind a different, forced tile."""
+    out = {}
+    for name, dt, fn, ntiles in (("sgemm", torch.float32, clblas_amd.sgemm, 5), ("dgemm", torch.float64, clblas_amd.dgemm, 2)):
+        rows, mispicks, worst = {}, [], 1.0
+        for (M, N, K) in TILE_MODEL_SHAPES:
+            if name == "dgemm" and M * N * K > 6.5e10:
+                continue
+            A = torch.rand(M * K, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            B = torch.rand(K * N, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            C = torch.zeros(M * N, device="cuda", dtype=dt)
+
+            def call():
+                st = fn(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, C, 0, M)
+                if st != 0:
+                    raise RuntimeError("clblas %s returned %d" % (name, st))
+            reps = int(min(40, max(4, 2e11 / (2.0 * M * N * K))))   # a few milliseconds per batch
+            ms_default = timed_batch(torch, call, reps, 2, batches=3)
+            import re
+            default_tile = re.search(r"<\w,(\d+x\d+)x", clblas_amd.last_dispatch()[0]).group(1)
+            best, best_tile, best_dims = None, -1, ""
+            for tile in range(ntiles):
+                os.environ["CLBLAS_AMD_GEMM_TILE"] = str(tile)
+                clblas_amd.reload_debug_env()
+                try:
+                    ms = timed_batch(torch, call, reps, 2, batches=3)
+                    dims = re.search(r"<\w,(\d+x\d+)x", clblas_amd.last_dispatch()[0]).group(1)
+                finally:
+                    os.environ.pop("CLBLAS_AMD_GEMM_TILE", None)
+                    clblas_amd.reload_debug_env()
+                if best is None or ms < best:
+                    best, best_tile, best_dims = ms, tile, dims
+            tf = lambda ms: round(2.0 * M * N * K / ms / 1e9, 1)
+            key = "%dx%dx%d" % (M, N, K)
+            rows[key] = [tf(ms_default), default_tile, tf(best), best_dims]
+            ratio = best / ms_default if best_dims != default_tile else 1.0   # the same tile twice: timing noise
+            worst = min(worst, ratio)
+            if ratio < 0.97:
+                mispicks.append(key)
+            del A, B, C
+        out[name] = {"shapes": rows, "mispicks": mispicks, "worst_default_over_best": round(worst, 3)}
+    return out
 
 
 def run_tiles_set(torch, clblas_amd, gen, reps):
@@ -182,7 +262,24 @@ def main():
             if st != 0:
                 raise RuntimeError("clblasSgemm returned %d" % st)
 
+        v = (torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1)
+        c0v = C.view(n, n).T.double() @ v   # column-major C times v, before the timed calls
+        c0abs_v = C.view(n, n).T.double().abs() @ v.abs()
         wall, ev_ms = timed_calls(torch, sgemm, steps, warmup)
+        dispatch = clblas_amd.last_dispatch()[0]
+        traffic, traffic_note = profiled_sgemm_traffic(dispatch) if n == 8192 else (None, "size is not 8192")
+        # Self-check of the timed result: every call did C <- A B + C, so after `calls` of them
+        # C v = C0 v + calls * A (B v).  Evaluated in double precision on the device.
+        calls = steps + warmup
+        Ad, Bd = A.view(n, n).T.double(), B.view(n, n).T.double()
+        want = c0v + calls * (Ad @ (Bd @ v))
+        got = C.view(n, n).T.double() @ v
+        # Tolerance 8 u calls |C| |v| by elements of C v: far below the worst-case bound
+        # calls (K + 2) u (...), so that a tile computed wrongly would show; the measured ratio is reported.
+        del c0abs_v
+        bound = 8 * calls * 2.0 ** -24 * (C.view(n, n).T.double().abs() @ v.abs())
+        sgemm_check = float(((got - want).abs() / bound).max())
+        del Ad, Bd, want, got, bound
         flops = 2.0 * n * n * n
         ms_per_step = wall * 1e3 / steps
         tflops = flops / (wall / steps) / 1e12
@@ -196,10 +293,13 @@ def main():
                                    "uniform[-1,1)" % n},
             "roofline": {"bound": "mfma", "achieved": round(kernel_tflops, 3), "peak": PEAK_FP32_MATRIX,
                          "unit": "TFLOP/s", "frac": round(kernel_tflops / PEAK_FP32_MATRIX, 4),
-                         "traffic": SGEMM_8192_TRAFFIC_BYTES if n == 8192 else None,
-                         "kernel": "gemm_mfma_kernel<float,256,128,16,...> (one launch per call)",
-                         "launch_ms": round(ev_ms, 4)},
+                         "traffic": traffic, "traffic_source": traffic_note,
+                         "kernel": dispatch, "launch_ms": round(ev_ms, 4)},
         }
+        extra["checked"] = {"sgemm": {"what": "C v = C0 v + calls A (B v) after the timed calls, in double precision",
+                                      "tolerance": "8 u calls |C| |v|", "worst_error_over_tolerance": float("%.3g" % sgemm_check), "ok": sgemm_check <= 1.0}}
+        if sgemm_check > 1.0:
+            raise RuntimeError("SGEMM result fails its linearity check: %.3g of the bound" % sgemm_check)
         extra["sgemm_pct_of_fp32_matrix_peak"] = round(100 * tflops / PEAK_FP32_MATRIX, 2)
         del A, B, C
 
@@ -214,11 +314,28 @@ def main():
             if st != 0:
                 raise RuntimeError("clblasDgemm returned %d" % st)
 
+        v = (torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1)
+        c0v = C.view(n, n).T @ v
+        c0abs_v = C.view(n, n).T.abs() @ v.abs()
         wall, ev_ms = timed_calls(torch, dgemm, steps, warmup)
+        dgemm_dispatch = clblas_amd.last_dispatch()[0]
+        # C <- A B^T + C / 2 every call: C v = C0 v / 2^calls + (2 - 2^(1 - calls)) A (B^T v)
+        calls = steps + warmup
+        Am, Bm = A.view(n, n).T, B.view(n, n).T       # column-major views; B is stored N x K and used transposed
+        want = c0v * 0.5 ** calls + (2 - 2.0 ** (1 - calls)) * (Am @ (Bm.T @ v))
+        got = C.view(n, n).T @ v
+        del c0abs_v
+        bound = 8 * calls * 2.0 ** -53 * (C.view(n, n).T.abs() @ v.abs())
+        dgemm_check = float(((got - want).abs() / bound).max())
+        del want, got, bound
+        if dgemm_check > 1.0:
+            raise RuntimeError("DGEMM result fails its linearity check: %.3g of the bound" % dgemm_check)
+        extra.setdefault("checked", {})["dgemm"] = {"what": "C v = C0 v / 2^calls + (2 - 2^(1-calls)) A (B^T v), in double precision",
+                                                     "tolerance": "8 u calls |C| |v|", "worst_error_over_tolerance": float("%.3g" % dgemm_check), "ok": True}
         d_tflops = 2.0 * n * n * n / (wall / steps) / 1e12
         extra["dgemm"] = {"workload": "BASELINE config 4: DGEMM column-major NT %d^3, alpha=1, beta=0.5, normal(0,1)" % n,
                           "tflops": round(d_tflops, 3), "ms_per_call": round(wall * 1e3 / steps, 4),
-                          "launch_ms": round(ev_ms, 4),
+                          "launch_ms": round(ev_ms, 4), "kernel": dgemm_dispatch,
                           "pct_of_fp64_matrix_peak": round(100 * d_tflops / PEAK_FP64_MATRIX, 2)}
         del A, B, C
     else:
@@ -243,10 +360,25 @@ def main():
                 raise RuntimeError("clblasDtrsm returned %d" % st)
 
         tsteps = max(3, steps // 2)
+        launches_before = clblas_amd.last_dispatch()[1]
         wall, ev_ms = timed_calls(torch, dtrsm, tsteps, 2, before_each=restore)
         t_tflops = float(n) * (n + 1) * n / (ev_ms * 1e-3) / 1e12
+        # Residual of the last timed solve on sampled right-hand sides: ||L X - B|| / (||L|| ||X|| + ||B||)
+        # by columns (inf-norms, double precision on the device) against 2 n eps.
+        cols = torch.randint(0, n, (64,), device="cuda", generator=gen)
+        L = torch.tril(torch.nan_to_num(Av.T))        # Av[c, r] is element (r, c)
+        X, Bs = B.view(n, n).index_select(0, cols).T, B0.view(n, n).index_select(0, cols).T
+        R = L @ X - Bs
+        be = R.abs().amax(dim=0) / (float(L.abs().sum(dim=1).max()) * X.abs().amax(dim=0) + Bs.abs().amax(dim=0))
+        dtrsm_check = float(be.max()) / (2 * n * 2.0 ** -52)
+        del L, X, Bs, R
+        if not (dtrsm_check <= 1.0):
+            raise RuntimeError("DTRSM result fails its residual check: %.3g of the bound" % dtrsm_check)
+        extra.setdefault("checked", {})["dtrsm"] = {"what": "backward error of 64 sampled right-hand sides against 2 n eps",
+                                                     "worst_error_over_bound": float("%.3g" % dtrsm_check), "ok": True}
         extra["dtrsm"] = {"workload": "BASELINE config 5: DTRSM Left/Lower/NoTrans/NonUnit M=N=%d, alpha=1" % n,
                           "tflops": round(t_tflops, 3), "ms_per_call": round(ev_ms, 4),
+                          "kernels_per_call": (clblas_amd.last_dispatch()[1] - launches_before) // (tsteps + 2),
                           "finite": bool(torch.isfinite(B).all().item())}
         if d_tflops:
             extra["dtrsm"]["pct_of_dgemm_rate"] = round(100 * t_tflops / d_tflops, 2)
@@ -402,6 +534,11 @@ def main():
                     "torch_mm_tflops": round(2.0 * M * N * K / vendor_ms / 1e9, 2)}
                 del A, B, C
         extra["small_c_deep_k"] = dk
+
+    # ---- The tile choice against the best forced tile, on shapes that are not whole rounds of any tile:
+    #      tracks how well the cost model in the launcher (choose_tile) fits the kernels as they are now. ----
+    if args.only in ("", "tilemodel"):
+        extra["tile_model"] = tile_model_block(torch, clblas_amd, gen)
 
     # ---- Yardstick: the vendor BLAS that torch calls (rocBLAS / hipBLASLt) on the same box, same sizes.
     #      Not the reference and not a target of the parity tests: it shows what the part gives a

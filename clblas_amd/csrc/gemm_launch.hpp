@@ -20,6 +20,7 @@ template <typename T> struct TileEntry {
     // 70.6 -> 66.5 us, 960 x 960 x 2048 38.0 -> 35.8, 1024^3 22.3 -> 21.7), but a first panel twice as
     // long to fetch before the first MFMA (512^3: 11.4 -> 12.9 us), so only from 1024 deep.
     int bk_deep;
+    double deep_gain;  // factor on `eff` where the deep form runs (plain products, K range from 1024)
     size_t smem_deep[4];
     void (*plain_deep[4])(const GemmParams<T>);
     void (*splitk_deep[4])(const GemmParams<T>);
@@ -78,6 +79,7 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
     // The same tile with panels of depth BK_DEEP (see TileEntry::bk_deep).
     if constexpr (BK_DEEP > 0) {
         e.bk_deep = BK_DEEP;
+        e.deep_gain = 1.05;
         e.smem_deep[0] = GemmCfg<T, BM, BN, BK_DEEP, WM, WN, false, true>::SMEM;
         e.smem_deep[1] = GemmCfg<T, BM, BN, BK_DEEP, WM, WN, false, false>::SMEM;
         e.smem_deep[2] = GemmCfg<T, BM, BN, BK_DEEP, WM, WN, true, true>::SMEM;
@@ -96,6 +98,7 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
         }
     } else {
         e.bk_deep = 0;
+        e.deep_gain = 1.0;
         for (int i = 0; i < 4; ++i) { e.smem_deep[i] = 0; e.plain_deep[i] = nullptr; e.splitk_deep[i] = nullptr; }
     }
     if constexpr (WITH_TRI) {
@@ -231,7 +234,8 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         // alone leave idle, at the price of the pass that adds them up.
         auto split_cost = [&](int i, int64_t t, int s) {
             const double alone = t * s <= kCUs ? tab[i].alone : 1.0;
-            return (double)ceil_div64(t * s, kCUs) * tab[i].bm * tab[i].bn / (s * tab[i].eff * alone) +
+            const double deep = (tab[i].bk_deep > 0 && K / s >= 1024) ? tab[i].deep_gain : 1.0;
+            return (double)ceil_div64(t * s, kCUs) * tab[i].bm * tab[i].bn / (s * tab[i].eff * deep * alone) +
                    split_overhead_cost<T>(M, N, K, s);
         };
         const bool split_model = knobs().split_model != 0 && !need_tri;
@@ -244,13 +248,18 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             const int64_t t = active_tiles(M, N, tab[i].bm, tab[i].bn, tri_c);
             double rounds = (double)ceil_div64(t, kCUs);
             const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
-            if (ts > 1) rounds = (double)(t / kCUs) + 1.0 / ts + tab[i].tail_extra;
+            // A sliced tail round lasts 1 / ts of a round plus what does not shrink with the depth of a slice
+            // (its first loads, the partial tiles written and added up by a second pass): about 120 deep.
+            if (ts > 1) rounds = (double)(t / kCUs) + 1.0 / ts + tab[i].tail_extra + 120.0 / K;
             // A triangular operand makes the tiles differ in depth (half of the full depth on
             // average, started deepest first): the CUs share the total evenly up to a fraction
             // of one full-depth tile, fitted to STRMM / DTRMM 4096 and 8192 (STRMM 4096: 256x128
             // tiles 0.77 ms, 128x128 0.60 ms, 64x64 0.67 ms).
             if (tri_operand) rounds = (double)t / (2.0 * kCUs) + 0.4;
-            const double eff = tri_operand ? tab[i].eff_tri : tri_c ? tab[i].eff_tri_c : tab[i].eff;
+            double eff = tri_operand ? tab[i].eff_tri : tri_c ? tab[i].eff_tri_c : tab[i].eff;
+            // (credited up to three rounds of tiles: beyond that the small tile's memory traffic costs more
+            // than the deeper panels gain - 2000^3 FP32 128 TFLOP/s with 128x64 tiles, 119 with 64x64)
+            if (!need_tri && ts <= 1 && tab[i].bk_deep > 0 && K >= 1024 && t <= 3 * kCUs) eff *= tab[i].deep_gain;
             double cost = rounds * tab[i].bm * tab[i].bn / eff;
             if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             cost *= 1.0 + tab[i].k0 / K;
