@@ -26,36 +26,46 @@ extern "C" {
 /* Same opaque stream type as <hip/hip_runtime_api.h>; repeating the typedef is legal. */
 typedef struct ihipStream_t *hipStream_t;
 
+/* In C++ the enumerations get a fixed underlying type (int, what a C compiler gives them on this
+ * ABI anyway), so that a value outside the enumerators - which a C caller can pass and which the
+ * entry points answer with clblasInvalidValue - is a valid value to read in the C++ implementation
+ * as well. */
+#ifdef __cplusplus
+#define CLBLAS_AMD_ENUM_BASE : int
+#else
+#define CLBLAS_AMD_ENUM_BASE
+#endif
+
 /* Enumerations: numeric values identical to reference src/clBLAS.h:78-113. */
-typedef enum clblasOrder_ {
+typedef enum clblasOrder_ CLBLAS_AMD_ENUM_BASE {
     clblasRowMajor = 0,
     clblasColumnMajor = 1
 } clblasOrder;
 
-typedef enum clblasTranspose_ {
+typedef enum clblasTranspose_ CLBLAS_AMD_ENUM_BASE {
     clblasNoTrans = 0,
     clblasTrans = 1,
     clblasConjTrans = 2 /* same as clblasTrans for real types (xgemm.cc:330-335) */
 } clblasTranspose;
 
-typedef enum clblasUplo_ {
+typedef enum clblasUplo_ CLBLAS_AMD_ENUM_BASE {
     clblasUpper = 0,
     clblasLower = 1
 } clblasUplo;
 
-typedef enum clblasDiag_ {
+typedef enum clblasDiag_ CLBLAS_AMD_ENUM_BASE {
     clblasUnit = 0,
     clblasNonUnit = 1
 } clblasDiag;
 
-typedef enum clblasSide_ {
+typedef enum clblasSide_ CLBLAS_AMD_ENUM_BASE {
     clblasLeft = 0,
     clblasRight = 1
 } clblasSide;
 
 /* Status codes: numeric values identical to reference src/clBLAS.h:123-155
  * (the OpenCL aliases keep the OpenCL numbers they had there). */
-typedef enum clblasStatus_ {
+typedef enum clblasStatus_ CLBLAS_AMD_ENUM_BASE {
     clblasSuccess = 0,
     clblasInvalidValue = -30,         /* CL_INVALID_VALUE: bad enum argument */
     clblasInvalidCommandQueue = -36,  /* CL_INVALID_COMMAND_QUEUE */

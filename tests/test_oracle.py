@@ -304,10 +304,29 @@ def test_generators_are_reproducible():
     assert a.min() >= -1.0 and a.max() < 1.0 and abs(a.mean()) < 0.1
     g = oracle.normal(20000, 9, np.float64)
     assert abs(g.mean()) < 0.05 and abs(g.std() - 1.0) < 0.05
-    # first values are part of the fixture: any change to the generator is caught here
-    np.testing.assert_allclose(oracle.uniform(4, 1, np.float64), oracle.uniform(8, 1, np.float64)[:4])
+    # a prefix of a longer draw is the shorter draw (counter-based generator)
+    np.testing.assert_array_equal(oracle.uniform(4, 1, np.float64), oracle.uniform(8, 1, np.float64)[:4])
     t = oracle.triangular(6, 8, True, 3, np.float64)
     T = t.reshape(6, 8).T[:6, :6]
     assert np.isnan(np.triu(T, 1)[np.triu_indices(6, 1)]).all()
     assert (np.diag(T) >= 1).all() and (np.diag(T) < 2).all()
     assert (np.abs(np.tril(T, -1)) <= 1 / 6).all()
+
+
+def test_generators_match_the_committed_fixtures():
+    """First / last values and a hash of the bytes of every seeded generator, as committed in
+    tests/golden/generator_fixtures.json (written by tests/golden/make_generator_fixtures.py): the
+    inputs of every seeded parity test are pinned to what they were when the tests were written."""
+    import importlib.util
+    import json
+    import os
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    spec = importlib.util.spec_from_file_location("make_generator_fixtures", os.path.join(here, "make_generator_fixtures.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    fixtures = json.load(open(os.path.join(here, "generator_fixtures.json")))
+    assert len(fixtures) == len(mod.CASES)
+    for fx in fixtures:
+        got = mod.describe(mod.generate(fx["generator"], fx["args"]))
+        for key in ("count", "first8", "last8", "sha256"):
+            assert got[key] == fx[key], (fx["generator"], fx["args"], key)
