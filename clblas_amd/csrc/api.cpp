@@ -47,6 +47,7 @@ void read_knobs() {
     k.xcd = env_int("CLBLAS_AMD_GEMM_XCD", 1);
     k.stagger = env_int("CLBLAS_AMD_GEMM_STAGGER", 1);
     k.deep_panels = env_int("CLBLAS_AMD_GEMM_DEEP", 1);
+    k.wide_ld = env_int("CLBLAS_AMD_GEMM_WIDE_LD", 0);
     k.log = env_int("CLBLAS_AMD_LOG", 0);
     g_knobs = k;
 }

@@ -13,7 +13,7 @@ namespace cba {
 static const TileEntry<Cx<float>> *c32_tiles(int *n) {
     static const TileEntry<Cx<float>> tab[] = {
         make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, true, true>(0.93),
-        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true, true>(0.90, 0.85, 0.84),
+        make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true, true, 0, true>(0.90, 0.85, 0.84),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

@@ -17,7 +17,7 @@ namespace cba {
 static const TileEntry<Cx<double>> *c64_tiles(int *n) {
     static const TileEntry<Cx<double>> tab[] = {
         make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, true, true>(0.93, 0.85, -1.0, 44.0),
-        make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true>(0.945, 0.85, 0.86, 35.0, 0.35, 0.86),
+        make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true, 0, true>(0.945, 0.85, 0.86, 35.0, 0.35, 0.86),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

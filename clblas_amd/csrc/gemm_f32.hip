@@ -29,7 +29,7 @@ static const TileEntry<float> *f32_tiles(int *n) {
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.12),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0),
         make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.97, 0.0),
-        make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64>(0.86, 0.95),
+        make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64, true>(0.86, 0.95),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

@@ -16,7 +16,7 @@ namespace cba {
 static const TileEntry<double> *f64_tiles(int *n) {
     static const TileEntry<double> tab[] = {
         make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 95.0),
-        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32>(0.90, 0.85, 0.84, 68.0),
+        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32, true>(0.90, 0.85, 0.84, 68.0),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

@@ -290,7 +290,24 @@ typedef __attribute__((address_space(3))) void lds_void_t;
 //             span of IL*MBLK rows hold the tile rows j*IL + e (IL == 1: identity).
 enum LoadMode { LM_DMA_X = 0, LM_DMA_K = 1 };
 
-template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1> struct PanelLoader {
+// Where a panel is read from: the operand's memory from the panel's first element on.  The plain
+// loaders turn it into one buffer descriptor per panel; the WIDE loaders keep pointer and length
+// and make a descriptor per row.
+struct PanelSrc {
+    __amdgpu_buffer_rsrc_t rsrc;  // the whole remainder from `base` on (what the plain loaders use)
+    const void *base;
+    int64_t bytes_left;
+    __device__ __forceinline__ PanelSrc() : base(nullptr), bytes_left(0) {}
+    __device__ __forceinline__ PanelSrc(const void *b, int64_t n) : rsrc(make_rsrc(b, n)), base(b), bytes_left(n) {}
+};
+
+// WIDE: for leading dimensions so large that the rows of a panel are further apart than the 32-bit
+// offset of a buffer load reaches (2 GiB).  Every row of the panel then gets its own descriptor,
+// based at the row's first element, and the lanes that hold other rows sit the load out; the
+// offsets inside a row stay below the row's length in the panel (at most 1 KiB).  One load
+// instruction per row instead of one per 64 lanes: slower, and only instantiated for the smallest
+// tile of each type, but there is no leading dimension it cannot serve.
+template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1, bool WIDE = false> struct PanelLoader {
     static constexpr int VEC = 16 / (int)sizeof(T);
     static constexpr int NVEC = BX * BK / VEC;
     static constexpr int PER = NVEC / NT;  // 16-byte vectors per thread = wave-wide loads per wave
@@ -329,38 +346,69 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
         return (x / span) * span + (r % MBLK) * IL + r / MBLK;
     }
 
-    uint32_t voff[PER];
+    // Rows (of stride ld) that one wave-wide load covers.
+    static constexpr int ROWS_PER_LOAD = MODE == LM_DMA_X ? (CHUNK / BX > 0 ? CHUNK / BX : 1) : 64 / S;
+    static_assert(!WIDE || MODE != LM_DMA_X || BX <= CHUNK, "WIDE: a row of the [k][x] image must not exceed one load");
+
+    uint32_t voff[PER];  // plain: byte offset of this lane's 16 bytes from the panel's first element; WIDE: from its row's
+    int64_t ld_bytes;    // WIDE only
+    int my_row;          // WIDE only: which of the ROWS_PER_LOAD rows of a load this lane holds
 
     __device__ __forceinline__ void init(int tid, int64_t ld) {
         const int lane = tid & 63, wave = tid >> 6;
+        ld_bytes = ld * (int64_t)sizeof(T);
+        my_row = 0;
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
             if (MODE == LM_DMA_X) {
                 const int e = (wave + i * NW) * CHUNK + lane * VEC;  // element index in the [k][x] image
                 const int k = e / BX, x = e % BX;
-                voff[i] = (uint32_t)(((int64_t)k * ld + x) * (int64_t)sizeof(T));
+                if (WIDE) {
+                    voff[i] = (uint32_t)(x * (int)sizeof(T));
+                    my_row = k - ((wave + i * NW) * CHUNK) / BX;  // the same for every i
+                } else {
+                    voff[i] = (uint32_t)(((int64_t)k * ld + x) * (int64_t)sizeof(T));
+                }
             } else {
                 const int x = (wave + i * NW) * (64 / S) + lane / S;
                 const int slot = (lane % S) ^ swz(x);  // logical slot stored in this lane's place
-                voff[i] = (uint32_t)(((int64_t)perm(x) * ld + slot * VEC) * (int64_t)sizeof(T));
+                if (WIDE) {
+                    voff[i] = (uint32_t)(slot * VEC * (int)sizeof(T));
+                    my_row = lane / S;
+                } else {
+                    voff[i] = (uint32_t)(((int64_t)perm(x) * ld + slot * VEC) * (int64_t)sizeof(T));
+                }
             }
         }
+    }
+
+    // WIDE: row (in units of ld from the panel's first element) that row r of load i of wave `wave_u` holds.
+    static __device__ __forceinline__ int wide_row(int wave_u, int i, int r) {
+        if (MODE == LM_DMA_X) return ((wave_u + i * NW) * CHUNK) / BX + r;
+        return perm((wave_u + i * NW) * (64 / S) + r);
     }
 
     // Starts the transfer of one panel.  base: first element of the panel; bytes_left:
     // footprint bytes from `base` on; lds: this operand's image in the receiving stage.
     __device__ __forceinline__ void issue(const T *base, int64_t bytes_left, T *lds, int wave_u) const {
-        __amdgpu_buffer_rsrc_t r = make_rsrc(base, bytes_left);
+        const PanelSrc src(base, bytes_left);
 #pragma unroll
-        for (int i = 0; i < PER; ++i)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH), 16,
-                                                     (int)voff[i], 0, 0, 0);
+        for (int i = 0; i < PER; ++i) issue_one(src, lds, wave_u, i);
     }
 
-    // One of the PER wave-wide loads of a panel (same arguments as issue()).
-    __device__ __forceinline__ void issue_one(__amdgpu_buffer_rsrc_t r, T *lds, int wave_u, int i) const {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH), 16,
-                                                 (int)voff[i], 0, 0, 0);
+    // One of the PER wave-wide loads of a panel.
+    __device__ __forceinline__ void issue_one(const PanelSrc &src, T *lds, int wave_u, int i) const {
+        lds_void_t *dst = (lds_void_t *)(lds + (wave_u + i * NW) * CHUNK_PITCH);
+        if (!WIDE) {
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src.rsrc, dst, 16, (int)voff[i], 0, 0, 0);
+        } else {
+#pragma nounroll  // (unrolled, the descriptors of all rows are kept live at once and registers spill)
+            for (int r = 0; r < ROWS_PER_LOAD; ++r) {
+                const int64_t off = (int64_t)wide_row(wave_u, i, r) * ld_bytes;
+                __amdgpu_buffer_rsrc_t rs = make_rsrc((const char *)src.base + off, src.bytes_left - off);
+                if (my_row == r) __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, dst, 16, (int)voff[i], 0, 0, 0);
+            }
+        }
     }
 
     // Triangular operand: in the 16 bytes each of this thread's loads delivered, zeroes the
@@ -409,7 +457,7 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
     }
 };
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC> struct GemmCfg {
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, bool WIDE = false> struct GemmCfg {
     typedef Mma<typename Elem<T>::Real> M;
     static constexpr bool CPLX = Elem<T>::CPLX;
     static constexpr int VEC = 16 / (int)sizeof(T);
@@ -428,8 +476,8 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static constexpr int VNM = B_KLAY ? 1 : VN;  // n interleave used by the fragment/epilogue mapping
     static constexpr int NG = KS;                // lane groups along k
     static_assert(BK % (VEC * NG) == 0, "panel depth must hold whole k groups");
-    typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_DMA_K : LM_DMA_X, VM, MB> LoaderA;
-    typedef PanelLoader<T, BN, BK, NT, B_KC ? LM_DMA_K : LM_DMA_X> LoaderB;
+    typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_DMA_K : LM_DMA_X, VM, MB, WIDE> LoaderA;
+    typedef PanelLoader<T, BN, BK, NT, B_KC ? LM_DMA_K : LM_DMA_X, 1, 1, WIDE> LoaderB;
     static constexpr int PITCH_A = LoaderA::LDS_PITCH, PITCH_B = LoaderB::LDS_PITCH;
     static constexpr int A_ELEMS = LoaderA::LDS_ELEMS;
     static constexpr int STAGE = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;  // elements per LDS stage
@@ -440,11 +488,11 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
 };
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, bool SPLITK, int MINW,
-          bool TRI = false>
+          bool TRI = false, bool WIDE = false>
 __global__ void __launch_bounds__((BM / WM) * (BN / WN) * 64, MINW)
 gemm_mfma_kernel(const GemmParams<T> p) {
     static_assert(!(SPLITK && TRI), "triangular variants do not split K");
-    typedef GemmCfg<T, BM, BN, BK, WM, WN, A_KC, B_KC> Cfg;
+    typedef GemmCfg<T, BM, BN, BK, WM, WN, A_KC, B_KC, WIDE> Cfg;
     typedef typename Elem<T>::Real R;
     typedef Mma<R> M;
     constexpr bool CPLX = Cfg::CPLX;
@@ -613,13 +661,13 @@ gemm_mfma_kernel(const GemmParams<T> p) {
             // the MFMAs of the first steps below, where their issue does not hold up this
             // wavefront's MFMAs (8192^3: FP32 144 -> 149 TFLOP/s, FP64 70.5 -> 74; 1024^3 FP32
             // 75 -> 81).  Only the descriptors are made here.
-            __amdgpu_buffer_rsrc_t ra, rb;
+            PanelSrc ra, rb;
             T *dst_next = stage_ptr(kp + 1);
             if (issued) {
                 const int k0n = k_begin + (kp + 1) * BK;
                 const int64_t ao = a_off(k0n), bo = b_off(k0n);
-                ra = make_rsrc(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
-                rb = make_rsrc(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
+                ra = PanelSrc(p.A + ao, p.a_bytes - ao * (int64_t)sizeof(T));
+                rb = PanelSrc(p.B + bo, p.b_bytes - bo * (int64_t)sizeof(T));
             }
             // (Complex FP64, with two long steps per panel, is the exception: 73.8 TFLOP/s at
             // 8192^3 with all loads up front, 72.7 with them behind the first step.)
@@ -976,27 +1024,6 @@ __global__ void __launch_bounds__(256) scale_c_kernel(int M, int N, int m_blocks
     if (m >= M || n >= N) return;
     T *c = C + (int64_t)n * ldc + m;
     *c = el_is_zero(beta) ? T() : el_scale(beta, *c);
-}
-
-// Plain kernel with 64-bit indexing for leading dimensions too large for the 32-bit
-// panel offsets of the MFMA kernel.  Same contract; one thread per C element.
-template <typename T>
-__global__ void __launch_bounds__(256)
-gemm_wide_ld_kernel(int transA, int transB, int conjA, int conjB, int M, int N, int K, int m_blocks, T alpha,
-                    const T *A, int64_t lda, const T *B, int64_t ldb, T beta, T *C, int64_t ldc) {
-    const int64_t m = (int64_t)(blockIdx.x % m_blocks) * 256 + threadIdx.x;
-    const int64_t n = blockIdx.x / m_blocks;
-    if (m >= M || n >= N) return;
-    T s = T();
-    for (int64_t k = 0; k < K; ++k) {
-        T a = transA ? A[k + m * lda] : A[m + k * lda];
-        T b = transB ? B[n + k * ldb] : B[k + n * ldb];
-        s = el_mad(a, conjA != 0, b, conjB != 0, s);
-    }
-    T *c = C + n * ldc + m;
-    T r = el_scale(alpha, s);
-    if (!el_is_zero(beta)) r = el_axpy(beta, *c, r);
-    *c = r;
 }
 
 }  // namespace cba

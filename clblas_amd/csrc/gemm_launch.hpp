@@ -45,10 +45,15 @@ template <typename T> struct TileEntry {
     void (*plain[4])(const GemmParams<T>);
     void (*splitk[4])(const GemmParams<T>);
     void (*tri[4])(const GemmParams<T>);  // variants that honour the triangular fields (or null)
+    // Variants for leading dimensions beyond the reach of a panel-wide buffer descriptor (one descriptor
+    // per row, see PanelLoader); built for the smallest tile of each type only.
+    void (*plain_wide[4])(const GemmParams<T>);
+    void (*splitk_wide[4])(const GemmParams<T>);
+    void (*tri_wide[4])(const GemmParams<T>);
 };
 
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false, int BK_DEEP = 0>
+template <typename T, int BM, int BN, int BK, int WM, int WN, int MINW, bool WITH_SPLITK, bool WITH_TRI = false, int BK_DEEP = 0, bool WITH_WIDE = false>
 TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -1.0, double k0 = 0.0,
                              double tail_extra = 0.05, double eff_tri_c = -1.0) {
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
@@ -75,6 +80,23 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
         e.splitk[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, true, MINW>;
     } else {
         for (int i = 0; i < 4; ++i) e.splitk[i] = nullptr;
+    }
+    if constexpr (WITH_WIDE) {
+        static_assert(WITH_SPLITK && WITH_TRI, "the wide-ld tile serves every kind of launch");
+        e.plain_wide[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, false, MINW, false, true>;
+        e.plain_wide[1] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, false, false, MINW, false, true>;
+        e.plain_wide[2] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, true, false, MINW, false, true>;
+        e.plain_wide[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, false, MINW, false, true>;
+        e.splitk_wide[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, true, MINW, false, true>;
+        e.splitk_wide[1] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, false, true, MINW, false, true>;
+        e.splitk_wide[2] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, true, true, MINW, false, true>;
+        e.splitk_wide[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, true, MINW, false, true>;
+        e.tri_wide[0] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, true, false, MINW, true, true>;
+        e.tri_wide[1] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, false, false, false, MINW, true, true>;
+        e.tri_wide[2] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, true, false, MINW, true, true>;
+        e.tri_wide[3] = gemm_mfma_kernel<T, BM, BN, BK, WM, WN, true, false, false, MINW, true, true>;
+    } else {
+        for (int i = 0; i < 4; ++i) { e.plain_wide[i] = nullptr; e.splitk_wide[i] = nullptr; e.tri_wide[i] = nullptr; }
     }
     // The same tile with panels of depth BK_DEEP (see TileEntry::bk_deep).
     if constexpr (BK_DEEP > 0) {
@@ -204,7 +226,9 @@ static inline int splits_for(int64_t t, int K, int bk) {
     int64_t want = (2 * kCUs) / t;
     const int64_t max_by_k = K / (4 * bk);
     if (want > max_by_k) want = max_by_k;
-    if (want > 64) want = 64;
+    // (up to 512 ranges: a single tile with a depth in the millions still gets a workgroup on every CU;
+    // DGEMM TN 64 x 64 x 2^21 in 64 ranges 6.1 ms, in 512 ranges see the tile comments)
+    if (want > 512) want = 512;
     return want < 1 ? 1 : (int)want;
 }
 
@@ -283,7 +307,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             const int64_t t = active_tiles(M, N, tab[last].bm, tab[last].bn, 0);
             const int s_max = splits_for(t, K, tab[last].bk);
             if (s_max > 1) {
-                static const int kCand[] = {2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 40, 48, 64};
+                static const int kCand[] = {2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 40, 48, 64, 96, 128, 192, 256, 384};
                 last_splits = 1;  // `best` is the cost of one range
                 for (int s : kCand) {
                     if (s >= s_max) break;
@@ -328,23 +352,17 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         return launch_kernel(scale_c_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream, M, N, mb,
                              beta, C, ldc);
     }
-    // 32-bit panel offsets: (tile edge or panel depth) * ld * sizeof(T) must stay < 2^31.
+    // 32-bit panel offsets: (tile edge or panel depth) * ld * sizeof(T) must stay < 2^31.  Beyond
+    // that the smallest tile's wide-ld kernels take over (one buffer descriptor per panel row).
     const int64_t max_edge = 256;
     const int64_t ld_limit = (int64_t)0x7fffffff / (max_edge * (int64_t)sizeof(T)) - 8;
-    if (lda > ld_limit || ldb > ld_limit) {
-        if (need_tri) return hipErrorNotSupported;
-        int mb = (int)ceil_div64(M, 256);
-        if ((int64_t)mb * N > kMaxGrid) return hipErrorInvalidValue;
-        log_dispatch(note_launch<T>("gemm_wide_ld_kernel", 0, 0, 0, 256, tA, tB, M, N, K, (unsigned)((int64_t)mb * N), 1));
-        return launch_kernel(gemm_wide_ld_kernel<T>, dim3((unsigned)((int64_t)mb * N)), dim3(256), 0, stream,
-                             tA ? 1 : 0, tB ? 1 : 0, cA ? 1 : 0, cB ? 1 : 0, M, N, K, mb, alpha, A, lda, B, ldb, beta,
-                             C, ldc);
-    }
+    const bool wide = lda > ld_limit || ldb > ld_limit || knobs().wide_ld != 0;
+    if (wide && !tab[ntab - 1].plain_wide[0]) return hipErrorNotSupported;
 
     int tile, splits;
     // The tail may be sliced unless tiles differ in depth (triangular operands).
     const bool tail_ok = !(need_tri && (tri->tri_a || tri->tri_b)) && knobs().tail != 0;
-    choose_tile(tab, ntab, M, N, K, knobs().gemm_tile, need_tri, need_tri ? tri->tri_c : 0,
+    choose_tile(tab, ntab, M, N, K, wide ? ntab - 1 : knobs().gemm_tile, need_tri, need_tri ? tri->tri_c : 0,
                 need_tri && (tri->tri_a || tri->tri_b), tail_ok, &tile, &splits);
     const TileEntry<T> &e = tab[tile];
 
@@ -383,11 +401,11 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     int64_t ntiles = (int64_t)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return hipErrorInvalidValue;
 
-    auto fn = e.plain[idx];
+    auto fn = wide ? e.plain_wide[idx] : e.plain[idx];
     int bk_used = e.bk;
     if (need_tri) {
         if (!e.tri[idx]) return hipErrorNotSupported;
-        fn = e.tri[idx];
+        fn = wide ? e.tri_wide[idx] : e.tri[idx];
         p.tri_c = tri->tri_c; p.tri_a = tri->tri_a; p.tri_b = tri->tri_b;
         p.unit_a = tri->unit_a; p.unit_b = tri->unit_b;
         p.herm_c = tri->herm_c;
@@ -419,7 +437,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
                 if (we != hipSuccess && (fixed || we != hipErrorOutOfMemory)) return we;
             }
             if (slices > 1 && w) {
-                fn = e.tri[idx];
+                fn = wide ? e.tri_wide[idx] : e.tri[idx];
                 p.tail_first = (int)(ntiles - r);
                 p.tail_slices = slices;
                 p.tail_kps = (int)kps;
@@ -439,7 +457,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             hipError_t we = scratch_for(stream, (size_t)(p.ws_slice * splits) * sizeof(T), fixed, &w);
             if (we != hipSuccess) return we;
             p.ws = (T *)w;
-            fn = e.splitk[idx];
+            fn = wide ? e.splitk_wide[idx] : e.splitk[idx];
         }
     }
     // The late start that keeps the workgroups of a CU out of lockstep (see the kernel).  Needed when
@@ -454,7 +472,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     }
     size_t smem = e.smem_of[idx];
     const int threads = e.threads;
-    if (e.bk_deep > 0 && !need_tri && p.tail_slices <= 1 && knobs().deep_panels != 0) {
+    if (e.bk_deep > 0 && !wide && !need_tri && p.tail_slices <= 1 && knobs().deep_panels != 0) {
         // A long K range per workgroup: the variant with deeper panels (K ranges are cut at multiples
         // of the tile's own depth, so they have to be multiples of the deeper one too).
         const int krange = splits > 1 ? p.k_per_split : K;
@@ -470,7 +488,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     }
     if (grid_x > kMaxGrid) return hipErrorInvalidValue;
     {
-        DispatchRecord &rec = note_launch<T>("gemm_mfma_kernel", e.bm, e.bn, bk_used, threads, tA, tB, M, N, K,
+        DispatchRecord &rec = note_launch<T>(wide ? "gemm_mfma_kernel(wide ld)" : "gemm_mfma_kernel", e.bm, e.bn, bk_used, threads, tA, tB, M, N, K,
                                              (unsigned)grid_x, (unsigned)splits);
         rec.splits = splits; rec.tail_slices = p.tail_slices; rec.tri = need_tri ? 1 : 0;
         log_dispatch(rec);

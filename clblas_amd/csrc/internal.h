@@ -39,6 +39,7 @@ template <typename R> struct Cx { R re, im; };
 //   CLBLAS_AMD_LOG=1: one line per kernel launch on stderr.
 struct DebugKnobs {
     int gemm_tile = -1, split_model = 1, splits = 0, tail = 1, group_m = 0, xcd = 1, stagger = 1, log = 0;
+    int wide_ld = 0;       // CLBLAS_AMD_GEMM_WIDE_LD=1: the wide-ld kernels whatever the leading dimensions (tests)
     int deep_panels = 1;   // CLBLAS_AMD_GEMM_DEEP: 0 never the deep-panel variant of a tile, 1 by the rule, 2 wherever built
 };
 const DebugKnobs &knobs();
@@ -53,7 +54,7 @@ struct DispatchRecord {
     int splits = 1, tail_slices = 1, tri = 0;
     unsigned grid_x = 0, grid_y = 0;
     unsigned long long launches = 0;  // kernel launches by this thread since the library was loaded
-    const char *kernel = "";          // kernel family ("gemm_mfma_kernel", "gemm_wide_ld_kernel", ...)
+    const char *kernel = "";          // kernel family ("gemm_mfma_kernel", "gemm_mfma_kernel(wide ld)", "scale_c_kernel")
 };
 DispatchRecord &dispatch_record();  // thread-local
 

@@ -54,9 +54,55 @@ copy_matrix_kernel(int M, int N, int m_blocks, const T *src, int64_t lds_, T *ds
     if (m < M && n < N) dst[(int64_t)n * ldd + m] = src[(int64_t)n * lds_ + m];
 }
 
+// C(m, n) <- alpha W(m, n) + beta C(m, n) on the lower / upper triangle of the N x N matrix C; beta == 0
+// does not read C; herm: the diagonal of C is read without and stored with a zero imaginary part.
+// Block b covers rows [256 * (b % m_blocks), +256) of column b / m_blocks.
+template <typename T>
+__global__ void __launch_bounds__(256)
+triangle_axpy_kernel(int N, int m_blocks, bool lower, bool herm, T alpha, const T *W, int64_t ldw, T beta, T *C,
+                     int64_t ldc) {
+    const int m = (blockIdx.x % m_blocks) * 256 + threadIdx.x;
+    const int n = blockIdx.x / m_blocks;
+    if (m >= N || n >= N || (lower ? m < n : m > n)) return;
+    T *c = C + (int64_t)n * ldc + m;
+    T r = el_scale(alpha, W[(int64_t)n * ldw + m]);
+    const bool diag = herm && m == n;
+    if (!el_is_zero(beta)) r = el_axpy(beta, diag ? el_real_only(*c) : *c, r);
+    if (diag) r = el_real_only(r);
+    *c = r;
+}
+
+// A rank-k update of a small C with a deep K.  The kernels that store one triangle of C do not cut K
+// into ranges, so a handful of tiles would walk through all of K on a handful of CUs (DSYRK 64 x 2^21:
+// one workgroup, 0.4 s).  Such a product runs as a plain GEMM - both triangles, twice the flops, but
+// with a K split over every CU - into a library-owned N x N buffer, and a small pass folds the wanted
+// triangle into C.  Used while the full square has at most 128 tiles of 64 x 64 (N <= 704) and K >= 4096.
+static inline bool rank_k_is_deep(int N, int K) {
+    const int64_t n64 = (N + 63) / 64;
+    return n64 * n64 <= 128 && K >= 4096;
+}
+template <typename T>
+static hipError_t rank_k_deep(bool lower, bool herm, bool tA, bool tB, bool cA, bool cB, int N, int K, T alpha,
+                              const T *A, int64_t lda, const T *B, int64_t ldb, T beta, T *C, int64_t ldc,
+                              hipStream_t stream) {
+    const int64_t ldw = ((int64_t)N + 63) / 64 * 64;
+    void *wv = nullptr;
+    hipError_t err = workspace_get(stream, (size_t)ldw * N * sizeof(T), 1, &wv);
+    if (err != hipSuccess) return err;
+    T *W = (T *)wv;
+    err = launch_gemm<T>(tA, tB, cA, cB, N, N, K, el_one<T>(), A, lda, B, ldb, T(), W, ldw, stream);
+    if (err != hipSuccess) return err;
+    const int mb = (N + 255) / 256;
+    dispatch_record().launches++;
+    return launch_kernel(triangle_axpy_kernel<T>, dim3((unsigned)(mb * N)), dim3(256), 0, stream, N, mb, lower, herm,
+                         alpha, (const T *)W, ldw, beta, C, ldc);
+}
+
 template <typename T>
 hipError_t syrk_colmajor(bool lower, bool trans, int N, int K, T alpha, const T *A, int64_t lda, T beta, T *C,
                          int64_t ldc, hipStream_t stream) {
+    if (rank_k_is_deep(N, K))
+        return rank_k_deep<T>(lower, false, trans, !trans, false, false, N, K, alpha, A, lda, A, lda, beta, C, ldc, stream);
     GemmTri tri;
     tri.tri_c = lower ? 1 : 2;
     // op(A) op(A)^T: the second operand is the same matrix with the opposite transpose flag.
@@ -120,6 +166,11 @@ hipError_t symm_colmajor(bool right, bool lower, int M, int N, T alpha, const T 
 template <typename T>
 hipError_t syr2k_colmajor(bool lower, bool trans, int N, int K, T alpha, const T *A, int64_t lda, const T *B,
                           int64_t ldb, T beta, T *C, int64_t ldc, hipStream_t stream) {
+    if (rank_k_is_deep(N, K)) {
+        hipError_t e = rank_k_deep<T>(lower, false, trans, !trans, false, false, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream);
+        if (e != hipSuccess) return e;
+        return rank_k_deep<T>(lower, false, trans, !trans, false, false, N, K, alpha, B, ldb, A, lda, el_one<T>(), C, ldc, stream);
+    }
     GemmTri tri;
     tri.tri_c = lower ? 1 : 2;
     // C <- alpha op(A) op(B)^T + beta C, then C <- alpha op(B) op(A)^T + C
@@ -134,6 +185,9 @@ template <typename R>
 hipError_t herk_colmajor(bool lower, bool ctrans, int N, int K, R alpha, const Cx<R> *A, int64_t lda, R beta,
                          Cx<R> *C, int64_t ldc, hipStream_t stream) {
     typedef Cx<R> T;
+    if (rank_k_is_deep(N, K))
+        return rank_k_deep<T>(lower, true, ctrans, !ctrans, ctrans, !ctrans, N, K, T{alpha, (R)0}, A, lda, A, lda,
+                              T{beta, (R)0}, C, ldc, stream);
     GemmTri tri;
     tri.tri_c = lower ? 1 : 2;
     tri.herm_c = 1;
@@ -146,6 +200,13 @@ template <typename R>
 hipError_t her2k_colmajor(bool lower, bool ctrans, int N, int K, Cx<R> alpha, const Cx<R> *A, int64_t lda,
                           const Cx<R> *B, int64_t ldb, R beta, Cx<R> *C, int64_t ldc, hipStream_t stream) {
     typedef Cx<R> T;
+    if (rank_k_is_deep(N, K)) {
+        hipError_t e = rank_k_deep<T>(lower, true, ctrans, !ctrans, ctrans, !ctrans, N, K, alpha, A, lda, B, ldb,
+                                      T{beta, (R)0}, C, ldc, stream);
+        if (e != hipSuccess) return e;
+        return rank_k_deep<T>(lower, true, ctrans, !ctrans, ctrans, !ctrans, N, K, T{alpha.re, -alpha.im}, B, ldb, A, lda,
+                              el_one<T>(), C, ldc, stream);
+    }
     GemmTri tri;
     tri.tri_c = lower ? 1 : 2;
     tri.herm_c = 1;

@@ -56,6 +56,26 @@ def test_syrk_integer_exact_all_tiles(gpu, dtype, order, uplo, trans):
 
 
 @pytest.mark.parametrize("dtype", ALL)
+@pytest.mark.parametrize("order,uplo,trans", list(itertools.product([ROW, COL], [UPPER, LOWER], [NOTRANS, TRANS])))
+def test_syrk_small_c_deep_k_integer_exact(gpu, dtype, order, uplo, trans):
+    """A small C from operands thousands deep runs as a plain product with a K split into a scratch
+    square and a pass that folds the wanted triangle into C: the other triangle of C (NaN here) and
+    everything around it stay untouched."""
+    alpha, beta = scalars(dtype)
+    for si, (N, K) in enumerate([(64, 5000), (300, 4100), (704, 4096)] if not is_cplx(dtype) else [(64, 5000), (200, 4100)]):
+        rows, cols = (N, K) if trans == NOTRANS else (K, N)
+        A, lda = matrix(order, rows, cols, 5, 3, 60 + si, dtype, True, limit=4)
+        C, ldc = matrix(order, N, N, 7, 2, 70 + si, dtype, True)
+        keep = tri_mask(N, uplo == LOWER)
+        logical_view(C, order, NOTRANS, N, N, 7, ldc)[~keep] = nan_of(dtype)
+        want = C.copy()
+        assert oracle.syrk(order, uplo, trans, N, K, alpha, A, 5, lda, beta, want, 7, ldc) == 0
+        st, got = gpu.syrk(order, uplo, trans, N, K, alpha, A, 5, lda, beta, C, 7, ldc)
+        assert st == 0
+        np.testing.assert_array_equal(got.view(np.uint8), want.view(np.uint8), err_msg="N=%d K=%d" % (N, K))
+
+
+@pytest.mark.parametrize("dtype", ALL)
 def test_syrk_uniform_data(gpu, dtype):
     alpha, beta = real_scalars(dtype)
     for uplo, trans, (N, K) in [(LOWER, NOTRANS, (700, 513)), (UPPER, TRANS, (1031, 300)), (LOWER, TRANS, (129, 2048))]:

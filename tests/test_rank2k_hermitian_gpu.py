@@ -107,10 +107,12 @@ def test_hemm_integer_exact_all_tiles(gpu, dtype, order, side, uplo):
 
 @pytest.mark.parametrize("kind,dtype,order,uplo,trans", rank2k_variants())
 def test_rank2k_long_thin_integer_exact(gpu, kind, dtype, order, uplo, trans):
-    """Rank-1 / rank-3 updates of a triangle of a few thousand rows, and a 1 x 1 result from
-    operands 3000 deep: exact-integer data, default tile choice."""
+    """Rank-1 / rank-3 updates of a triangle of a few thousand rows, a 1 x 1 result from
+    operands 3000 deep, and small results from operands thousands deep (those run as a plain
+    product with a K split into a scratch square, folded into the triangle by a second pass):
+    exact-integer data, default tile choice."""
     alpha, beta = rank2k_scalars(kind, dtype, True)
-    for si, (N, K) in enumerate([(3000, 1), (1, 3000), (2049, 3)]):
+    for si, (N, K) in enumerate([(3000, 1), (1, 3000), (2049, 3), (64, 5000), (300, 4100)]):
         A, lda, B, ldb, C, ldc, keep = rank2k_case(kind, dtype, order, uplo, trans, N, K, 210 + 3 * si, True)
         want = C.copy()
         assert call_rank2k(oracle, kind, order, uplo, trans, N, K, alpha, A, 5, lda, B, 3, ldb, beta, want, 7, ldc) == 0
