@@ -5,7 +5,7 @@
 // for STRSM, the legacy block solver (src/library/blas/gens/trsm.c:1213-1456).  The
 // reference inverts every 128x128 diagonal block (trtri kernels) and then alternates
 // "X_i = inv(A_ii) B_i" with a trailing DGEMM update, using an M x N temporary.  Here the
-// diagonal blocks (256 x 256) are solved inside one kernel by block substitution over their
+// diagonal blocks (512 x 512, 256 x 256 for complex types) are solved inside one kernel by block substitution over their
 // 16 x 16 sub-blocks on the MFMA units (only the 16 x 16 diagonal sub-triangles are inverted,
 // by substitution, in a packing pass), the sweep is recursive so that almost all flops land
 // in large-K GEMM updates, and B is solved in place without a temporary.
@@ -54,38 +54,44 @@ template <> struct Mma16<float> {
 // nb-1-P) so that equation P only involves unknowns Q <= P.  coef(P,Q) is the factor of
 // unknown Q in equation P:   left: op(A)(iP, iQ)   right: op(A)(iQ, iP),
 // so with teff = trans XOR right it is A[iP + iQ*lda] (teff false) or A[iQ + iP*lda].
-// In that order every diagonal block is lower triangular, L = (L_ws), 16 x 16 sub-blocks of
-// 16 x 16, and the solve is the block substitution
-//     X_s = inv(L_ss) Y_s ;   Y_w -= L_ws X_s  (w > s)        s = 0..15.
+// In that order every diagonal block is lower triangular, L = (L_ws), NBLK x NBLK sub-blocks of
+// 16 x 16 (NBLK = 32 for real types, 16 for complex ones), and the solve is the block substitution
+//     X_s = inv(L_ss) Y_s ;   Y_w -= L_ws X_s  (w > s)        s = 0..NBLK-1.
 // A packing pass (trsm_pack_kernel, once per call, all diagonal blocks at once) reads the
-// referenced triangle of A - never the other one, nor a unit diagonal - inverts the sixteen
-// small triangles L_ss by substitution and writes, per diagonal block, the 136 sub-blocks
+// referenced triangle of A - never the other one, nor a unit diagonal - inverts the
+// small triangles L_ss by substitution and writes, per diagonal block, the NBLK (NBLK+1)/2 sub-blocks
 // inv(L_ss) and -L_ws in the order the MFMA "A" operand wants them: entry [lane][c] is
 // element (p = lane%16, q = krow(lane/16, c)), so a lane fetches its four values of a
 // sub-block with one or two 16-byte loads and nothing is broadcast.  Row w's sub-blocks
 // (w,0..w) are consecutive, so each wavefront streams its own row straight from memory
-// (L2), two steps ahead of their use.
+// (L2), one to three sub-blocks ahead of their use.
 // (The reference inverts whole 128 x 128 blocks, trtri/*.cpp; inverting only the 16 x 16
 // ones keeps the result much closer to plain substitution.)
 //
 // Leaf kernel: one workgroup = one diagonal block x CW = 16 or 32 right-hand sides, 16
-// wavefronts; wavefront w owns equations [16w, 16w+16) as CW/16 accumulator blocks of 16 x 16
-// (lane l: right-hand side l%16 of each block, equations krow(l/16, v)).  Accumulator layout and
-// MFMA "B" operand layout coincide, so Y_s feeds the MFMAs as it is and X_s goes to the
-// other wavefronts through LDS in the same per-lane order.  Step s: wavefronts w > s subtract
-// L_ws X_s (4 MFMAs per block); wavefront s+1 then computes X_(s+1) (4 per block) and publishes it
-// while the others are still updating; one barrier per step.
+// wavefronts; wavefront w owns sub-block rows w (and w+16), each as CW/16 accumulator blocks of
+// 16 x 16 (lane l: right-hand side l%16 of each block, equations krow(l/16, v)).  Accumulator layout
+// and MFMA "B" operand layout coincide, so Y_s feeds the MFMAs as it is and X_s goes to the
+// other wavefronts through LDS in the same per-lane order.  A row subtracts L_ws X_s (4 MFMAs per
+// block) for every s below it as the X_s appear, then computes X_w (4 per block) and publishes
+// it; the wavefronts are synchronised by one flag per X_s in LDS, not by barriers.
 // For side=left a right-hand side is a column of B; the panel moves between HBM and the
 // accumulator layout through an LDS staging area so that global accesses run along columns.
 template <typename T, bool RIGHT = false> struct TrsmLeaf {
     typedef typename Elem<T>::Real R;
     static constexpr bool CPLX = Elem<T>::CPLX;
-    static constexpr int NB = 256, IB = 16, NBLK = NB / IB, THREADS = 64 * NBLK;
-    // Right-hand sides per workgroup.  16: two workgroups fit a CU and cover each other's
-    // serial solves (DTRSM left 2048: 0.36 -> 0.31 ms, 4096: 1.36 -> 1.28 ms, 8192 x 512: 1.52 ->
-    // 1.34 ms).  Side = right with real elements keeps 32: its right-hand sides are rows of B,
-    // and 16 of them are too short a run of memory (8192: 0.5 - 1.5 % slower with 16).
-    static constexpr int CW = (RIGHT && !CPLX) ? 32 : 16, NBK = CW / 16;
+    // Row blocks per wavefront.  Real types: two, i.e. a leaf of 512 equations.  The updates of
+    // the second row block fill the MFMA pipes while the serial chain of the first 256 equations
+    // runs, and the 256-row GEMM update between two leaves of 256 (a launch of its own, short of
+    // work: 17 us against 14 us for a leaf at 2048 right-hand sides) is gone.  Complex types keep
+    // one row block (their packed sub-blocks are three times the size; LDS and registers).
+    static constexpr int WAVES = 16, RW = CPLX ? 1 : 2;
+    static constexpr int IB = 16, NB = WAVES * IB * RW, NBLK = NB / IB, THREADS = 64 * WAVES;
+    // Right-hand sides per workgroup.  16 gives a launch twice the workgroups (DTRSM left 2048:
+    // 0.36 -> 0.31 ms, 4096: 1.36 -> 1.28 ms, 8192 x 512: 1.52 -> 1.34 ms when it was introduced).
+    // Side = right in FP32 keeps 32: its right-hand sides are rows of B, and 16 of them are too
+    // short a run of memory; in FP64 two column blocks times two row blocks do not fit the registers.
+    static constexpr int CW = (RIGHT && !CPLX && sizeof(R) == 4) ? 32 : 16, NBK = CW / 16;
     static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;  // sub-blocks (bi,bj), bi >= bj, at bi*(bi+1)/2 + bj
     // Packed sub-block: PLANES x 64 lanes x 4 reals.  Real: the values.  Complex: real parts,
     // imaginary parts, negated imaginary parts (so that no sign has to be flipped in the solve).
@@ -93,10 +99,16 @@ template <typename T, bool RIGHT = false> struct TrsmLeaf {
     static constexpr int SUB_REALS = PLANES * IB * IB;
     static constexpr int PACK_REALS = N_EBLK * SUB_REALS;  // per diagonal block
     static constexpr int NP = CPLX ? 2 : 1;                // accumulators per block (re, im)
-    static constexpr int X_REALS = 2 * NP * NBK * 64 * 4;  // two buffers of X_s in per-lane order
+    static constexpr int XS_REALS = NP * NBK * 64 * 4;     // one X_s in per-lane order
+    static constexpr int X_REALS = NBLK * XS_REALS;        // every X_s keeps a slot of its own
     static constexpr int SP = NB + 2;                      // pitch of the right-hand-side staging area
-    static constexpr int S_ELEMS = CW * SP;
-    static constexpr size_t SMEM = (size_t)X_REALS * sizeof(R) + (size_t)S_ELEMS * sizeof(T);
+    static constexpr int S_ELEMS = RIGHT ? 0 : CW * SP;    // side = right moves its rows directly
+    // The staging area is only used before the first and after the last step, so it shares its
+    // memory with the X slots; one "published" flag per step follows.
+    static constexpr size_t X_BYTES = (size_t)X_REALS * sizeof(R), S_BYTES = (size_t)S_ELEMS * sizeof(T);
+    static constexpr size_t FLAGS_AT = ((X_BYTES > S_BYTES ? X_BYTES : S_BYTES) + 15) / 16 * 16;
+    static constexpr size_t SMEM = FLAGS_AT + NBLK * sizeof(int);
+    static constexpr int PACK_CHUNK = 8;                   // sub-blocks per workgroup of the packing pass
 };
 
 // Element helpers for the packing pass (real and complex).
@@ -126,8 +138,9 @@ template <typename R> static __device__ __forceinline__ void tr_put(R *sub, int 
     sub[512 + w] = -v.im;
 }
 
-// Packs all diagonal blocks of the n x n triangle (see above).  Workgroup (bi, b) of 256
-// threads packs sub-block row bi of diagonal block b (rows/columns [256 b, 256 b + nb)).
+// Packs all diagonal blocks of the n x n triangle (see above).  Workgroup (bi, chunk, b) of 256
+// threads packs up to PACK_CHUNK sub-blocks of sub-block row bi of diagonal block b (rows/columns
+// [NB b, NB b + nb)).
 // `conj` conjugates the coefficients (complex, clblasConjTrans).
 template <typename T, bool FORWARD>
 __global__ void __launch_bounds__(256)
@@ -138,8 +151,10 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
     typedef Mma16<R> M;
     constexpr int IB = L::IB;
     __shared__ T Ld[IB][IB + 1];  // the diagonal sub-triangle, then its inverse
+    constexpr int CHUNKS = L::NBLK / L::PACK_CHUNK;
     const int tid = threadIdx.x;
-    const int bi = blockIdx.x;
+    const int bi = blockIdx.x / CHUNKS, chunk = blockIdx.x % CHUNKS;
+    if (chunk > bi / L::PACK_CHUNK) return;  // nothing of row bi lies in this chunk
     const int i0 = blockIdx.y * L::NB;
     const int nb = n - i0 < L::NB ? n - i0 : L::NB;
     const T *Ablk = A + i0 + (int64_t)i0 * lda;
@@ -148,14 +163,17 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
         const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
         return tr_conj_if(teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda], conj);
     };
-    // off-diagonal sub-blocks (bi, 0..bi-1), negated; rows past nb are zero
-    for (int e = tid; e < bi * IB * IB; e += 256) {
+    // off-diagonal sub-blocks (bi, bj) of this chunk, bj < bi, negated; rows past nb are zero
+    const int bj_lo = chunk * L::PACK_CHUNK;
+    const int bj_hi = bj_lo + L::PACK_CHUNK < bi ? bj_lo + L::PACK_CHUNK : bi;
+    for (int e = bj_lo * IB * IB + tid; e < bj_hi * IB * IB; e += 256) {
         const int bj = e / (IB * IB), w = e % (IB * IB);
         const int lane = w / 4, c = w % 4;
         const int P = bi * IB + lane % 16, Q = bj * IB + M::krow(lane / 16, c);
         // Q < P always holds here; Q < nb follows from P < nb
         tr_put(out + bj * L::SUB_REALS, w, (P < nb) ? tr_sub(T(), coef(P, Q)) : T());
     }
+    if (chunk != bi / L::PACK_CHUNK) return;  // the chunk that holds column bi also inverts (bi, bi)
     // diagonal sub-triangle into LDS (identity where the block is short)
     {
         const int p = tid / IB, q = tid % IB;
@@ -195,6 +213,8 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
     }
 }
 
+template <int N> struct IntC { static constexpr int value = N; };
+
 template <typename T, bool RIGHT, bool FORWARD>
 __global__ void __launch_bounds__(TrsmLeaf<T>::THREADS)
 trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk,
@@ -205,12 +225,14 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     typedef typename M::Acc Acc;
     constexpr bool CPLX = L::CPLX;
     constexpr int IB = L::IB, CW = L::CW, NBK = L::NBK, NT = L::THREADS, NBLK = L::NBLK, NP = L::NP;
-    constexpr int PLANES = L::PLANES;
+    constexpr int PLANES = L::PLANES, RW = L::RW, WAVES = L::WAVES;
     constexpr int V = 16 / (int)sizeof(R);  // reals per 16 bytes
+    constexpr int CH = 4 / V;               // 16-byte pieces of an accumulator block
     typedef R VT __attribute__((ext_vector_type(V)));
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     R *X = reinterpret_cast<R *>(smem_raw);
-    T *S = reinterpret_cast<T *>(X + L::X_REALS);
+    T *S = reinterpret_cast<T *>(smem_raw);  // shares its memory with X: used before and after the steps only
+    int *published = reinterpret_cast<int *>(smem_raw + L::FLAGS_AT);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -218,13 +240,20 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     const int g = lane >> 4, jj = lane & 15;
     const int64_t j0 = (int64_t)blockIdx.x * CW;
     const int nsteps = (nb + IB - 1) / IB;  // sub-block rows that exist
+    if (tid < NBLK) published[tid] = 0;
 
-    // A lane's values of sub-block (wave, s): MFMA "A" operand, plane pl, chunk c = element c.
-    const R *erow = packed + (int64_t)(wave * (wave + 1) / 2) * L::SUB_REALS + lane * 4;
-    auto load_e = [&](int s, R (&a)[PLANES][4]) {
+    // This wavefront owns the sub-block rows wave + WAVES*h, h < RW.
+    // A lane's values of sub-block (row, s): MFMA "A" operand, plane pl, chunk c = element c.
+    const R *erow[RW];
+#pragma unroll
+    for (int h = 0; h < RW; ++h) {
+        const int row = wave + WAVES * h;
+        erow[h] = packed + (int64_t)(row * (row + 1) / 2) * L::SUB_REALS + lane * 4;
+    }
+    auto load_e = [&](int h, int s, R (&a)[PLANES][4]) {
 #pragma unroll
         for (int pl = 0; pl < PLANES; ++pl) {
-            const R *src = erow + s * L::SUB_REALS + pl * (IB * IB);
+            const R *src = erow[h] + s * L::SUB_REALS + pl * (IB * IB);
 #pragma unroll
             for (int c = 0; c < 4; c += V) {
                 VT t = *reinterpret_cast<const VT *>(src + c);
@@ -233,36 +262,74 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
             }
         }
     };
-    constexpr int RING = CPLX ? 2 : 3;  // sub-blocks in flight: this step's and the next one or two
+    // A wavefront finishes its first row block before it starts on its second, so one ring of
+    // sub-blocks in flight serves both, one after the other.
+    constexpr int RING = CPLX ? 2 : 4;  // sub-blocks in flight: the current one and the next one to three
     R ea[RING][PLANES][4];
-#pragma unroll
-    for (int s = 0; s < RING - 1; ++s)
-        if (s <= wave && wave < nsteps) load_e(s, ea[s]);
-
-    // ---- right-hand sides into the accumulator layout: y[.][k][v] = alpha * b(equation krow(g,v)
-    //      of this wavefront, right-hand side j0 + 16k + jj); complex: [0] real, [1] imaginary ----
-    Acc y[NP][NBK];
-    auto put_y = [&](int k, int v, T b) {
-        const T ab = el_scale(alpha, b);
-        if constexpr (CPLX) { y[0][k][v] = ab.re; y[1][k][v] = ab.im; } else { y[0][k][v] = ab; }
+    // Every wavefront requests the same number of sub-blocks at the same places of the program, needed
+    // or not (a row's own diagonal sub-block again once it is past it): with requests under
+    // conditions the compiler can only wait for ALL outstanding loads before each use, which puts a
+    // full memory latency into every step.
+    auto prefetch = [&](int h, int s) {
+        const int row = wave + WAVES * h;
+        load_e(h, s < row ? s : row, ea[s % RING]);
     };
-    auto get_y = [&](int k, int v) -> T {
-        if constexpr (CPLX) return T{y[0][k][v], y[1][k][v]};
-        else return y[0][k][v];
+    // Real types keep each row's own diagonal sub-block (its inverse) in registers of its own, requested
+    // first of all, so that a solve never waits for memory; the complex kernels have no registers
+    // to spare for that and take it from the ring.
+    constexpr bool DIAG_REGS = !CPLX;
+    R ed[DIAG_REGS ? RW : 1][PLANES][4];
+    if constexpr (DIAG_REGS) {
+#pragma unroll
+        for (int h = 0; h < RW; ++h) load_e(h, wave + WAVES * h, ed[h]);
+    }
+#pragma unroll
+    for (int s = 0; s < RING - 1; ++s) prefetch(0, s);
+    constexpr int LOADS_PER_SUB = PLANES * (4 / V);  // load instructions per sub-block and lane
+    // Waits until at most n of this wavefront's global loads are outstanding (they return in order).
+    auto wait_loads = [&](int n) {
+        switch (n) {  // (n is known at compile time where this is used)
+            case 0: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0)); break;
+            case 1: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(1)); break;
+            case 2: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(2)); break;
+            case 3: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(3)); break;
+            case 4: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(4)); break;
+            case 5: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(5)); break;
+            case 6: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(6)); break;
+            default: __builtin_amdgcn_s_waitcnt(CBA_VMCNT_ONLY(0)); break;
+        }
+    };
+
+    // ---- right-hand sides into the accumulator layout: y[h][.][k][v] = alpha * b(equation
+    //      krow(g,v) of row block h of this wavefront, right-hand side j0 + 16k + jj); complex: [0]
+    //      real, [1] imaginary ----
+    Acc y[RW][NP][NBK];
+    auto put_y = [&](int h, int k, int v, T b) {
+        const T ab = el_scale(alpha, b);
+        if constexpr (CPLX) { y[h][0][k][v] = ab.re; y[h][1][k][v] = ab.im; } else { y[h][0][k][v] = ab; }
+    };
+    auto get_y = [&](int h, int k, int v) -> T {
+        if constexpr (CPLX) return T{y[h][0][k][v], y[h][1][k][v]};
+        else return y[h][0][k][v];
     };
     auto mem_row = [&](int P) { return FORWARD ? P : nb - 1 - P; };
     if (RIGHT) {
 #pragma unroll
-        for (int k = 0; k < NBK; ++k) {
-            const int64_t j = j0 + 16 * k + jj;
+        for (int h = 0; h < RW; ++h)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int P = wave * IB + M::krow(g, v);
-                T b = T();
-                if (P < nb && j < nrhs) b = Bblk[j + (int64_t)mem_row(P) * ldb];
-                put_y(k, v, b);
+            for (int k = 0; k < NBK; ++k) {
+                const int64_t j = j0 + 16 * k + jj;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int P = (wave + WAVES * h) * IB + M::krow(g, v);
+                    // (every lane loads, from a harmless address if it has no element: loads under
+                    // conditions are waited for one by one)
+                    const bool have = P < nb && j < nrhs;
+                    const T b = Bblk[have ? j + (int64_t)mem_row(P) * ldb : 0];
+                    put_y(h, k, v, have ? b : T());
+                }
             }
-        }
+        __syncthreads();  // the flags are cleared
     } else {
         constexpr int NLD = CW * (L::NB / 2) / NT;
         // (kept as real components: arrays of complex structs end up in scratch memory)
@@ -279,13 +346,12 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
         for (int u = 0; u < NLD; ++u) {
             const int e = tid + u * NT;
             const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-#pragma unroll
-            for (int q = 0; q < NC; ++q) v0[u][q] = v1[u][q] = (R)0;
-            if (j0 + c < nrhs) {
-                const T *src = Bblk + r + (j0 + c) * ldb;
-                if (r < nb) split(src[0], v0[u]);
-                if (r + 1 < nb) split(src[1], v1[u]);
-            }
+            // (every lane loads, from a harmless address if it has no element: loads under
+            // conditions are waited for one by one)
+            const bool have0 = j0 + c < nrhs && r < nb, have1 = j0 + c < nrhs && r + 1 < nb;
+            const T b0 = Bblk[have0 ? r + (j0 + c) * ldb : 0], b1 = Bblk[have1 ? r + 1 + (j0 + c) * ldb : 0];
+            split(have0 ? b0 : T(), v0[u]);
+            split(have1 ? b1 : T(), v1[u]);
         }
 #pragma unroll
         for (int u = 0; u < NLD; ++u) {
@@ -296,12 +362,15 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
         }
         __syncthreads();
 #pragma unroll
-        for (int k = 0; k < NBK; ++k)
+        for (int h = 0; h < RW; ++h)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int P = wave * IB + M::krow(g, v);
-                put_y(k, v, (P < nb) ? S[(16 * k + jj) * L::SP + mem_row(P)] : T());
-            }
+            for (int k = 0; k < NBK; ++k)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int P = (wave + WAVES * h) * IB + M::krow(g, v);
+                    put_y(h, k, v, (P < nb) ? S[(16 * k + jj) * L::SP + mem_row(P)] : T());
+                }
+        __syncthreads();  // the staging area becomes the X slots
     }
 
     // out (+)= E * in for one sub-block E (this lane's packed values e) and the blocks `in` in
@@ -316,77 +385,159 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                     out[1][k] = M::run(e[0][c], in[1][k][c], out[1][k]);
                     out[0][k] = M::run(e[2][c], in[1][k][c], out[0][k]);
                     out[1][k] = M::run(e[1][c], in[0][k][c], out[1][k]);
-                } else {
+                } else if (NBK > 1) {
                     out[0][k] = M::run(e[0][c], in[0][k][c], out[0][k]);
                 }
             }
-    };
-    // X_s = inv(L_ss) Y_s by the wavefront that owns row s; published in buffer s & 1.
-    auto solve_row = [&](int s) {
-        Acc x[NP][NBK];
-#pragma unroll
-        for (int pp = 0; pp < NP; ++pp)
-#pragma unroll
-            for (int k = 0; k < NBK; ++k) x[pp][k] = Acc{0, 0, 0, 0};
-        block_mma(ea[s % RING], y, x);
-        R *Xs = X + (s & 1) * (NP * NBK * 64 * 4);
-#pragma unroll
-        for (int pp = 0; pp < NP; ++pp)
-#pragma unroll
-            for (int k = 0; k < NBK; ++k) {
-                y[pp][k] = x[pp][k];
-                *reinterpret_cast<Acc *>(Xs + ((pp * NBK + k) * 64 + lane) * 4) = x[pp][k];
-            }
-    };
-    if (wave == 0) solve_row(0);
-    __syncthreads();
-    // Step s: every row w > s subtracts L_ws X_s; the owner of row s+1 then solves it at once,
-    // while the other wavefronts are still updating, so each step costs one barrier and the
-    // solves stay off the critical path of everyone else.
-#pragma unroll
-    for (int s = 0; s < NBLK; ++s) {
-        if (s < nsteps) {  // uniform over the workgroup
-            const R *Xs = X + (s & 1) * (NP * NBK * 64 * 4);
-            // Sub-block (wave, s+RING-1) goes into the ring slot that step s-1 used.  With a ring
-            // of two it is the one solve_row(s+1) needs below, so it is requested first; with
-            // three it is requested behind this step's MFMAs.
-            const bool fetch = s + RING - 1 <= wave && wave < nsteps;
-            if (RING == 2 && fetch) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
-            if (wave > s && wave < nsteps) {
-                Acc xb[NP][NBK];
-#pragma unroll
-                for (int pp = 0; pp < NP; ++pp)
-#pragma unroll
-                    for (int k = 0; k < NBK; ++k)
-                        xb[pp][k] = *reinterpret_cast<const Acc *>(Xs + ((pp * NBK + k) * 64 + lane) * 4);
-                block_mma(ea[s % RING], xb, y);
-                __builtin_amdgcn_sched_barrier(0);
-                if (wave == s + 1) solve_row(s + 1);
-            }
-            if (RING > 2 && fetch) load_e(s + RING - 1, ea[(s + RING - 1) % RING]);
-            __syncthreads();
+        if constexpr (!CPLX && NBK == 1) {
+            // Two chains of two dependent MFMAs instead of one of four (the complex kernels and two
+            // column blocks have two chains anyway): half the latency on the critical path.
+            out[0][0] = M::run(e[0][0], in[0][0][0], out[0][0]);
+            Acc t = M::run(e[0][2], in[0][0][2], Acc{0, 0, 0, 0});
+            out[0][0] = M::run(e[0][1], in[0][0][1], out[0][0]);
+            t = M::run(e[0][3], in[0][0][3], t);
+            out[0][0] += t;
         }
+    };
+    // A block of X in LDS: 16-byte pieces, each piece of all 64 lanes together, so that the lanes of a
+    // 16-byte access are 16 bytes apart (no bank conflicts for FP64 either).
+    auto x_put = [&](R *Xs, int pp, int k, const Acc &a) {
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+            VT t;
+#pragma unroll
+            for (int e = 0; e < V; ++e) t[e] = a[ch * V + e];
+            *reinterpret_cast<VT *>(Xs + (((pp * NBK + k) * CH + ch) * 64 + lane) * V) = t;
+        }
+    };
+    auto x_get = [&](const R *Xs, int pp, int k) -> Acc {
+        Acc a;
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) {
+            const VT t = *reinterpret_cast<const VT *>(Xs + (((pp * NBK + k) * CH + ch) * 64 + lane) * V);
+#pragma unroll
+            for (int e = 0; e < V; ++e) a[ch * V + e] = t[e];
+        }
+        return a;
+    };
+    // There are no barriers between the steps.  Every X_s has an LDS slot of its own and a flag that
+    // its owner sets once the slot is written; a wavefront that needs X_s polls the flag.  LDS
+    // operations of one wavefront are carried out in order, so a wavefront that reads the flag as
+    // set reads the complete X_s after it.  A wavefront takes its row blocks one after the other:
+    // row w needs X_0 .. X_(w-1) as they appear, is solved and published; then row w+16 is brought up
+    // to date with everything published so far and follows the chain until its own turn.  The chain
+    // "update row s+1 with X_s, solve, publish X_(s+1)" thus competes for the MFMA pipes only with
+    // rows that are about to be needed and with wavefronts catching up, not with 31 - s updates
+    // per step that a barrier would all put in front of the next solve.
+    // Every flag a wavefront waits for belongs to a lower row, so the waits end; the poll count is
+    // bounded all the same, so that a mistake would show as a wrong result and not as a hang.
+    auto publish = [&](int s) {
+        asm volatile("" ::: "memory");  // (compiler only) the X_s stores stay in front of the flag store
+        if (lane == 0) __hip_atomic_store(published + s, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    auto wait_for = [&](int s, bool urgent) {
+        for (int polls = 0; polls < (1 << 22); ++polls) {
+            // (an atomic load: a plain one may be hoisted out of the loop, a volatile one is compiled as
+            // a flat access, which also waits for every outstanding global load)
+            if (__builtin_amdgcn_readfirstlane(
+                    __hip_atomic_load(published + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != 0)
+                break;
+            if (!urgent) __builtin_amdgcn_s_sleep(1);
+        }
+        asm volatile("" ::: "memory");  // (compiler only) the X_s loads stay behind the flag load
+    };
+    // Row block h of this wavefront: updates with X_0 .. X_(row-1), then X_row = inv(L_row,row) Y.
+    // The loop runs over groups of RING steps so that the register ring is indexed by constants;
+    // every step of a group requests a sub-block, needed or not (see above), and only steps up to
+    // the row's own do any work.
+    auto run_row = [&](auto hcst) __attribute__((always_inline)) {
+        constexpr int h = decltype(hcst)::value;
+        const int row = wave + WAVES * h;
+        if (row >= nsteps) return;
+        if constexpr (h > 0) {
+#pragma unroll
+            for (int s = 0; s < RING - 1; ++s) prefetch(h, s);
+        }
+#pragma nounroll
+        for (int s0 = 0; s0 <= row; s0 += RING) {
+#pragma unroll
+            for (int j = 0; j < RING; ++j) {
+                const int s = s0 + j;
+                {  // sub-block (row, s+RING-1) into the slot that step s-1 used
+                    const int nxt = s + RING - 1;
+                    load_e(h, nxt < row ? nxt : row, ea[(j + RING - 1) % RING]);
+                }
+                if (s < row) {
+                    const bool solves_next = s + 1 == row;
+                    if (solves_next) __builtin_amdgcn_s_setprio(2);
+                    wait_for(s, solves_next);
+                    // Said explicitly: left to itself the compiler, which cannot know which of the
+                    // conditional uses were executed, waits for all outstanding loads.
+                    wait_loads((RING - 1) * LOADS_PER_SUB);
+                    Acc xb[NP][NBK];
+                    const R *Xs = X + s * L::XS_REALS;
+#pragma unroll
+                    for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+                        for (int k = 0; k < NBK; ++k) xb[pp][k] = x_get(Xs, pp, k);
+                    block_mma(ea[j], xb, y[h]);
+                    __builtin_amdgcn_sched_barrier(0);
+                } else if (s == row) {  // every update is in: solve and publish
+                    Acc x[NP][NBK];
+#pragma unroll
+                    for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+                        for (int k = 0; k < NBK; ++k) x[pp][k] = Acc{0, 0, 0, 0};
+                    if constexpr (DIAG_REGS) {
+                        block_mma(ed[h], y[h], x);
+                    } else {
+                        wait_loads((RING - 1) * LOADS_PER_SUB);
+                        block_mma(ea[j], y[h], x);
+                    }
+                    R *Xs = X + s * L::XS_REALS;
+#pragma unroll
+                    for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+                        for (int k = 0; k < NBK; ++k) {
+                            y[h][pp][k] = x[pp][k];
+                            x_put(Xs, pp, k, x[pp][k]);
+                        }
+                    publish(s);
+                    __builtin_amdgcn_s_setprio(0);
+                }
+            }
+        }
+    };
+    if constexpr (DIAG_REGS) {
+        if (wave == 0) wait_loads((RING - 1) * LOADS_PER_SUB);  // its diagonal sub-block is needed at once
     }
+    run_row(IntC<0>{});
+    if constexpr (RW > 1) run_row(IntC<1>{});
+    static_assert(RW <= 2, "one run_row call per row block");
+    __syncthreads();  // every X_s has been read: the slots may become the staging area again
 
     if (RIGHT) {
 #pragma unroll
-        for (int k = 0; k < NBK; ++k) {
-            const int64_t j = j0 + 16 * k + jj;
+        for (int h = 0; h < RW; ++h)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int P = wave * IB + M::krow(g, v);
-                if (P < nb && j < nrhs) Bblk[j + (int64_t)mem_row(P) * ldb] = get_y(k, v);
+            for (int k = 0; k < NBK; ++k) {
+                const int64_t j = j0 + 16 * k + jj;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int P = (wave + WAVES * h) * IB + M::krow(g, v);
+                    if (P < nb && j < nrhs) Bblk[j + (int64_t)mem_row(P) * ldb] = get_y(h, k, v);
+                }
             }
-        }
     } else {
-        // The staging area was last read before the first barrier of the solve.
 #pragma unroll
-        for (int k = 0; k < NBK; ++k)
+        for (int h = 0; h < RW; ++h)
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int P = wave * IB + M::krow(g, v);
-                if (P < nb) S[(16 * k + jj) * L::SP + mem_row(P)] = get_y(k, v);
-            }
+            for (int k = 0; k < NBK; ++k)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int P = (wave + WAVES * h) * IB + M::krow(g, v);
+                    if (P < nb) S[(16 * k + jj) * L::SP + mem_row(P)] = get_y(h, k, v);
+                }
         __syncthreads();
         constexpr int NLD = CW * (L::NB / 2) / NT;
 #pragma unroll
@@ -432,9 +583,9 @@ template <typename T> struct TrsmDriver {
         pack = w;
         dispatch_record().launches++;
         if (forward)
-            return launch_kernel(trsm_pack_kernel<T, true>, dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
+            return launch_kernel(trsm_pack_kernel<T, true>, dim3(L::NBLK * (L::NBLK / L::PACK_CHUNK), nblk), dim3(256), 0, stream, A, lda, n, teff,
                                  conj, unit, w);
-        return launch_kernel(trsm_pack_kernel<T, false>, dim3(L::NBLK, nblk), dim3(256), 0, stream, A, lda, n, teff,
+        return launch_kernel(trsm_pack_kernel<T, false>, dim3(L::NBLK * (L::NBLK / L::PACK_CHUNK), nblk), dim3(256), 0, stream, A, lda, n, teff,
                              conj, unit, w);
     }
 
