@@ -385,19 +385,10 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                     out[1][k] = M::run(e[0][c], in[1][k][c], out[1][k]);
                     out[0][k] = M::run(e[2][c], in[1][k][c], out[0][k]);
                     out[1][k] = M::run(e[1][c], in[0][k][c], out[1][k]);
-                } else if (NBK > 1) {
+                } else {
                     out[0][k] = M::run(e[0][c], in[0][k][c], out[0][k]);
                 }
             }
-        if constexpr (!CPLX && NBK == 1) {
-            // Two chains of two dependent MFMAs instead of one of four (the complex kernels and two
-            // column blocks have two chains anyway): half the latency on the critical path.
-            out[0][0] = M::run(e[0][0], in[0][0][0], out[0][0]);
-            Acc t = M::run(e[0][2], in[0][0][2], Acc{0, 0, 0, 0});
-            out[0][0] = M::run(e[0][1], in[0][0][1], out[0][0]);
-            t = M::run(e[0][3], in[0][0][3], t);
-            out[0][0] += t;
-        }
     };
     // A block of X in LDS: 16-byte pieces, each piece of all 64 lanes together, so that the lanes of a
     // 16-byte access are 16 bytes apart (no bank conflicts for FP64 either).
