@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|tilemodel|vendor|tiles|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|trsm|tilemodel|vendor|tiles|copy]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
@@ -217,7 +217,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, vendor, tiles or copy "
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, trsm, vendor, tiles or copy "
                     "(profiling; copy = a plain 1 GiB device copy used to scale the HBM traffic counters; tiles = every tile "
                     "the five configurations use, --steps times each, for the counter profile)")
     args = ap.parse_args()
@@ -534,6 +534,34 @@ def main():
                     "torch_mm_tflops": round(2.0 * M * N * K / vendor_ms / 1e9, 2)}
                 del A, B, C
         extra["small_c_deep_k"] = dk
+
+    # ---- TRSM below 8192 (left, lower, no transpose, non-unit; square B, alpha = 1): a chain of short
+    #      dependent launches (packing pass, leaves of 512 equations, GEMM updates).  Each solve overwrites B
+    #      with a solution of similar size (diagonal 1..2, off-diagonal < 1/n), so calls can be repeated in
+    #      place.  The vendor's torch.linalg.solve_triangular on the same box beside it. ----
+    if args.only in ("", "trsm"):
+        ts = {}
+        for name, dt, fn in (("dtrsm", torch.float64, clblas_amd.dtrsm), ("strsm", torch.float32, clblas_amd.strsm)):
+            for m in (512, 1024, 2048, 4096):
+                A = (torch.rand(m, m, device="cuda", dtype=dt, generator=gen) - 0.5) / m     # column-major
+                A.diagonal().copy_(torch.rand(m, device="cuda", dtype=dt, generator=gen) + 1)
+                B = torch.rand(m, m, device="cuda", dtype=dt, generator=gen)
+
+                def call():
+                    st = fn(COL, LEFT, LOWER, NOTRANS, NONUNIT, m, m, 1.0, A, 0, m, B, 0, m)
+                    if st != 0:
+                        raise RuntimeError("clblas %s returned %d" % (name, st))
+                ms = timed_batch(torch, call, 20, 3)
+                launches = clblas_amd.last_dispatch()[1]
+                call()
+                launches = clblas_amd.last_dispatch()[1] - launches
+                Lt = torch.tril(A.T).contiguous()      # the same triangle as a row-major torch matrix
+                vendor_ms = timed_batch(torch, lambda: torch.linalg.solve_triangular(Lt, B, upper=False), 5, 2)
+                flops = float(m) * (m + 1) * m
+                ts["%s %d" % (name, m)] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2), "kernels_per_call": launches,
+                                           "torch_solve_triangular_tflops": round(flops / vendor_ms / 1e9, 2)}
+                del A, B, Lt
+        extra["trsm_sizes"] = ts
 
     # ---- The tile choice against the best forced tile, on shapes that are not whole rounds of any tile:
     #      tracks how well the cost model in the launcher (choose_tile) fits the kernels as they are now. ----
