@@ -77,7 +77,7 @@ template <> struct Mma16<float> {
 // it; the wavefronts are synchronised by one flag per X_s in LDS, not by barriers.
 // For side=left a right-hand side is a column of B; the panel moves between HBM and the
 // accumulator layout through an LDS staging area so that global accesses run along columns.
-template <typename T, bool RIGHT = false> struct TrsmLeaf {
+template <typename T, bool RIGHT = false, bool WIDE = false> struct TrsmLeaf {
     typedef typename Elem<T>::Real R;
     static constexpr bool CPLX = Elem<T>::CPLX;
     // Row blocks per wavefront.  Real types: two, i.e. a leaf of 512 equations.  The updates of
@@ -87,11 +87,7 @@ template <typename T, bool RIGHT = false> struct TrsmLeaf {
     // one row block (their packed sub-blocks are three times the size; LDS and registers).
     static constexpr int WAVES = 16, RW = CPLX ? 1 : 2;
     static constexpr int IB = 16, NB = WAVES * IB * RW, NBLK = NB / IB, THREADS = 64 * WAVES;
-    // Right-hand sides per workgroup.  16 gives a launch twice the workgroups (DTRSM left 2048:
-    // 0.36 -> 0.31 ms, 4096: 1.36 -> 1.28 ms, 8192 x 512: 1.52 -> 1.34 ms when it was introduced).
-    // Side = right in FP32 keeps 32: its right-hand sides are rows of B, and 16 of them are too
-    // short a run of memory; in FP64 two column blocks times two row blocks do not fit the registers.
-    static constexpr int CW = (RIGHT && !CPLX && sizeof(R) == 4) ? 32 : 16, NBK = CW / 16;
+    static constexpr int CW = WIDE ? 32 : 16, NBK = CW / 16;
     static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;  // sub-blocks (bi,bj), bi >= bj, at bi*(bi+1)/2 + bj
     // Packed sub-block: PLANES x 64 lanes x 4 reals.  Real: the values.  Complex: real parts,
     // imaginary parts, negated imaginary parts (so that no sign has to be flipped in the solve).
@@ -102,7 +98,7 @@ template <typename T, bool RIGHT = false> struct TrsmLeaf {
     static constexpr int XS_REALS = NP * NBK * 64 * 4;     // one X_s in per-lane order
     static constexpr int X_REALS = NBLK * XS_REALS;        // every X_s keeps a slot of its own
     static constexpr int SP = NB + 2;                      // pitch of the right-hand-side staging area
-    static constexpr int S_ELEMS = RIGHT ? 0 : CW * SP;    // side = right moves its rows directly
+    static constexpr int S_ELEMS = RIGHT ? 0 : 16 * SP;    // 16 right-hand sides at a time; side = right moves its rows directly
     // The staging area is only used before the first and after the last step, so it shares its
     // memory with the X slots; one "published" flag per step follows.
     static constexpr size_t X_BYTES = (size_t)X_REALS * sizeof(R), S_BYTES = (size_t)S_ELEMS * sizeof(T);
@@ -215,11 +211,11 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
 
 template <int N> struct IntC { static constexpr int value = N; };
 
-template <typename T, bool RIGHT, bool FORWARD>
+template <typename T, bool RIGHT, bool FORWARD, bool WIDE>
 __global__ void __launch_bounds__(TrsmLeaf<T>::THREADS)
 trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk,
                  int64_t ldb, int nrhs) {
-    typedef TrsmLeaf<T, RIGHT> L;
+    typedef TrsmLeaf<T, RIGHT, WIDE> L;
     typedef typename Elem<T>::Real R;
     typedef Mma16<R> M;
     typedef typename M::Acc Acc;
@@ -277,7 +273,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     // Real types keep each row's own diagonal sub-block (its inverse) in registers of its own, requested
     // first of all, so that a solve never waits for memory; the complex kernels have no registers
     // to spare for that and take it from the ring.
-    constexpr bool DIAG_REGS = !CPLX;
+    constexpr bool DIAG_REGS = !CPLX && !(WIDE && sizeof(R) == 8);  // (FP64 with 32 right-hand sides: no registers to spare either)
     R ed[DIAG_REGS ? RW : 1][PLANES][4];
     if constexpr (DIAG_REGS) {
 #pragma unroll
@@ -331,10 +327,9 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
             }
         __syncthreads();  // the flags are cleared
     } else {
-        constexpr int NLD = CW * (L::NB / 2) / NT;
+        constexpr int NLD = 16 * (L::NB / 2) / NT;
         // (kept as real components: arrays of complex structs end up in scratch memory)
         constexpr int NC = CPLX ? 2 : 1;
-        R v0[NLD][NC], v1[NLD][NC];
         auto split = [&](T t, R (&out)[NC]) {
             if constexpr (CPLX) { out[0] = t.re; out[1] = t.im; } else { out[0] = t; }
         };
@@ -343,33 +338,37 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
             else return in[0];
         };
 #pragma unroll
-        for (int u = 0; u < NLD; ++u) {
-            const int e = tid + u * NT;
-            const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-            // (every lane loads, from a harmless address if it has no element: loads under
-            // conditions are waited for one by one)
-            const bool have0 = j0 + c < nrhs && r < nb, have1 = j0 + c < nrhs && r + 1 < nb;
-            const T b0 = Bblk[have0 ? r + (j0 + c) * ldb : 0], b1 = Bblk[have1 ? r + 1 + (j0 + c) * ldb : 0];
-            split(have0 ? b0 : T(), v0[u]);
-            split(have1 ? b1 : T(), v1[u]);
-        }
+        for (int k = 0; k < NBK; ++k) {  // 16 right-hand sides at a time through the staging area
+            R v0[NLD][NC], v1[NLD][NC];
 #pragma unroll
-        for (int u = 0; u < NLD; ++u) {
-            const int e = tid + u * NT;
-            const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-            S[c * L::SP + r] = join(v0[u]);
-            S[c * L::SP + r + 1] = join(v1[u]);
-        }
-        __syncthreads();
+            for (int u = 0; u < NLD; ++u) {
+                const int e = tid + u * NT;
+                const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
+                const int64_t col = j0 + 16 * k + c;
+                // (every lane loads, from a harmless address if it has no element: loads under
+                // conditions are waited for one by one)
+                const bool have0 = col < nrhs && r < nb, have1 = col < nrhs && r + 1 < nb;
+                const T b0 = Bblk[have0 ? r + col * ldb : 0], b1 = Bblk[have1 ? r + 1 + col * ldb : 0];
+                split(have0 ? b0 : T(), v0[u]);
+                split(have1 ? b1 : T(), v1[u]);
+            }
+            if (k > 0) __syncthreads();  // the previous sixteen have been taken out
 #pragma unroll
-        for (int h = 0; h < RW; ++h)
+            for (int u = 0; u < NLD; ++u) {
+                const int e = tid + u * NT;
+                const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
+                S[c * L::SP + r] = join(v0[u]);
+                S[c * L::SP + r + 1] = join(v1[u]);
+            }
+            __syncthreads();
 #pragma unroll
-            for (int k = 0; k < NBK; ++k)
+            for (int h = 0; h < RW; ++h)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const int P = (wave + WAVES * h) * IB + M::krow(g, v);
-                    put_y(h, k, v, (P < nb) ? S[(16 * k + jj) * L::SP + mem_row(P)] : T());
+                    put_y(h, k, v, (P < nb) ? S[jj * L::SP + mem_row(P)] : T());
                 }
+        }
         __syncthreads();  // the staging area becomes the X slots
     }
 
@@ -520,25 +519,28 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                 }
             }
     } else {
+        constexpr int NLD = 16 * (L::NB / 2) / NT;
 #pragma unroll
-        for (int h = 0; h < RW; ++h)
+        for (int k = 0; k < NBK; ++k) {  // 16 right-hand sides at a time through the staging area
+            if (k > 0) __syncthreads();  // the previous sixteen have been written out
 #pragma unroll
-            for (int k = 0; k < NBK; ++k)
+            for (int h = 0; h < RW; ++h)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const int P = (wave + WAVES * h) * IB + M::krow(g, v);
-                    if (P < nb) S[(16 * k + jj) * L::SP + mem_row(P)] = get_y(h, k, v);
+                    if (P < nb) S[jj * L::SP + mem_row(P)] = get_y(h, k, v);
                 }
-        __syncthreads();
-        constexpr int NLD = CW * (L::NB / 2) / NT;
+            __syncthreads();
 #pragma unroll
-        for (int u = 0; u < NLD; ++u) {
-            const int e = tid + u * NT;
-            const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-            if (j0 + c < nrhs) {
-                T *dst = Bblk + r + (j0 + c) * ldb;
-                if (r < nb) dst[0] = S[c * L::SP + r];
-                if (r + 1 < nb) dst[1] = S[c * L::SP + r + 1];
+            for (int u = 0; u < NLD; ++u) {
+                const int e = tid + u * NT;
+                const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
+                const int64_t col = j0 + 16 * k + c;
+                if (col < nrhs) {
+                    T *dst = Bblk + r + col * ldb;
+                    if (r < nb) dst[0] = S[c * L::SP + r];
+                    if (r + 1 < nb) dst[1] = S[c * L::SP + r + 1];
+                }
             }
         }
     }
@@ -580,13 +582,13 @@ template <typename T> struct TrsmDriver {
                              conj, unit, w);
     }
 
-    template <bool RIGHT> hipError_t leaf_side(int i0, int nb, T alpha) {
-        typedef TrsmLeaf<T, RIGHT> L;
+    template <bool RIGHT, bool WIDE> hipError_t leaf_side(int i0, int nb, T alpha) {
+        typedef TrsmLeaf<T, RIGHT, WIDE> L;
         const int nrhs = RIGHT ? M : N;
         T *Bblk = RIGHT ? B + (int64_t)i0 * ldb : B + i0;
         const R *packed = pack + (int64_t)(i0 / NBL) * L::PACK_REALS;
         void (*fn)(const R *, int, T, T *, int64_t, int) =
-            forward ? trsm_diag_kernel<T, RIGHT, true> : trsm_diag_kernel<T, RIGHT, false>;
+            forward ? trsm_diag_kernel<T, RIGHT, true, WIDE> : trsm_diag_kernel<T, RIGHT, false, WIDE>;
         if (L::SMEM > 64 * 1024) {
             hipError_t e = ensure_dynamic_lds((const void *)fn, L::SMEM);
             if (e != hipSuccess) return e;
@@ -595,7 +597,19 @@ template <typename T> struct TrsmDriver {
         dispatch_record().launches++;
         return launch_kernel(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs);
     }
-    hipError_t leaf(int i0, int nb, T alpha) { return right ? leaf_side<true>(i0, nb, alpha) : leaf_side<false>(i0, nb, alpha); }
+    // Right-hand sides per workgroup.  16 gives a launch twice the workgroups; 32 (real types) gives each
+    // sub-block of coefficients twice the work and is taken when 16 would make more than one round of
+    // workgroups anyway (more than 256 x 16 right-hand sides), and for FP32 with side = right, whose
+    // right-hand sides are rows of B: 16 floats are too short a run of memory.
+    hipError_t leaf(int i0, int nb, T alpha) {
+        constexpr bool CAN_WIDEN = !Elem<T>::CPLX;
+        const int nrhs = right ? M : N;
+        const bool wide = CAN_WIDEN && (nrhs > 256 * 16 || (right && sizeof(R) == 4));
+        if constexpr (CAN_WIDEN) {
+            if (wide) return right ? leaf_side<true, true>(i0, nb, alpha) : leaf_side<false, true>(i0, nb, alpha);
+        }
+        return right ? leaf_side<true, false>(i0, nb, alpha) : leaf_side<false, false>(i0, nb, alpha);
+    }
 
     // Off-diagonal update of the block range `dst` (length nd, start d0) with the solved
     // range `src` (length ns, start s0):   B_dst <- beta * B_dst - coupling * X_src.

@@ -70,7 +70,9 @@ def backward_error(order, side, uplo, tA, diag, M, N, alpha, A, offA, lda, B0, X
 
 VARIANTS = list(itertools.product([LEFT, RIGHT], [UPPER, LOWER], [NOTRANS, TRANS], [UNIT, NONUNIT]))
 SIZES = [(1, 1), (5, 3), (37, 29), (130, 17), (23, 300), (257, 64), (300, 520), (512, 33), (513, 40), (48, 1030),
-         (3000, 1), (1, 3000), (2049, 2), (2, 2049)]
+         (3000, 1), (1, 3000), (2049, 2), (2, 2049),
+         # more than 4096 right-hand sides: the leaf takes 32 of them per workgroup
+         (37, 4130), (4130, 29), (530, 4100)]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
