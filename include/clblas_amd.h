@@ -339,8 +339,8 @@ clblasStatus clblasAmdReleaseStream(hipStream_t stream);
  * (bytes; 0 leaves a buffer alone): gemm_bytes for GEMM-shaped calls that cut K into ranges
  * (ranges x M x N elements, M rounded up to 64) or slice their last round of tiles (at most 256
  * tiles of 256 x 128 elements), trmm_bytes for TRMM's copy of B (M x N elements), trsm_bytes
- * for TRSM's packed diagonal blocks (about 35 000 elements per 256 rows of the triangle; three
- * times that for complex types).  A later call on the stream whose needs fit allocates nothing,
+ * for TRSM's packed diagonal blocks (real types: 135 168 elements per 512 rows of the triangle or
+ * part thereof; complex types: 104 448 real elements per 256 rows).  A later call on the stream whose needs fit allocates nothing,
  * so it can be the first thing recorded into a HIP graph.  A call that would have to allocate
  * while its stream is being captured returns clblasInvalidOperation and leaves the capture valid. */
 clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, size_t trmm_bytes, size_t trsm_bytes);

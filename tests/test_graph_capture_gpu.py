@@ -72,3 +72,80 @@ def test_calls_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         for i, (x, e) in enumerate(zip(ins, eager)):
             assert torch.equal(x, e), "replay %d, output %d differs from the eager result" % (rep, i)
+
+
+def test_capture_needs_buffers_that_exist_and_reserve_provides_them():
+    """A call that would have to allocate its scratch buffer while the stream is being captured
+    returns clblasInvalidOperation, enqueues nothing and leaves the capture usable;
+    clblasAmdReserveWorkspace makes the same calls capturable as the very first use of a stream;
+    clblasAmdReleaseStream gives the buffers back."""
+    import torch
+    import clblas_amd
+    assert clblas_amd.setup() == 0
+    INVALID_OPERATION = -59
+    f32, f64 = np.float32, np.float64
+
+    def dev(x):
+        return torch.from_numpy(x).cuda()
+
+    a1, b1 = dev(oracle.uniform(100 * 4096, 1, f32)), dev(oracle.uniform(4096 * 90, 2, f32))
+    c1 = dev(oracle.uniform(100 * 90, 3, f32))          # split-K: needs a workspace
+    a0, b0 = dev(oracle.uniform(512 * 64, 4, f32)), dev(oracle.uniform(64 * 512, 5, f32))
+    c0 = torch.zeros(512 * 512, device="cuda", dtype=torch.float32)   # one plain launch: needs none
+    n = 600
+    ta, tb = dev(oracle.triangular(n, n, True, 7, f64)), dev(oracle.uniform(n * 300, 8, f64))
+    c1_keep, tb_keep = c1.clone(), tb.clone()
+
+    def split_k():
+        return clblas_amd.sgemm(COL, NOTRANS, NOTRANS, 100, 90, 4096, 0.5, a1, 0, 100, b1, 0, 4096, -1.5, c1, 0, 100)
+
+    def plain():
+        return clblas_amd.sgemm(COL, NOTRANS, NOTRANS, 512, 512, 64, 1.0, a0, 0, 512, b0, 0, 64, 0.0, c0, 0, 512)
+
+    def trsm():
+        return clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, 300, 2.0, ta, 0, n, tb, 0, n)
+
+    # eager results on the default stream
+    assert split_k() == 0 and plain() == 0 and trsm() == 0
+    torch.cuda.synchronize()
+    want_c1, want_c0, want_tb = c1.clone(), c0.clone(), tb.clone()
+
+    # 1. a stream the library has never seen: the call that needs a buffer is refused under capture
+    stream = torch.cuda.Stream()
+    c1.copy_(c1_keep); c0.zero_()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        st_split = split_k()
+        st_plain = plain()
+    assert st_split == INVALID_OPERATION, st_split
+    assert st_plain == 0
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(c1, c1_keep), "the refused call must not have enqueued anything"
+    assert torch.equal(c0, want_c0)
+    del graph
+
+    # 2. the same stream after reserving: the first uses of the buffers are inside the capture
+    streams_before, _ = clblas_amd.workspace_stats()
+    assert clblas_amd.reserve_workspace(4 << 20, 0, 4 << 20, stream=stream.cuda_stream) == 0
+    streams_reserved, bytes_reserved = clblas_amd.workspace_stats()
+    assert streams_reserved == streams_before + 1 and bytes_reserved >= (8 << 20)
+    c1.copy_(c1_keep); tb.copy_(tb_keep)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        sts = [split_k(), trsm()]
+    assert sts == [0, 0], sts
+    assert clblas_amd.workspace_stats() == (streams_reserved, bytes_reserved), "a capture must not allocate"
+    for _ in range(2):
+        c1.copy_(c1_keep); tb.copy_(tb_keep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(c1, want_c1) and torch.equal(tb, want_tb)
+    del graph
+
+    # 3. releasing the stream gives its buffers back
+    assert clblas_amd.release_stream(stream.cuda_stream) == 0
+    assert clblas_amd.workspace_stats()[0] == streams_before
