@@ -75,8 +75,9 @@ template <> struct Mma16<float> {
 // other wavefronts through LDS in the same per-lane order.  A row subtracts L_ws X_s (4 MFMAs per
 // block) for every s below it as the X_s appear, then computes X_w (4 per block) and publishes
 // it; the wavefronts are synchronised by one flag per X_s in LDS, not by barriers.
-// For side=left a right-hand side is a column of B; the panel moves between HBM and the
-// accumulator layout through an LDS staging area so that global accesses run along columns.
+// Every wavefront moves its own rows between memory and the accumulator layout directly (side = left:
+// a right-hand side is a column of B, and the loads of a row block touch one cache line per column;
+// side = right: a row of B); a row is written back as soon as it is solved.
 template <typename T, bool RIGHT = false, bool WIDE = false> struct TrsmLeaf {
     typedef typename Elem<T>::Real R;
     static constexpr bool CPLX = Elem<T>::CPLX;
@@ -97,12 +98,8 @@ template <typename T, bool RIGHT = false, bool WIDE = false> struct TrsmLeaf {
     static constexpr int NP = CPLX ? 2 : 1;                // accumulators per block (re, im)
     static constexpr int XS_REALS = NP * NBK * 64 * 4;     // one X_s in per-lane order
     static constexpr int X_REALS = NBLK * XS_REALS;        // every X_s keeps a slot of its own
-    static constexpr int SP = NB + 2;                      // pitch of the right-hand-side staging area
-    static constexpr int S_ELEMS = RIGHT ? 0 : 16 * SP;    // 16 right-hand sides at a time; side = right moves its rows directly
-    // The staging area is only used before the first and after the last step, so it shares its
-    // memory with the X slots; one "published" flag per step follows.
-    static constexpr size_t X_BYTES = (size_t)X_REALS * sizeof(R), S_BYTES = (size_t)S_ELEMS * sizeof(T);
-    static constexpr size_t FLAGS_AT = ((X_BYTES > S_BYTES ? X_BYTES : S_BYTES) + 15) / 16 * 16;
+    // LDS: the X slots, then one "published" flag per step.
+    static constexpr size_t FLAGS_AT = ((size_t)X_REALS * sizeof(R) + 15) / 16 * 16;
     static constexpr size_t SMEM = FLAGS_AT + NBLK * sizeof(int);
     static constexpr int PACK_CHUNK = 8;                   // sub-blocks per workgroup of the packing pass
 };
@@ -220,14 +217,13 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     typedef Mma16<R> M;
     typedef typename M::Acc Acc;
     constexpr bool CPLX = L::CPLX;
-    constexpr int IB = L::IB, CW = L::CW, NBK = L::NBK, NT = L::THREADS, NBLK = L::NBLK, NP = L::NP;
+    constexpr int IB = L::IB, CW = L::CW, NBK = L::NBK, NBLK = L::NBLK, NP = L::NP;
     constexpr int PLANES = L::PLANES, RW = L::RW, WAVES = L::WAVES;
     constexpr int V = 16 / (int)sizeof(R);  // reals per 16 bytes
     constexpr int CH = 4 / V;               // 16-byte pieces of an accumulator block
     typedef R VT __attribute__((ext_vector_type(V)));
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     R *X = reinterpret_cast<R *>(smem_raw);
-    T *S = reinterpret_cast<T *>(smem_raw);  // shares its memory with X: used before and after the steps only
     int *published = reinterpret_cast<int *>(smem_raw + L::FLAGS_AT);
 
     const int tid = threadIdx.x;
@@ -309,68 +305,63 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
         else return y[h][0][k][v];
     };
     auto mem_row = [&](int P) { return FORWARD ? P : nb - 1 - P; };
-    if (RIGHT) {
+    // Element (equation P, right-hand side j) of the panel: rows of B for side = left, columns for right.
+    auto at = [&](int P, int64_t j) -> int64_t {
+        return RIGHT ? j + (int64_t)mem_row(P) * ldb : (int64_t)mem_row(P) + j * ldb;
+    };
+    // Every wavefront fetches its own rows straight into the accumulator layout (side = left: the four
+    // loads of a row block touch the same 16 cache lines, one per right-hand side) and writes each row
+    // back as soon as it is solved: no staging through LDS, no barrier, and both ends of the kernel
+    // overlap with the solve.
+    // FP32, side = left: a lane's four equations krow(g, 0..3) = 4g .. 4g+3 are neighbours in memory.
+    constexpr bool ROWS4 = !RIGHT && !CPLX && sizeof(R) == 4;
+    typedef float f32x4u_t __attribute__((ext_vector_type(4), aligned(4)));
 #pragma unroll
-        for (int h = 0; h < RW; ++h)
+    for (int h = 0; h < RW; ++h)
 #pragma unroll
-            for (int k = 0; k < NBK; ++k) {
-                const int64_t j = j0 + 16 * k + jj;
+        for (int k = 0; k < NBK; ++k) {
+            const int64_t j = j0 + 16 * k + jj;
+            const int P0 = (wave + WAVES * h) * IB + M::krow(g, 0);
+            if (ROWS4 && P0 + 3 < nb && j < nrhs) {
+                if constexpr (ROWS4) {
+                    const f32x4u_t t = *reinterpret_cast<const f32x4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j)));
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) put_y(h, k, v, t[FORWARD ? v : 3 - v]);
+                }
+            } else {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const int P = (wave + WAVES * h) * IB + M::krow(g, v);
                     // (every lane loads, from a harmless address if it has no element: loads under
                     // conditions are waited for one by one)
                     const bool have = P < nb && j < nrhs;
-                    const T b = Bblk[have ? j + (int64_t)mem_row(P) * ldb : 0];
+                    const T b = Bblk[have ? at(P, j) : 0];
                     put_y(h, k, v, have ? b : T());
                 }
             }
-        __syncthreads();  // the flags are cleared
-    } else {
-        constexpr int NLD = 16 * (L::NB / 2) / NT;
-        // (kept as real components: arrays of complex structs end up in scratch memory)
-        constexpr int NC = CPLX ? 2 : 1;
-        auto split = [&](T t, R (&out)[NC]) {
-            if constexpr (CPLX) { out[0] = t.re; out[1] = t.im; } else { out[0] = t; }
-        };
-        auto join = [&](const R (&in)[NC]) -> T {
-            if constexpr (CPLX) return T{in[0], in[1]};
-            else return in[0];
-        };
+        }
+    __syncthreads();  // the flags are cleared
+    auto store_row = [&](int h) {
 #pragma unroll
-        for (int k = 0; k < NBK; ++k) {  // 16 right-hand sides at a time through the staging area
-            R v0[NLD][NC], v1[NLD][NC];
+        for (int k = 0; k < NBK; ++k) {
+            const int64_t j = j0 + 16 * k + jj;
+            const int P0 = (wave + WAVES * h) * IB + M::krow(g, 0);
+            if (ROWS4 && P0 + 3 < nb && j < nrhs) {
+                if constexpr (ROWS4) {
+                    f32x4u_t t;
 #pragma unroll
-            for (int u = 0; u < NLD; ++u) {
-                const int e = tid + u * NT;
-                const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-                const int64_t col = j0 + 16 * k + c;
-                // (every lane loads, from a harmless address if it has no element: loads under
-                // conditions are waited for one by one)
-                const bool have0 = col < nrhs && r < nb, have1 = col < nrhs && r + 1 < nb;
-                const T b0 = Bblk[have0 ? r + col * ldb : 0], b1 = Bblk[have1 ? r + 1 + col * ldb : 0];
-                split(have0 ? b0 : T(), v0[u]);
-                split(have1 ? b1 : T(), v1[u]);
-            }
-            if (k > 0) __syncthreads();  // the previous sixteen have been taken out
-#pragma unroll
-            for (int u = 0; u < NLD; ++u) {
-                const int e = tid + u * NT;
-                const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-                S[c * L::SP + r] = join(v0[u]);
-                S[c * L::SP + r + 1] = join(v1[u]);
-            }
-            __syncthreads();
-#pragma unroll
-            for (int h = 0; h < RW; ++h)
+                    for (int v = 0; v < 4; ++v) t[FORWARD ? v : 3 - v] = get_y(h, k, v);
+                    *reinterpret_cast<f32x4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j))) = t;
+                }
+            } else {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
                     const int P = (wave + WAVES * h) * IB + M::krow(g, v);
-                    put_y(h, k, v, (P < nb) ? S[jj * L::SP + mem_row(P)] : T());
+                    if (P < nb && j < nrhs) Bblk[at(P, j)] = get_y(h, k, v);
                 }
+            }
         }
-        __syncthreads();  // the staging area becomes the X slots
-    }
+    };
 
     // out (+)= E * in for one sub-block E (this lane's packed values e) and the blocks `in` in
     // MFMA "B" operand order.  Complex: Re += er*inr + (-ei)*ini, Im += er*ini + ei*inr.
@@ -494,6 +485,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                         }
                     publish(s);
                     __builtin_amdgcn_s_setprio(0);
+                    store_row(h);
                 }
             }
         }
@@ -504,46 +496,6 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     run_row(IntC<0>{});
     if constexpr (RW > 1) run_row(IntC<1>{});
     static_assert(RW <= 2, "one run_row call per row block");
-    __syncthreads();  // every X_s has been read: the slots may become the staging area again
-
-    if (RIGHT) {
-#pragma unroll
-        for (int h = 0; h < RW; ++h)
-#pragma unroll
-            for (int k = 0; k < NBK; ++k) {
-                const int64_t j = j0 + 16 * k + jj;
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int P = (wave + WAVES * h) * IB + M::krow(g, v);
-                    if (P < nb && j < nrhs) Bblk[j + (int64_t)mem_row(P) * ldb] = get_y(h, k, v);
-                }
-            }
-    } else {
-        constexpr int NLD = 16 * (L::NB / 2) / NT;
-#pragma unroll
-        for (int k = 0; k < NBK; ++k) {  // 16 right-hand sides at a time through the staging area
-            if (k > 0) __syncthreads();  // the previous sixteen have been written out
-#pragma unroll
-            for (int h = 0; h < RW; ++h)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int P = (wave + WAVES * h) * IB + M::krow(g, v);
-                    if (P < nb) S[jj * L::SP + mem_row(P)] = get_y(h, k, v);
-                }
-            __syncthreads();
-#pragma unroll
-            for (int u = 0; u < NLD; ++u) {
-                const int e = tid + u * NT;
-                const int c = e / (L::NB / 2), r = (e % (L::NB / 2)) * 2;
-                const int64_t col = j0 + 16 * k + c;
-                if (col < nrhs) {
-                    T *dst = Bblk + r + col * ldb;
-                    if (r < nb) dst[0] = S[c * L::SP + r];
-                    if (r + 1 < nb) dst[1] = S[c * L::SP + r + 1];
-                }
-            }
-        }
-    }
 }
 
 template <typename T> struct TrsmDriver {
