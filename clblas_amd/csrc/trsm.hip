@@ -233,6 +233,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     const int64_t j0 = (int64_t)blockIdx.x * CW;
     const int nsteps = (nb + IB - 1) / IB;  // sub-block rows that exist
     if (tid < NBLK) published[tid] = 0;
+    __syncthreads();  // the only barrier: from here on every wavefront runs at its own pace
 
     // This wavefront owns the sub-block rows wave + WAVES*h, h < RW.
     // A lane's values of sub-block (row, s): MFMA "A" operand, plane pl, chunk c = element c.
@@ -340,7 +341,6 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                 }
             }
         }
-    __syncthreads();  // the flags are cleared
     auto store_row = [&](int h) {
 #pragma unroll
         for (int k = 0; k < NBK; ++k) {
@@ -439,6 +439,19 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
 #pragma unroll
             for (int s = 0; s < RING - 1; ++s) prefetch(h, s);
         }
+        // A second row block starts behind the chain: X_0 .. X_(row - WAVES) were published before this
+        // wavefront published its previous row.  Those steps are taken two at a time, without
+        // looking at flags: both X read together, the two products on separate accumulators so that
+        // their MFMAs alternate.  One step at a time the rate is set by the latencies of a step (flag,
+        // X, four dependent MFMAs), and the last rows of a leaf are finished by such wavefronts alone.
+        // (Which steps are paired depends on the row only, so the order of summation is fixed.)
+        constexpr bool PAIRS = h > 0 && RING >= 4 && !(WIDE && sizeof(R) == 8);
+        Acc y2[NP][NBK];
+#pragma unroll
+        for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+            for (int k = 0; k < NBK; ++k) y2[pp][k] = Acc{0, 0, 0, 0};
+        bool next_done = false;
 #pragma nounroll
         for (int s0 = 0; s0 <= row; s0 += RING) {
 #pragma unroll
@@ -448,7 +461,31 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                     const int nxt = s + RING - 1;
                     load_e(h, nxt < row ? nxt : row, ea[(j + RING - 1) % RING]);
                 }
-                if (s < row) {
+                if (PAIRS && next_done) {  // this step went with the one before
+                    next_done = false;
+                } else if (PAIRS && j % 2 == 0 && s + 1 <= row - WAVES) {
+                    if constexpr (PAIRS) {
+                        wait_loads((RING - 2) * LOADS_PER_SUB);
+                        Acc xa[NP][NBK], xb[NP][NBK];
+                        const R *Xa = X + s * L::XS_REALS, *Xb = Xa + L::XS_REALS;
+#pragma unroll
+                        for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+                            for (int k = 0; k < NBK; ++k) {
+                                xa[pp][k] = x_get(Xa, pp, k);
+                                xb[pp][k] = x_get(Xb, pp, k);
+                            }
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+#pragma unroll
+                            for (int k = 0; k < NBK; ++k) {
+                                y[h][0][k] = M::run(ea[j][0][c], xa[0][k][c], y[h][0][k]);
+                                y2[0][k] = M::run(ea[(j + 1) % RING][0][c], xb[0][k][c], y2[0][k]);
+                            }
+                        __builtin_amdgcn_sched_barrier(0);
+                        next_done = true;
+                    }
+                } else if (s < row) {
                     const bool solves_next = s + 1 == row;
                     if (solves_next) __builtin_amdgcn_s_setprio(2);
                     wait_for(s, solves_next);
@@ -464,6 +501,12 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                     block_mma(ea[j], xb, y[h]);
                     __builtin_amdgcn_sched_barrier(0);
                 } else if (s == row) {  // every update is in: solve and publish
+                    if constexpr (PAIRS) {
+#pragma unroll
+                        for (int pp = 0; pp < NP; ++pp)
+#pragma unroll
+                            for (int k = 0; k < NBK; ++k) y[h][pp][k] += y2[pp][k];
+                    }
                     Acc x[NP][NBK];
 #pragma unroll
                     for (int pp = 0; pp < NP; ++pp)
