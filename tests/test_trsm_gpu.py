@@ -112,6 +112,21 @@ def test_conjtrans_is_trans_and_alpha_zero(gpu):
     assert (logical_view(x0, COL, NOTRANS, M, N, 7, ldb) == 0).all()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_repeated_calls_give_the_same_bits(gpu, dtype):
+    """The leaf's wavefronts run at their own pace (flags, no barriers), and which X a wavefront finds
+    published first differs from run to run: the order of summation must not."""
+    for (side, uplo, tA, M, N) in [(LEFT, LOWER, NOTRANS, 1100, 530), (LEFT, UPPER, TRANS, 520, 4200),
+                                   (RIGHT, UPPER, NOTRANS, 300, 1500), (RIGHT, LOWER, TRANS, 4200, 600)]:
+        A, lda, B, ldb = make_inputs(COL, side, uplo, NONUNIT, M, N, dtype, 5)
+        st, first = gpu.trsm(COL, side, uplo, tA, NONUNIT, M, N, 1.0, A, 5, lda, B, 7, ldb)
+        assert st == 0
+        for _ in range(3):
+            st, again = gpu.trsm(COL, side, uplo, tA, NONUNIT, M, N, 1.0, A, 5, lda, B, 7, ldb)
+            assert st == 0
+            np.testing.assert_array_equal(again, first, err_msg=str((side, uplo, tA, M, N)))
+
+
 def test_config5_dtrsm_8192(gpu):
     """BASELINE config 5 at full size: Left/Lower/NoTrans/NonUnit, M=N=8192, alpha=1.
     (a) backward error on sampled right-hand sides, computed in fp64 on the host;
