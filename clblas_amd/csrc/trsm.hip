@@ -439,19 +439,26 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
 #pragma unroll
             for (int s = 0; s < RING - 1; ++s) prefetch(h, s);
         }
-        // A second row block starts behind the chain: X_0 .. X_(row - WAVES) were published before this
-        // wavefront published its previous row.  Those steps are taken two at a time, without
-        // looking at flags: both X read together, the two products on separate accumulators so that
-        // their MFMAs alternate.  One step at a time the rate is set by the latencies of a step (flag,
-        // X, four dependent MFMAs), and the last rows of a leaf are finished by such wavefronts alone.
+        // Steps are taken two at a time wherever the row is not about to be solved: both X read together,
+        // the two products on separate accumulators so that their MFMAs alternate.  One step at a time
+        // costs a wavefront the latencies of a step (flag, X, four dependent MFMAs, the way round the
+        // loop) every time, a wavefront that falls behind the chain makes the chain wait when its row's
+        // turn comes, and the last rows of a leaf are finished by such wavefronts alone.  The X are
+        // published in order, so the flag of the later one covers both; a second row block starts
+        // behind the chain (X_0 .. X_(row - WAVES) were published before this wavefront published its
+        // previous row) and needs no flags there.  The last PAIR_GAP steps before the solve go one by
+        // one: they are not to wait for a second X.
         // (Which steps are paired depends on the row only, so the order of summation is fixed.)
-        constexpr bool PAIRS = h > 0 && RING >= 4 && !(WIDE && sizeof(R) == 8);
+        constexpr int PAIR_GAP = 3;
+        constexpr bool PAIRS = RING >= 4 && !(WIDE && sizeof(R) == 8);
         Acc y2[NP][NBK];
 #pragma unroll
         for (int pp = 0; pp < NP; ++pp)
 #pragma unroll
             for (int k = 0; k < NBK; ++k) y2[pp][k] = Acc{0, 0, 0, 0};
         bool next_done = false;
+        constexpr bool SOLVE_AT_ONCE = DIAG_REGS && !WIDE;
+        bool solved = false;
 #pragma nounroll
         for (int s0 = 0; s0 <= row; s0 += RING) {
 #pragma unroll
@@ -463,8 +470,10 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                 }
                 if (PAIRS && next_done) {  // this step went with the one before
                     next_done = false;
-                } else if (PAIRS && j % 2 == 0 && s + 1 <= row - WAVES) {
+                } else if (PAIRS && j % 2 == 0 && s + 1 <= row - PAIR_GAP) {
                     if constexpr (PAIRS) {
+                        // (the X are published in order: the flag of the later one covers both)
+                        if (s + 1 > row - WAVES) wait_for(s + 1, false);
                         wait_loads((RING - 2) * LOADS_PER_SUB);
                         Acc xa[NP][NBK], xb[NP][NBK];
                         const R *Xa = X + s * L::XS_REALS, *Xb = Xa + L::XS_REALS;
@@ -500,7 +509,23 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                         for (int k = 0; k < NBK; ++k) xb[pp][k] = x_get(Xs, pp, k);
                     block_mma(ea[j], xb, y[h]);
                     __builtin_amdgcn_sched_barrier(0);
-                } else if (s == row) {  // every update is in: solve and publish
+                    if constexpr (SOLVE_AT_ONCE) {
+                        // The row's last update is followed by its solve without going round the loop
+                        // (a request for coefficients, tests, a taken branch: 300 cycles on the chain).
+                        if (solves_next) {
+                            if constexpr (PAIRS) y[h][0][0] += y2[0][0];
+                            Acc x = Acc{0, 0, 0, 0};
+#pragma unroll
+                            for (int c = 0; c < 4; ++c) x = M::run(ed[h][0][c], y[h][0][0][c], x);
+                            y[h][0][0] = x;
+                            x_put(X + row * L::XS_REALS, 0, 0, x);
+                            publish(row);
+                            __builtin_amdgcn_s_setprio(0);
+                            store_row(h);
+                            solved = true;
+                        }
+                    }
+                } else if (s == row && !(SOLVE_AT_ONCE && solved)) {  // every update is in: solve and publish
                     if constexpr (PAIRS) {
 #pragma unroll
                         for (int pp = 0; pp < NP; ++pp)
