@@ -30,7 +30,8 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef double f64x4_t __attribute__((ext_vector_type(4)));
 
 // 16 x 16 x 4 MFMA: D[i][j] += sum_k A[i][k] B[k][j]; lane l supplies A[l%16][l/16] and
-// B[l/16][l%16] and holds D[krow(l/16, v)][l%16] in accumulator element v (layouts checked
+// B[l/16][l%16] and holds D[hw(l/16, v)][l%16] in accumulator element v, hw(g, v) = 4g + v for FP32
+// and g + 4v for FP64 (layouts checked
 // on the device).
 template <typename T> struct Mma16;
 template <> struct Mma16<double> {
@@ -38,7 +39,12 @@ template <> struct Mma16<double> {
     static __device__ __forceinline__ Acc run(double a, double b, Acc c) {
         return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
     }
-    static __host__ __device__ __forceinline__ int krow(int g, int v) { return g + 4 * v; }
+    // Which equation of a sub-block a row of the MFMA stands for is free, as long as the coefficients
+    // are packed to match: row i stands for equation arow(i) = 4 (i % 4) + i / 4, so that the four
+    // rows g + 4v that a lane holds are the neighbouring equations krow(g, v) = 4g + v (one run of
+    // memory per lane, as for FP32, instead of four).
+    static __host__ __device__ __forceinline__ int krow(int g, int v) { return 4 * g + v; }
+    static __host__ __device__ __forceinline__ int arow(int i) { return 4 * (i % 4) + i / 4; }
 };
 template <> struct Mma16<float> {
     typedef f32x4_t Acc;
@@ -46,6 +52,7 @@ template <> struct Mma16<float> {
         return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
     }
     static __host__ __device__ __forceinline__ int krow(int g, int v) { return 4 * g + v; }
+    static __host__ __device__ __forceinline__ int arow(int i) { return i; }
 };
 
 // Diagonal blocks (up to 256 x 256) are solved in 16 x 16 sub-blocks on the MFMA units.
@@ -61,7 +68,7 @@ template <> struct Mma16<float> {
 // referenced triangle of A - never the other one, nor a unit diagonal - inverts the
 // small triangles L_ss by substitution and writes, per diagonal block, the NBLK (NBLK+1)/2 sub-blocks
 // inv(L_ss) and -L_ws in the order the MFMA "A" operand wants them: entry [lane][c] is
-// element (p = lane%16, q = krow(lane/16, c)), so a lane fetches its four values of a
+// element (p = arow(lane%16), q = krow(lane/16, c)), so a lane fetches its four values of a
 // sub-block with one or two 16-byte loads and nothing is broadcast.  Row w's sub-blocks
 // (w,0..w) are consecutive, so each wavefront streams its own row straight from memory
 // (L2), one to three sub-blocks ahead of their use.
@@ -162,7 +169,7 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
     for (int e = bj_lo * IB * IB + tid; e < bj_hi * IB * IB; e += 256) {
         const int bj = e / (IB * IB), w = e % (IB * IB);
         const int lane = w / 4, c = w % 4;
-        const int P = bi * IB + lane % 16, Q = bj * IB + M::krow(lane / 16, c);
+        const int P = bi * IB + M::arow(lane % 16), Q = bj * IB + M::krow(lane / 16, c);
         // Q < P always holds here; Q < nb follows from P < nb
         tr_put(out + bj * L::SUB_REALS, w, (P < nb) ? tr_sub(T(), coef(P, Q)) : T());
     }
@@ -202,7 +209,7 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
     __syncthreads();
     {
         const int lane = tid / 4, c = tid % 4;
-        tr_put(out + bi * L::SUB_REALS, tid, Ld[lane % 16][M::krow(lane / 16, c)]);
+        tr_put(out + bi * L::SUB_REALS, tid, Ld[M::arow(lane % 16)][M::krow(lane / 16, c)]);
     }
 }
 
@@ -314,9 +321,9 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     // loads of a row block touch the same 16 cache lines, one per right-hand side) and writes each row
     // back as soon as it is solved: no staging through LDS, no barrier, and both ends of the kernel
     // overlap with the solve.
-    // FP32, side = left: a lane's four equations krow(g, 0..3) = 4g .. 4g+3 are neighbours in memory.
-    constexpr bool ROWS4 = !RIGHT && !CPLX && sizeof(R) == 4;
-    typedef float f32x4u_t __attribute__((ext_vector_type(4), aligned(4)));
+    // Side = left: a lane's four equations krow(g, 0..3) = 4g .. 4g+3 are neighbours in memory.
+    constexpr bool ROWS4 = !RIGHT && !CPLX;
+    typedef R rx4u_t __attribute__((ext_vector_type(4), aligned(sizeof(R))));
 #pragma unroll
     for (int h = 0; h < RW; ++h)
 #pragma unroll
@@ -325,7 +332,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
             const int P0 = (wave + WAVES * h) * IB + M::krow(g, 0);
             if (ROWS4 && P0 + 3 < nb && j < nrhs) {
                 if constexpr (ROWS4) {
-                    const f32x4u_t t = *reinterpret_cast<const f32x4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j)));
+                    const rx4u_t t = *reinterpret_cast<const rx4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j)));
 #pragma unroll
                     for (int v = 0; v < 4; ++v) put_y(h, k, v, t[FORWARD ? v : 3 - v]);
                 }
@@ -348,10 +355,10 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
             const int P0 = (wave + WAVES * h) * IB + M::krow(g, 0);
             if (ROWS4 && P0 + 3 < nb && j < nrhs) {
                 if constexpr (ROWS4) {
-                    f32x4u_t t;
+                    rx4u_t t;
 #pragma unroll
                     for (int v = 0; v < 4; ++v) t[FORWARD ? v : 3 - v] = get_y(h, k, v);
-                    *reinterpret_cast<f32x4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j))) = t;
+                    *reinterpret_cast<rx4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j))) = t;
                 }
             } else {
 #pragma unroll
