@@ -188,7 +188,11 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
         Ld[p][q] = v;
     }
     __syncthreads();
-    // invert: thread zc < 16 solves L z = e_zc by substitution
+    // invert: thread zc < 16 solves L z = e_zc by substitution.  The sixteen reciprocals of the diagonal
+    // are taken first, all at once: one division's latency instead of sixteen in a row.
+    __shared__ T Rd[IB];
+    if (tid < IB) Rd[tid] = tr_div(el_one<T>(), Ld[tid][tid]);
+    __syncthreads();
     T z[IB];
     const int zc = tid;
     if (tid < IB) {
@@ -198,7 +202,7 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
 #pragma unroll
             for (int q = 0; q < IB; ++q)
                 if (q < p) acc = tr_sub(acc, tr_mul(Ld[p][q], z[q]));
-            z[p] = (p < zc) ? T() : tr_div(acc, Ld[p][p]);
+            z[p] = (p < zc) ? T() : tr_mul(acc, Rd[p]);
         }
     }
     __syncthreads();
