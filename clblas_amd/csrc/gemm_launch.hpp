@@ -18,7 +18,8 @@ template <typename T> struct TileEntry {
     // The same tile with deeper panels (bk_deep; 0: none), for workgroups with a long K range: half
     // the barriers and loop overhead per flop (FP32 64x64 with depth 64 instead of 32: 1024 x 1024 x 4096
     // 70.6 -> 66.5 us, 960 x 960 x 2048 38.0 -> 35.8, 1024^3 22.3 -> 21.7), but a first panel twice as
-    // long to fetch before the first MFMA (512^3: 11.4 -> 12.9 us), so only from 1024 deep.
+    // long to fetch before the first MFMA (512^3: 11.4 -> 12.9 us), so only from 1024 deep (512 for a single
+    // round of workgroups: see where the variant is chosen).
     int bk_deep;
     double deep_gain;  // factor on `eff` where the deep form runs (plain products, K range from 1024)
     size_t smem_deep[4];
@@ -258,7 +259,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         // alone leave idle, at the price of the pass that adds them up.
         auto split_cost = [&](int i, int64_t t, int s) {
             const double alone = t * s <= kCUs ? tab[i].alone : 1.0;
-            const double deep = (tab[i].bk_deep > 0 && K / s >= 1024) ? tab[i].deep_gain : 1.0;
+            const double deep = (tab[i].bk_deep > 0 && (K / s >= 1024 || (K / s >= 512 && t * s <= kCUs))) ? tab[i].deep_gain : 1.0;
             return (double)ceil_div64(t * s, kCUs) * tab[i].bm * tab[i].bn / (s * tab[i].eff * deep * alone) +
                    split_overhead_cost<T>(M, N, K, s);
         };
@@ -283,7 +284,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             double eff = tri_operand ? tab[i].eff_tri : tri_c ? tab[i].eff_tri_c : tab[i].eff;
             // (credited up to three rounds of tiles: beyond that the small tile's memory traffic costs more
             // than the deeper panels gain - 2000^3 FP32 128 TFLOP/s with 128x64 tiles, 119 with 64x64)
-            if (!need_tri && ts <= 1 && tab[i].bk_deep > 0 && K >= 1024 && t <= 3 * kCUs) eff *= tab[i].deep_gain;
+            if (!need_tri && ts <= 1 && tab[i].bk_deep > 0 && ((K >= 1024 && t <= 3 * kCUs) || (K >= 512 && t <= kCUs))) eff *= tab[i].deep_gain;
             double cost = rounds * tab[i].bm * tab[i].bn / eff;
             if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             cost *= 1.0 + tab[i].k0 / K;
@@ -476,7 +477,12 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         // A long K range per workgroup: the variant with deeper panels (K ranges are cut at multiples
         // of the tile's own depth, so they have to be multiples of the deeper one too).
         const int krange = splits > 1 ? p.k_per_split : K;
-        if ((krange >= 1024 || knobs().deep_panels > 1) && (splits <= 1 || p.k_per_split % e.bk_deep == 0)) {
+        // From 1024 deep; from 512 where the launch is a single round of workgroups (there the shorter loop
+        // wins - DGEMM 512 x 2048 x 512 22.2 -> 21.0 us, 1024 x 1024 x 768 31.1 -> 29.3 - while launches of
+        // several rounds lose the workgroups per CU that the larger LDS stage costs: 4096 x 4096 x 512 +3 %).
+        const int64_t wgs = grid_x * (splits > 1 ? splits : 1);
+        const int deep_from = knobs().deep_panels > 2 ? knobs().deep_panels : (wgs <= 256 ? 512 : 1024);  // (knob above 2: that threshold)
+        if ((krange >= deep_from || knobs().deep_panels == 2) && (splits <= 1 || p.k_per_split % e.bk_deep == 0)) {
             fn = splits > 1 ? e.splitk_deep[idx] : e.plain_deep[idx];
             smem = e.smem_deep[idx];
             bk_used = e.bk_deep;

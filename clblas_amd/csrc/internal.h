@@ -40,7 +40,7 @@ template <typename R> struct Cx { R re, im; };
 struct DebugKnobs {
     int gemm_tile = -1, split_model = 1, splits = 0, tail = 1, group_m = 0, xcd = 1, stagger = 1, log = 0;
     int wide_ld = 0;       // CLBLAS_AMD_GEMM_WIDE_LD=1: the wide-ld kernels whatever the leading dimensions (tests)
-    int deep_panels = 1;   // CLBLAS_AMD_GEMM_DEEP: 0 never the deep-panel variant of a tile, 1 by the rule, 2 wherever built
+    int deep_panels = 1;   // CLBLAS_AMD_GEMM_DEEP: 0 never the deep-panel variant of a tile, 1 by the rule, 2 wherever built, more: from that depth of a K range
 };
 const DebugKnobs &knobs();
 void reload_knobs();
