@@ -67,9 +67,9 @@ template <> struct Mma16<float> {
 // A packing pass (trsm_pack_kernel, once per call, all diagonal blocks at once) reads the
 // referenced triangle of A - never the other one, nor a unit diagonal - inverts the
 // small triangles L_ss by substitution and writes, per diagonal block, the NBLK (NBLK+1)/2 sub-blocks
-// inv(L_ss) and -L_ws in the order the MFMA "A" operand wants them: entry [lane][c] is
-// element (p = arow(lane%16), q = krow(lane/16, c)), so a lane fetches its four values of a
-// sub-block with one or two 16-byte loads and nothing is broadcast.  Row w's sub-blocks
+// inv(L_ss) and -L_ws in the order the MFMA "A" operand wants them: value c of lane `lane` is
+// element (p = arow(lane%16), q = krow(lane/16, c)), filed at packed_at(lane, c), so a lane fetches its
+// four values of a sub-block with one or two 16-byte loads and nothing is broadcast.  Row w's sub-blocks
 // (w,0..w) are consecutive, so each wavefront streams its own row straight from memory
 // (L2), one to three sub-blocks ahead of their use.
 // (The reference inverts whole 128 x 128 blocks, trtri/*.cpp; inverting only the 16 x 16
@@ -129,13 +129,21 @@ template <typename R> static __device__ __forceinline__ Cx<R> tr_div(Cx<R> a, Cx
     const R d = b.re * b.re + b.im * b.im;
     return Cx<R>{(a.re * b.re + a.im * b.im) / d, (a.im * b.re - a.re * b.im) / d};
 }
-// Writes value v (to be used as it is) into the planes of a packed sub-block at index w.
-static __device__ __forceinline__ void tr_put(float *sub, int w, float v) { sub[w] = v; }
-static __device__ __forceinline__ void tr_put(double *sub, int w, double v) { sub[w] = v; }
+// Place of value c (0..3) of lane `lane` in a plane of a packed sub-block: the plane is a row of 16-byte
+// pieces, piece k of all 64 lanes together, so that one load instruction of a wavefront reads 1 KB in one
+// run (whole cache lines; FP32: a lane's four values are one piece anyway).
+template <typename R> static __host__ __device__ __forceinline__ int packed_at(int lane, int c) {
+    constexpr int V = 16 / (int)sizeof(R);
+    return (c / V) * (64 * V) + lane * V + c % V;
+}
+// Writes value v (to be used as it is) into the planes of a packed sub-block, value w % 4 of lane w / 4.
+static __device__ __forceinline__ void tr_put(float *sub, int w, float v) { sub[packed_at<float>(w / 4, w % 4)] = v; }
+static __device__ __forceinline__ void tr_put(double *sub, int w, double v) { sub[packed_at<double>(w / 4, w % 4)] = v; }
 template <typename R> static __device__ __forceinline__ void tr_put(R *sub, int w, Cx<R> v) {
-    sub[w] = v.re;
-    sub[256 + w] = v.im;
-    sub[512 + w] = -v.im;
+    const int at = packed_at<R>(w / 4, w % 4);
+    sub[at] = v.re;
+    sub[256 + at] = v.im;
+    sub[512 + at] = -v.im;
 }
 
 // Packs all diagonal blocks of the n x n triangle (see above).  Workgroup (bi, chunk, b) of 256
@@ -252,7 +260,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
 #pragma unroll
     for (int h = 0; h < RW; ++h) {
         const int row = wave + WAVES * h;
-        erow[h] = packed + (int64_t)(row * (row + 1) / 2) * L::SUB_REALS + lane * 4;
+        erow[h] = packed + (int64_t)(row * (row + 1) / 2) * L::SUB_REALS + lane * V;
     }
     auto load_e = [&](int h, int s, R (&a)[PLANES][4]) {
 #pragma unroll
@@ -260,7 +268,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
             const R *src = erow[h] + s * L::SUB_REALS + pl * (IB * IB);
 #pragma unroll
             for (int c = 0; c < 4; c += V) {
-                VT t = *reinterpret_cast<const VT *>(src + c);
+                VT t = *reinterpret_cast<const VT *>(src + (c / V) * (64 * V));
 #pragma unroll
                 for (int e = 0; e < V && c + e < 4; ++e) a[pl][c + e] = t[e];
             }
