@@ -334,8 +334,16 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     // back as soon as it is solved: no staging through LDS, no barrier, and both ends of the kernel
     // overlap with the solve.
     // Side = left: a lane's four equations krow(g, 0..3) = 4g .. 4g+3 are neighbours in memory.
-    constexpr bool ROWS4 = !RIGHT && !CPLX;
-    typedef R rx4u_t __attribute__((ext_vector_type(4), aligned(sizeof(R))));
+    constexpr bool ROWS4 = !RIGHT;
+    constexpr int RPE = CPLX ? 2 : 1;  // reals per element
+    typedef R rx4u_t __attribute__((ext_vector_type(4 * RPE), aligned(sizeof(R))));
+    auto elem_of = [&](const rx4u_t &t, int v) -> T {
+        if constexpr (CPLX) return T{t[2 * v], t[2 * v + 1]};
+        else return t[v];
+    };
+    auto set_elem = [&](rx4u_t &t, int v, T x) {
+        if constexpr (CPLX) { t[2 * v] = x.re; t[2 * v + 1] = x.im; } else { t[v] = x; }
+    };
 #pragma unroll
     for (int h = 0; h < RW; ++h)
 #pragma unroll
@@ -346,7 +354,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                 if constexpr (ROWS4) {
                     const rx4u_t t = *reinterpret_cast<const rx4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j)));
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) put_y(h, k, v, t[FORWARD ? v : 3 - v]);
+                    for (int v = 0; v < 4; ++v) put_y(h, k, v, elem_of(t, FORWARD ? v : 3 - v));
                 }
             } else {
 #pragma unroll
@@ -369,7 +377,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                 if constexpr (ROWS4) {
                     rx4u_t t;
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) t[FORWARD ? v : 3 - v] = get_y(h, k, v);
+                    for (int v = 0; v < 4; ++v) set_elem(t, FORWARD ? v : 3 - v, get_y(h, k, v));
                     *reinterpret_cast<rx4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j))) = t;
                 }
             } else {
