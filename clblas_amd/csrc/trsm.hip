@@ -55,7 +55,7 @@ template <> struct Mma16<float> {
     static __host__ __device__ __forceinline__ int arow(int i) { return i; }
 };
 
-// Diagonal blocks (up to 256 x 256) are solved in 16 x 16 sub-blocks on the MFMA units.
+// Diagonal blocks (up to 512 x 512; complex types 256 x 256) are solved in 16 x 16 sub-blocks on the MFMA units.
 //
 // "Equation order" P = 0..nb-1 walks a diagonal block forward (index P) or backward (index
 // nb-1-P) so that equation P only involves unknowns Q <= P.  coef(P,Q) is the factor of
