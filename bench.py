@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|trsm|tilemodel|vendor|tiles|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|trsm|host|tilemodel|vendor|tiles|copy]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
@@ -10,7 +10,11 @@ count 2*M*N*K (src/client/clfunc_xgemm.hpp:95-107); DGEMM (config 4) and DTRSM (
 M*(M+1)*N flops, src/client/clfunc_xtrsm.hpp:70-92) are reported in `extra`, and so are CGEMM /
 ZGEMM at the same size (8*M*N*K flops, clfunc_xgemm.hpp:95-107) and S/D SYRK, TRMM, SYMM.
 `cpu_baseline` times the CPU oracle (a port of the reference arithmetic, OpenMP over the
-host cores) on a bounded sample of the same workload; it is a reported baseline only.
+host cores) on the same seeded inputs - configs 2 and 1 in full, configs 4 and 5 on stated
+sub-problems - and says what a run-time probe of the box's OpenCL loader found for running
+the reference itself on a CPU device; it is a reported baseline only.
+Inputs of the five BASELINE configurations come from a counter-based generator (one seed per
+matrix) that is evaluated on the device and checked against the parity tests' CPU generator.
 """
 import argparse
 import json
@@ -28,35 +32,62 @@ PEAK_FP64_MATRIX = 78.6
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "bench_8192_counters.md")
 
 
-def profiled_sgemm_traffic(dispatch):
-    """HBM-side bytes per launch of the SGEMM 8192^3 kernel, read from the tracked rocprofv3 summary
-    (two --pmc runs, FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain
-    1 GiB device copy).  Counters cannot be read from inside this process, so the figure is the
-    profile's - and it is only reported when the kernel that ran here (`dispatch`, the library's own
-    description of its last launch) is the kernel the profile measured: same tile, one launch per call.
-    Returns (bytes or None, note)."""
+def profiled_traffic(workload, dispatch, kernels_per_call=None):
+    """HBM-side bytes per call of one of the 8192 workloads ("sgemm", "dgemm", "dtrsm"), read from the
+    tracked rocprofv3 summary (two --pmc runs, FETCH_SIZE and WRITE_SIZE, each scaled by what the same
+    counter reads for a plain 1 GiB device copy).  Counters cannot be read from inside this process, so
+    the figure is the profile's - and it is only reported when what ran here is what the profile
+    measured: for the GEMMs the same tile in one plain launch (`dispatch` is the library's own
+    description of its last launch), for DTRSM the same number of kernels per call and the same tile
+    in its largest update.  Returns (bytes or None, note)."""
     import re
-    m = re.search(r"<s,(\d+)x(\d+)x(\d+),", dispatch)
-    if not m or "splits=1 " not in dispatch + " " or "tail_slices=1" not in dispatch:
-        return None, "the launch is not a single plain GEMM kernel"
-    tile = "gemm_mfma_kernel<float, %s, %s, %s," % m.groups()
-    total, seen = 0.0, set()
+    letter = {"sgemm": "s", "dgemm": "d", "dtrsm": "d"}[workload]
+    ctype = {"s": "float", "d": "double"}[letter]
+    m = re.search(r"<%s,(\d+)x(\d+)x(\d+)," % letter, dispatch or "")
+    if not m:
+        return None, "no GEMM launch on record"
+    tile = "gemm_mfma_kernel<%s, %s, %s, %s," % ((ctype,) + m.groups())
     try:
-        for line in open(TRAFFIC_PROFILE):
-            cells = [c.strip() for c in line.split("|")]
-            if len(cells) >= 6 and cells[1] == "sgemm" and cells[3] in ("FETCH_SIZE", "WRITE_SIZE"):
-                if tile not in cells[2]:
-                    return None, "profiles/bench_8192_counters.md was measured on %s, this run used %s" % (cells[2], tile)
-                total += float(cells[5].split()[0]) * 1e9
-                seen.add(cells[3])
+        lines = open(TRAFFIC_PROFILE).read().splitlines()
     except OSError as e:
         return None, "no traffic profile: %s" % e
+    if workload == "dtrsm":
+        prof_kernels, total, tile_seen = None, None, False
+        for line in lines:
+            mk = re.match(r"\* dtrsm: (\d+) kernels per call", line)
+            if mk:
+                prof_kernels = int(mk.group(1))
+            mt = re.match(r"\* dtrsm: ([0-9.]+) GB per call", line)
+            if mt:
+                total = float(mt.group(1)) * 1e9
+            cells = [c.strip() for c in line.split("|")]
+            if len(cells) >= 6 and cells[1] == "dtrsm" and tile in cells[2]:
+                tile_seen = True
+        if total is None or prof_kernels is None:
+            return None, "profiles/bench_8192_counters.md has no whole-call dtrsm figure with its kernel count"
+        if prof_kernels != kernels_per_call or not tile_seen:
+            return None, "profiles/bench_8192_counters.md measured %d kernels per call%s, this run launched %s" % (
+                prof_kernels, "" if tile_seen else " without %s...>" % tile, kernels_per_call)
+        return total, "profiles/bench_8192_counters.md, whole call of %d kernels" % prof_kernels
+    if "splits=1 " not in dispatch + " " or "tail_slices=1" not in dispatch:
+        return None, "the launch is not a single plain GEMM kernel"
+    total, seen = 0.0, set()
+    for line in lines:
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) >= 6 and cells[1] == workload and cells[3] in ("FETCH_SIZE", "WRITE_SIZE"):
+            if tile not in cells[2]:
+                return None, "profiles/bench_8192_counters.md was measured on %s, this run used %s" % (cells[2], tile)
+            total += float(cells[5].split()[0]) * 1e9
+            seen.add(cells[3])
     if seen != {"FETCH_SIZE", "WRITE_SIZE"}:
-        return None, "profiles/bench_8192_counters.md has no sgemm FETCH_SIZE / WRITE_SIZE rows"
+        return None, "profiles/bench_8192_counters.md has no %s FETCH_SIZE / WRITE_SIZE rows" % workload
     return total, "profiles/bench_8192_counters.md, kernel %s...>" % tile
 
 COL, NOTRANS, TRANS = 1, 0, 1
 LEFT, LOWER, NONUNIT = 0, 1, 1
+
+# One seed per matrix (A, B, C take seed, seed + 1, seed + 2); the CPU baseline draws the same streams.
+SEEDS = {"sgemm": 1, "dgemm": 11, "dtrsm": 21, "sgemm_config1": 31, "sgemm_config3": 41}
 
 
 def timed_calls(torch, call, steps, warmup, before_each=None):
@@ -99,6 +130,122 @@ def timed_batch(torch, call, reps, warmup, batches=3):
         torch.cuda.synchronize()
         best = min(best, start.elapsed_time(stop) / reps)
     return best
+
+
+# ---- Synthetic inputs: the counter-based generator of the parity tests, evaluated on the device ----
+# Value i of stream `seed` is mix(mix(seed) + i * GOLD) with the splitmix64 finaliser `mix`; uniform[-1,1)
+# in FP32 takes the top 24 bits (exactly representable), FP64 takes 53 bits; normal(0,1) is Box-Muller
+# on values 2i and 2i+1 of the stream.  One seed per matrix.  tests/test_bench_inputs.py checks these
+# functions against the CPU generator the GPU parity tests draw from, so the bench and the tests see
+# the same matrices for the same seeds.  (torch has no unsigned 64-bit arithmetic: int64 products wrap
+# to the same bits, and a logical right shift is an arithmetic one with the sign copies masked off.)
+def _s64(x):
+    return x - (1 << 64) if x >= (1 << 63) else x
+
+
+_GOLD, _MIX1, _MIX2 = _s64(0x9E3779B97F4A7C15), _s64(0xBF58476D1CE4E5B9), _s64(0x94D049BB133111EB)
+
+
+def _lsr(torch, z, s):
+    return (z >> s) & ((1 << (64 - s)) - 1)
+
+
+def _mix64(torch, z):
+    z = z + _GOLD
+    z = (z ^ _lsr(torch, z, 30)) * _MIX1
+    z = (z ^ _lsr(torch, z, 27)) * _MIX2
+    return z ^ _lsr(torch, z, 31)
+
+
+def _mix64_int(z):
+    m = (1 << 64) - 1
+    z = (z + 0x9E3779B97F4A7C15) & m
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & m
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & m
+    return z ^ (z >> 31)
+
+
+def stream_u64(torch, seed, first, count, device, stride=1, offset=0):
+    """Values first*stride+offset, (first+1)*stride+offset, ... of stream `seed`, as int64 bit patterns."""
+    i = torch.arange(first, first + count, device=device, dtype=torch.int64) * stride + offset
+    return _mix64(torch, i * _GOLD + _s64(_mix64_int(seed & ((1 << 64) - 1))))
+
+
+def _in_chunks(torch, n, device, dtype, piece, chunk=1 << 24):
+    out = torch.empty(n, device=device, dtype=dtype)
+    for first in range(0, n, chunk):
+        count = min(chunk, n - first)
+        out[first:first + count] = piece(first, count)
+    return out
+
+
+def gen_uniform(torch, n, seed, dtype, device="cuda"):
+    """n values uniform in [-1, 1) from stream `seed`."""
+    if dtype == torch.float32:
+        return _in_chunks(torch, n, device, dtype, lambda f, c: (
+            _lsr(torch, stream_u64(torch, seed, f, c, device), 40).double() * (1.0 / 8388608.0) - 1.0).float())
+    return _in_chunks(torch, n, device, dtype, lambda f, c: (
+        2.0 * (_lsr(torch, stream_u64(torch, seed, f, c, device), 11).double() * (1.0 / 9007199254740992.0)) - 1.0))
+
+
+def gen_normal(torch, n, seed, dtype, device="cuda"):
+    """n values from normal(0, 1): Box-Muller on values 2i, 2i+1 of stream `seed`."""
+    import math
+
+    def piece(f, c):
+        u1 = 1.0 - _lsr(torch, stream_u64(torch, seed, f, c, device, 2, 0), 11).double() * (1.0 / 9007199254740992.0)
+        u2 = _lsr(torch, stream_u64(torch, seed, f, c, device, 2, 1), 11).double() * (1.0 / 9007199254740992.0)
+        return (torch.sqrt(-2.0 * torch.log(u1)) * torch.cos((2.0 * math.pi) * u2)).to(dtype)
+    return _in_chunks(torch, n, device, dtype, piece)
+
+
+def gen_triangular(torch, n, seed, dtype, device="cuda"):
+    """Column-major n x n (tight ld) lower triangle: strict part uniform[-1,1)/n, diagonal uniform[1,2),
+    NaN above the diagonal (element (r, c) is value r + c n of stream `seed`)."""
+    unit = _in_chunks(torch, n * n, device, torch.float64, lambda f, c: (
+        _lsr(torch, stream_u64(torch, seed, f, c, device), 11).double() * (1.0 / 9007199254740992.0)))
+    U = unit.view(n, n)                       # U[c, r] is element (r, c)
+    A = (2.0 * U - 1.0) / float(n)
+    A.diagonal().copy_(1.0 + U.diagonal())
+    upper = torch.ones(n, n, device=device, dtype=torch.bool).tril(-1)   # c > r in this view
+    A.masked_fill_(upper, float("nan"))
+    return A.to(dtype).reshape(-1)
+
+
+def opencl_cpu_probe():
+    """What the OpenCL loader on this box offers for running the reference clBLAS on the host cores:
+    enumerates the platforms and asks each for CL_DEVICE_TYPE_CPU devices.  Returns (usable, text)."""
+    import ctypes
+    import ctypes.util
+    name = ctypes.util.find_library("OpenCL") or "libOpenCL.so.1"
+    try:
+        cl = ctypes.CDLL(name)
+    except OSError as e:
+        return False, "no OpenCL loader (%s)" % e
+    try:
+        nplat = ctypes.c_uint(0)
+        rc = cl.clGetPlatformIDs(0, None, ctypes.byref(nplat))
+        if rc != 0 or nplat.value == 0:
+            return False, "%s loads, clGetPlatformIDs -> code %d, %d platforms" % (name, rc, nplat.value)
+        plats = (ctypes.c_void_p * nplat.value)()
+        cl.clGetPlatformIDs(nplat.value, plats, None)
+        seen, cpus = [], 0
+        for p in plats:
+            buf = ctypes.create_string_buffer(256)
+            cl.clGetPlatformInfo(ctypes.c_void_p(p), 0x0902, 256, buf, None)            # CL_PLATFORM_NAME
+            ncpu, nall = ctypes.c_uint(0), ctypes.c_uint(0)
+            rc_cpu = cl.clGetDeviceIDs(ctypes.c_void_p(p), ctypes.c_uint64(2), 0, None, ctypes.byref(ncpu))   # CL_DEVICE_TYPE_CPU
+            rc_all = cl.clGetDeviceIDs(ctypes.c_void_p(p), ctypes.c_uint64(0xFFFFFFFF), 0, None, ctypes.byref(nall))
+            if rc_cpu != 0:
+                ncpu.value = 0
+            if rc_all != 0:
+                nall.value = 0
+            cpus += ncpu.value
+            seen.append("'%s': %d CPU devices (code %d), %d devices of any type (code %d)" % (
+                buf.value.decode(errors="replace"), ncpu.value, rc_cpu, nall.value, rc_all))
+        return cpus > 0, "%s: %d platform(s): %s" % (name, nplat.value, "; ".join(seen))
+    except Exception as e:   # a loader without these entry points
+        return False, "%s: probe failed: %s" % (name, e)
 
 
 TILE_MODEL_SHAPES = (
@@ -253,9 +400,9 @@ def main():
 
     # ---- SGEMM, BASELINE config 2 -------------------------------------------------------
     if args.only in ("", "sgemm"):
-        A = torch.rand(n * n, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
-        B = torch.rand(n * n, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
-        C = torch.rand(n * n, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+        A = gen_uniform(torch, n * n, SEEDS["sgemm"], torch.float32)
+        B = gen_uniform(torch, n * n, SEEDS["sgemm"] + 1, torch.float32)
+        C = gen_uniform(torch, n * n, SEEDS["sgemm"] + 2, torch.float32)
 
         def sgemm():
             st = clblas_amd.sgemm(COL, NOTRANS, NOTRANS, n, n, n, 1.0, A, 0, n, B, 0, n, 1.0, C, 0, n)
@@ -267,7 +414,7 @@ def main():
         c0abs_v = C.view(n, n).T.double().abs() @ v.abs()
         wall, ev_ms = timed_calls(torch, sgemm, steps, warmup)
         dispatch = clblas_amd.last_dispatch()[0]
-        traffic, traffic_note = profiled_sgemm_traffic(dispatch) if n == 8192 else (None, "size is not 8192")
+        traffic, traffic_note = profiled_traffic("sgemm", dispatch) if n == 8192 else (None, "size is not 8192")
         # Self-check of the timed result: every call did C <- A B + C, so after `calls` of them
         # C v = C0 v + calls * A (B v).  Evaluated in double precision on the device.
         calls = steps + warmup
@@ -305,9 +452,9 @@ def main():
 
     # ---- DGEMM, BASELINE config 4 -------------------------------------------------------
     if args.only in ("", "dgemm"):
-        A = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
-        B = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
-        C = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
+        A = gen_normal(torch, n * n, SEEDS["dgemm"], torch.float64)
+        B = gen_normal(torch, n * n, SEEDS["dgemm"] + 1, torch.float64)
+        C = gen_normal(torch, n * n, SEEDS["dgemm"] + 2, torch.float64)
 
         def dgemm():
             st = clblas_amd.dgemm(COL, NOTRANS, TRANS, n, n, n, 1.0, A, 0, n, B, 0, n, 0.5, C, 0, n)
@@ -333,22 +480,24 @@ def main():
         extra.setdefault("checked", {})["dgemm"] = {"what": "C v = C0 v / 2^calls + (2 - 2^(1-calls)) A (B^T v), in double precision",
                                                      "tolerance": "8 u calls |C| |v|", "worst_error_over_tolerance": float("%.3g" % dgemm_check), "ok": True}
         d_tflops = 2.0 * n * n * n / (wall / steps) / 1e12
+        d_kernel_tflops = 2.0 * n * n * n / (ev_ms * 1e-3) / 1e12
+        d_traffic, d_note = profiled_traffic("dgemm", dgemm_dispatch) if n == 8192 else (None, "size is not 8192")
         extra["dgemm"] = {"workload": "BASELINE config 4: DGEMM column-major NT %d^3, alpha=1, beta=0.5, normal(0,1)" % n,
                           "tflops": round(d_tflops, 3), "ms_per_call": round(wall * 1e3 / steps, 4),
-                          "launch_ms": round(ev_ms, 4), "kernel": dgemm_dispatch,
-                          "pct_of_fp64_matrix_peak": round(100 * d_tflops / PEAK_FP64_MATRIX, 2)}
+                          "pct_of_fp64_matrix_peak": round(100 * d_tflops / PEAK_FP64_MATRIX, 2),
+                          "roofline": {"bound": "mfma", "achieved": round(d_kernel_tflops, 3), "peak": PEAK_FP64_MATRIX,
+                                       "unit": "TFLOP/s", "frac": round(d_kernel_tflops / PEAK_FP64_MATRIX, 4),
+                                       "traffic": d_traffic, "traffic_source": d_note, "kernel": dgemm_dispatch,
+                                       "launch_ms": round(ev_ms, 4)}}
         del A, B, C
     else:
         d_tflops = None
 
     # ---- DTRSM, BASELINE config 5 -------------------------------------------------------
     if args.only in ("", "dtrsm"):
-        A = torch.rand(n * n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1
-        A /= n
+        A = gen_triangular(torch, n, SEEDS["dtrsm"], torch.float64)   # NaN above the diagonal: must not be read
         Av = A.view(n, n)  # Av[c, r] is element (r, c) of the column-major matrix
-        Av.diagonal().copy_(torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) + 1)
-        Av.copy_(torch.where(torch.ones(n, n, device="cuda", dtype=torch.bool).tril(-1), torch.full_like(Av, float("nan")), Av))
-        B0 = torch.randn(n * n, device="cuda", dtype=torch.float64, generator=gen)
+        B0 = gen_normal(torch, n * n, SEEDS["dtrsm"] + 1, torch.float64)
         B = B0.clone()
 
         def restore():
@@ -362,6 +511,7 @@ def main():
         tsteps = max(3, steps // 2)
         launches_before = clblas_amd.last_dispatch()[1]
         wall, ev_ms = timed_calls(torch, dtrsm, tsteps, 2, before_each=restore)
+        trsm_dispatch, trsm_launches_after = clblas_amd.last_dispatch()
         t_tflops = float(n) * (n + 1) * n / (ev_ms * 1e-3) / 1e12
         # Residual of the last timed solve on sampled right-hand sides: ||L X - B|| / (||L|| ||X|| + ||B||)
         # by columns (inf-norms, double precision on the device) against 2 n eps.
@@ -376,10 +526,19 @@ def main():
             raise RuntimeError("DTRSM result fails its residual check: %.3g of the bound" % dtrsm_check)
         extra.setdefault("checked", {})["dtrsm"] = {"what": "backward error of 64 sampled right-hand sides against 2 n eps",
                                                      "worst_error_over_bound": float("%.3g" % dtrsm_check), "ok": True}
-        extra["dtrsm"] = {"workload": "BASELINE config 5: DTRSM Left/Lower/NoTrans/NonUnit M=N=%d, alpha=1" % n,
+        kernels_per_call = (trsm_launches_after - launches_before) // (tsteps + 2)
+        t_traffic, t_note = profiled_traffic("dtrsm", trsm_dispatch, kernels_per_call) if n == 8192 else (None, "size is not 8192")
+        extra["dtrsm"] = {"workload": "BASELINE config 5: DTRSM Left/Lower/NoTrans/NonUnit M=N=%d, alpha=1; A: strict lower triangle "
+                                      "uniform[-1,1)/M, diagonal uniform[1,2), NaN above; B normal(0,1)" % n,
                           "tflops": round(t_tflops, 3), "ms_per_call": round(ev_ms, 4),
-                          "kernels_per_call": (clblas_amd.last_dispatch()[1] - launches_before) // (tsteps + 2),
-                          "finite": bool(torch.isfinite(B).all().item())}
+                          "kernels_per_call": kernels_per_call,
+                          "finite": bool(torch.isfinite(B).all().item()),
+                          # one call = all of its kernels on one stream: achieved = M (M + 1) N flops over the call's time
+                          "roofline": {"bound": "mfma", "achieved": round(t_tflops, 3), "peak": PEAK_FP64_MATRIX,
+                                       "unit": "TFLOP/s", "frac": round(t_tflops / PEAK_FP64_MATRIX, 4),
+                                       "traffic": t_traffic, "traffic_source": t_note,
+                                       "kernel": "%d kernels per call; last update: %s" % (kernels_per_call, trsm_dispatch),
+                                       "launch_ms": round(ev_ms, 4)}}
         if d_tflops:
             extra["dtrsm"]["pct_of_dgemm_rate"] = round(100 * t_tflops / d_tflops, 2)
         del A, B, B0
@@ -474,13 +633,13 @@ def main():
     if args.only in ("", "configs"):
         shapes = {}
 
-        def sgemm_case(M, N, K, tA, tB, alpha, beta, pad, offs):
+        def sgemm_case(M, N, K, tA, tB, alpha, beta, pad, offs, seed):
             ra, ca = (K, M) if tA else (M, K)   # rows x columns as stored (column-major)
             rb, cb = (N, K) if tB else (K, N)
             lda, ldb, ldc = ra + pad, rb + pad, M + pad
-            A = torch.rand(offs[0] + lda * ca, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
-            B = torch.rand(offs[1] + ldb * cb, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
-            C = torch.rand(offs[2] + ldc * N, device="cuda", dtype=torch.float32, generator=gen) * 2 - 1
+            A = gen_uniform(torch, offs[0] + lda * ca, seed, torch.float32)
+            B = gen_uniform(torch, offs[1] + ldb * cb, seed + 1, torch.float32)
+            C = gen_uniform(torch, offs[2] + ldc * N, seed + 2, torch.float32)
 
             def call():
                 st = clblas_amd.sgemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2],
@@ -489,7 +648,7 @@ def main():
                     raise RuntimeError("clblasSgemm returned %d" % st)
             return timed_batch(torch, call, 20 if 2.0 * M * N * K > 1e10 else 100, 5)
 
-        ms = sgemm_case(1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0))
+        ms = sgemm_case(1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0), SEEDS["sgemm_config1"])
         shapes["config1 1024x1024x1024 NN"] = {"ms": round(ms, 4), "tflops": round(2.0 * 1024 ** 3 / ms / 1e9, 2)}
         for (M, N, K) in ((4097, 4095, 1031), (65536, 64, 4096), (64, 65536, 4096), (127, 129, 8192)):
             flops = 2.0 * M * N * K
@@ -498,7 +657,7 @@ def main():
                    "hbm_bound_ms": round(nbytes / 8e12 * 1e3, 4)}
             for tA, tB, tag in ((NOTRANS, NOTRANS, "NN"), (NOTRANS, TRANS, "NT"), (TRANS, NOTRANS, "TN"),
                                 (TRANS, TRANS, "TT")):
-                ms = sgemm_case(M, N, K, tA, tB, 0.7, -1.3, 3, (5, 7, 11))
+                ms = sgemm_case(M, N, K, tA, tB, 0.7, -1.3, 3, (5, 7, 11), SEEDS["sgemm_config3"])
                 row[tag] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2),
                             "GBps": round(nbytes / ms / 1e6, 1)}
             shapes["config3 %dx%dx%d" % (M, N, K)] = row
@@ -563,6 +722,51 @@ def main():
                 del A, B, Lt
         extra["trsm_sizes"] = ts
 
+    # ---- Host time per call: 10 000 back-to-back calls, CPU clock around the enqueue loop only (the device
+    #      is drained before and after, outside the clock).  Calls go straight to the C symbols with
+    #      prebuilt ctypes arguments; `ctypes_floor_us` is the same loop on a call that fails validation
+    #      at once (M = 0), i.e. the cost of getting from Python into the library and back.  When the
+    #      device is slower than the host the loop blocks on the full queue, so `us_per_call` is an upper
+    #      bound on the host cost and never less than the device time per call. ----
+    if args.only in ("", "host"):
+        import ctypes
+        lib = clblas_amd.load_library()
+        sz, vp, dbl = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_double
+        m = 512
+        A = gen_triangular(torch, m, 51, torch.float64)
+        A = torch.nan_to_num(A)
+        B = gen_uniform(torch, m * m, 52, torch.float64)
+        C = torch.zeros(m * m, device="cuda", dtype=torch.float64)
+        stream = vp(torch.cuda.current_stream().cuda_stream)
+        host = {}
+
+        def loop(f, argv, calls):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(calls):
+                f(*argv)
+            dt = time.perf_counter() - t0
+            torch.cuda.synchronize()
+            return dt / calls * 1e6
+
+        def gemm_args(mm):
+            return (COL, NOTRANS, NOTRANS, sz(mm), sz(m), sz(m), dbl(1.0), vp(A.data_ptr()), sz(0), sz(m), vp(B.data_ptr()), sz(0),
+                    sz(m), dbl(0.0), vp(C.data_ptr()), sz(0), sz(m), stream)
+
+        def trsm_args(mm):
+            return (COL, LEFT, LOWER, NOTRANS, NONUNIT, sz(mm), sz(m), dbl(1.0), vp(A.data_ptr()), sz(0), sz(m), vp(B.data_ptr()),
+                    sz(0), sz(m), stream)
+        for name, f, mk in (("dgemm_512", lib.clblasDgemm, gemm_args), ("dtrsm_512", lib.clblasDtrsm, trsm_args)):
+            if f(*mk(m)) != 0:
+                raise RuntimeError("%s failed" % name)
+            n0 = clblas_amd.last_dispatch()[1]
+            us = min(loop(f, mk(m), 10000) for _ in range(2))
+            kernels = (clblas_amd.last_dispatch()[1] - n0) / 20000.0
+            floor = loop(f, mk(0), 10000)
+            host[name] = {"us_per_call": round(us, 2), "ctypes_floor_us": round(floor, 2), "kernels_per_call": kernels}
+        del A, B, C
+        extra["host_enqueue_us"] = host
+
     # ---- The tile choice against the best forced tile, on shapes that are not whole rounds of any tile:
     #      tracks how well the cost model in the launcher (choose_tile) fits the kernels as they are now. ----
     if args.only in ("", "tilemodel"):
@@ -595,29 +799,70 @@ def main():
         del T, Bt
         extra["vendor_yardstick"] = vy
 
-    # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores ----
+    # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores, same seeds as the
+    #      GPU legs; config 2 and config 1 in full, configs 4 and 5 on stated sub-problems (the same
+    #      streams at the smaller size).  The reference library itself would need a CPU OpenCL device:
+    #      the probe below reports what this box's OpenCL loader offers. ----
     cpu = None
     if not args.no_cpu and args.only == "":
         import numpy as np
         import oracle
-        m_s, n_s, k_s = n, n, n           # the whole workload (about 10 s on 16 host cores)
-        a = oracle.uniform(m_s * k_s, 1, np.float32)
-        b = oracle.uniform(k_s * n_s, 2, np.float32)
-        c = oracle.uniform(m_s * n_s, 3, np.float32)
-        oracle.gemm(COL, NOTRANS, NOTRANS, 256, 64, 256, 1.0, a, 0, m_s, b, 0, k_s, 1.0, c, 0, m_s)  # warm-up
-        t0 = time.perf_counter()
-        oracle.gemm(COL, NOTRANS, NOTRANS, m_s, n_s, k_s, 1.0, a, 0, m_s, b, 0, k_s, 1.0, c, 0, m_s)
-        dt = time.perf_counter() - t0
-        cpu = {"value": round(2.0 * m_s * n_s * k_s / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(),
+        usable, seen = opencl_cpu_probe()
+        pocl = ("reference-on-PoCL: unavailable (%s%s)" % (
+            seen, "; a CPU device is present but no reference libclBLAS is built for it" if usable else ""))
+
+        def clock(f):
+            t0 = time.perf_counter()
+            st = f()
+            if st not in (0, None):
+                raise RuntimeError("oracle call returned %s" % st)
+            return time.perf_counter() - t0
+
+        m_s = n                         # config 2, the whole workload (about 10 s on 16 host cores)
+        a = oracle.uniform(m_s * m_s, SEEDS["sgemm"], np.float32)
+        b = oracle.uniform(m_s * m_s, SEEDS["sgemm"] + 1, np.float32)
+        c = oracle.uniform(m_s * m_s, SEEDS["sgemm"] + 2, np.float32)
+        oracle.gemm(COL, NOTRANS, NOTRANS, 256, 64, 256, 1.0, a, 0, m_s, b, 0, m_s, 1.0, c, 0, m_s)  # warm-up
+        dt = clock(lambda: oracle.gemm(COL, NOTRANS, NOTRANS, m_s, m_s, m_s, 1.0, a, 0, m_s, b, 0, m_s, 1.0, c, 0, m_s))
+        cpu = {"value": round(2.0 * m_s ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": oracle.num_threads(),
                "kind": "port",
-               "sample": "oracle SGEMM NN, M=%d N=%d K=%d, one call (%.1f s); the reference clBLAS itself needs an "
-                         "OpenCL device (PoCL), which this image does not have" % (m_s, n_s, k_s, dt)}
+               "sample": "config 2 in full: oracle SGEMM NN %d^3, one call, %.1f s" % (m_s, dt),
+               "reference_on_pocl": pocl}
+        del a, b, c
+        others = {}
+        m1 = 1024                       # config 1 in full
+        a = oracle.uniform(m1 * m1, SEEDS["sgemm_config1"], np.float32)
+        b = oracle.uniform(m1 * m1, SEEDS["sgemm_config1"] + 1, np.float32)
+        c = oracle.uniform(m1 * m1, SEEDS["sgemm_config1"] + 2, np.float32)
+        dt = min(clock(lambda: oracle.gemm(COL, NOTRANS, NOTRANS, m1, m1, m1, 1.0, a, 0, m1, b, 0, m1, 0.0, c, 0, m1))
+                 for _ in range(3))
+        others["config1_sgemm_1024"] = {"value": round(2.0 * m1 ** 3 / dt / 1e12, 5), "unit": "TFLOP/s",
+                                        "sample": "config 1 in full: SGEMM NN 1024^3, beta=0, best of 3 calls, %.3f s" % dt}
+        m4 = min(n, 2048)               # config 4 on its leading 2048^3 problem (flops scale with M N K: x%d for the whole)
+        a = oracle.normal(m4 * m4, SEEDS["dgemm"], np.float64)
+        b = oracle.normal(m4 * m4, SEEDS["dgemm"] + 1, np.float64)
+        c = oracle.normal(m4 * m4, SEEDS["dgemm"] + 2, np.float64)
+        dt = clock(lambda: oracle.gemm(COL, NOTRANS, TRANS, m4, m4, m4, 1.0, a, 0, m4, b, 0, m4, 0.5, c, 0, m4))
+        others["config4_dgemm"] = {"value": round(2.0 * m4 ** 3 / dt / 1e12, 5), "unit": "TFLOP/s",
+                                   "sample": "config 4 at M=N=K=%d (1/%d of the flops of %d^3): DGEMM NT, alpha=1, beta=0.5, "
+                                             "one call, %.2f s" % (m4, (n // m4) ** 3, n, dt)}
+        m5 = min(n, 4096)               # config 5 at 4096: the reference's blocked algorithm (inverted 128-blocks + GEMM sweeps)
+        a = oracle.triangular(m5, m5, True, SEEDS["dtrsm"], np.float64)
+        b = oracle.normal(m5 * m5, SEEDS["dtrsm"] + 1, np.float64)
+        dt = clock(lambda: oracle.trsm_blocked(COL, LEFT, LOWER, NOTRANS, NONUNIT, m5, m5, 1.0, a, 0, m5, b, 0, m5))
+        others["config5_dtrsm"] = {"value": round(float(m5) * (m5 + 1) * m5 / dt / 1e12, 5), "unit": "TFLOP/s",
+                                   "sample": "config 5 at M=N=%d (1/%d of the flops of %d): oracle restatement of gpu_dtrsm128, "
+                                             "one call, %.2f s" % (m5, (n // m5) ** 3, n, dt)}
+        del a, b, c
+        cpu["other_configs"] = others
 
     if result is None:
         result = {"metric": "partial run (--only %s)" % args.only, "value": None, "unit": "TFLOP/s", "n_gpus": 1,
                   "steps": steps, "warmup": warmup}
     result["cpu_baseline"] = cpu
-    result["extra"] = extra
+    # The bulky tables first, the other two BASELINE workloads last: a reader of the end of the line sees them.
+    last = ("sgemm_configs_1_and_3", "trsm_sizes", "host_enqueue_us", "checked", "sgemm_pct_of_fp32_matrix_peak", "dgemm", "dtrsm")
+    result["extra"] = {k: extra[k] for k in sorted(extra, key=lambda k: last.index(k) if k in last else -1)}
     print(json.dumps(result))
 
 

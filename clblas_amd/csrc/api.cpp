@@ -49,6 +49,7 @@ void read_knobs() {
     k.deep_panels = env_int("CLBLAS_AMD_GEMM_DEEP", 1);
     k.wide_ld = env_int("CLBLAS_AMD_GEMM_WIDE_LD", 0);
     k.log = env_int("CLBLAS_AMD_LOG", 0);
+    k.check_mem = env_int("CLBLAS_AMD_CHECK_MEM", 0);
     g_knobs = k;
 }
 }  // namespace
@@ -89,12 +90,15 @@ void hip_ws_release(int device, void *ptr) {
     (void)hipFree(ptr);
     if (cur != device) (void)hipSetDevice(cur);
 }
-void hip_ws_sync(int device) {
+bool hip_ws_sync(int device) {
     int cur = 0;
     (void)hipGetDevice(&cur);
     if (cur != device) (void)hipSetDevice(device);
-    (void)hipDeviceSynchronize();
+    // (fails, for one, while a stream of the device is being captured in global mode)
+    const hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) (void)hipGetLastError();
     if (cur != device) (void)hipSetDevice(cur);
+    return e == hipSuccess;
 }
 WorkspaceCache &ws_cache() {
     static WorkspaceCache cache(WorkspaceAllocator{hip_ws_alloc, hip_ws_release, hip_ws_sync});
@@ -102,47 +106,134 @@ WorkspaceCache &ws_cache() {
 }
 std::mutex g_lds_mutex;
 std::map<std::pair<int, const void *>, size_t> g_lds_limit;
+
+thread_local DryRun *tl_dry_run = nullptr;
+thread_local CallLease *tl_lease = nullptr;
+
+bool stream_is_capturing(hipStream_t stream) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return cap != hipStreamCaptureStatusNone;
+}
 }  // namespace
+
+DryRun *&dry_run_slot() { return tl_dry_run; }
+
+CallLease::CallLease() : outer(tl_lease) { tl_lease = this; }
+CallLease::~CallLease() {
+    if (held) ws_cache().unlease(device, (const void *)stream);
+    tl_lease = outer;
+}
 
 hipError_t workspace_get(hipStream_t stream, size_t bytes, int kind, void **out) {
     *out = nullptr;
+    if (DryRun *dry = tl_dry_run) {  // only the size is wanted; the pointer is never used
+        if (bytes > dry->need[kind]) dry->need[kind] = bytes;
+        *out = reinterpret_cast<void *>(uintptr_t(256));
+        return hipSuccess;
+    }
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
+    // The first request of an API call takes the call's lease on the stream's entry (CallLease).
+    CallLease *lease = tl_lease;
+    const bool want_lease = lease && !lease->held;
     WorkspaceError why = WS_OK;
-    // Fast path: the buffer exists (no question about capture needed).
-    void *p = ws_cache().get(dev, (const void *)stream, kind, bytes, false, &why);
-    if (!p) {
+    bool pinned = false;
+    // Fast path: the buffer exists.
+    void *p = ws_cache().get(dev, (const void *)stream, kind, bytes, false, &why, want_lease, &pinned);
+    if (p) {
+        // A buffer handed out under capture ends up in a graph: the entry is pinned from then on.
+        if (!pinned && stream_is_capturing(stream)) ws_cache().pin(dev, (const void *)stream);
+    } else {
         // It has to be allocated: not on a stream that is being captured into a graph (hipMalloc
         // there would fail and invalidate the capture).
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(stream, &cap) != hipSuccess) cap = hipStreamCaptureStatusNone;
-        if (cap != hipStreamCaptureStatusNone) return hipErrorStreamCaptureUnsupported;
-        p = ws_cache().get(dev, (const void *)stream, kind, bytes, true, &why);
+        if (stream_is_capturing(stream)) return hipErrorStreamCaptureUnsupported;
+        p = ws_cache().get(dev, (const void *)stream, kind, bytes, true, &why, want_lease, &pinned);
         if (!p) return hipErrorOutOfMemory;
+    }
+    if (want_lease) {
+        lease->held = true;
+        lease->device = dev;
+        lease->stream = stream;
     }
     *out = p;
     return hipSuccess;
 }
 
-void workspace_release_all() { ws_cache().release_all(); }
+bool workspace_release_all() { return ws_cache().release_all(); }
 void ws_release_stream(int device, hipStream_t stream) { ws_cache().release_stream(device, (const void *)stream); }
 void ws_stats(size_t *streams, size_t *bytes) {
     if (streams) *streams = ws_cache().stream_count();
     if (bytes) *bytes = ws_cache().bytes_held();
 }
 
+// Kernels that need more than 64 KiB of dynamic LDS have the limit raised once per (function,
+// device).  Every launch of such a kernel asks, so the answer for the usual case - already raised -
+// comes from a small open-addressed table of atomics without taking a lock; the mutex and the map
+// behind it serve the first call per pair and anything the table has no room for.
+namespace {
+constexpr int kLdsSlots = 1024, kLdsDevices = 16;
+struct LdsSlot {
+    std::atomic<const void *> fn{nullptr};
+    std::atomic<size_t> limit[kLdsDevices];
+};
+LdsSlot g_lds_slots[kLdsSlots];
+
+std::atomic<size_t> *lds_slot_for(const void *fn, int dev) {
+    if (dev < 0 || dev >= kLdsDevices) return nullptr;
+    size_t h = (reinterpret_cast<uintptr_t>(fn) >> 4) * 0x9e3779b97f4a7c15ULL >> 40;
+    for (int probe = 0; probe < 16; ++probe, ++h) {
+        LdsSlot &s = g_lds_slots[h % kLdsSlots];
+        const void *cur = s.fn.load(std::memory_order_acquire);
+        if (cur == nullptr) {
+            const void *expected = nullptr;
+            if (s.fn.compare_exchange_strong(expected, fn, std::memory_order_acq_rel)) cur = fn;
+            else cur = expected;
+        }
+        if (cur == fn) return &s.limit[dev];
+    }
+    return nullptr;
+}
+}  // namespace
+
 hipError_t ensure_dynamic_lds(const void *fn, size_t bytes) {
     int dev = 0;
     hipError_t err = hipGetDevice(&dev);
     if (err != hipSuccess) return err;
+    std::atomic<size_t> *fast = lds_slot_for(fn, dev);
+    if (fast && fast->load(std::memory_order_acquire) >= bytes) return hipSuccess;
     std::lock_guard<std::mutex> lock(g_lds_mutex);
     size_t &cur = g_lds_limit[std::make_pair(dev, fn)];
-    if (cur >= bytes) return hipSuccess;
-    err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (err == hipSuccess) cur = bytes;
-    return err;
+    if (cur < bytes) {
+        err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (err != hipSuccess) return err;
+        cur = bytes;
+    }
+    if (fast) fast->store(cur, std::memory_order_release);
+    return hipSuccess;
 }
+
+// ---- CLBLAS_AMD_CHECK_MEM: how much memory lies behind a device pointer ----
+namespace {
+size_t hip_mem_probe(const void *ptr) {
+    hipDeviceptr_t base = nullptr;
+    size_t size = 0;
+    if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr) != hipSuccess || !base) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    const uintptr_t b = reinterpret_cast<uintptr_t>(base), p = reinterpret_cast<uintptr_t>(ptr);
+    return (p >= b && p - b < size) ? size - (p - b) : 0;
+}
+std::atomic<MemProbe> g_mem_probe{hip_mem_probe};
+}  // namespace
+
+void set_mem_probe(MemProbe probe) { g_mem_probe.store(probe ? probe : hip_mem_probe); }
+size_t mem_behind(const void *ptr) { return g_mem_probe.load()(ptr); }
 
 }  // namespace cba
 
@@ -154,17 +245,36 @@ clblasStatus lead_dim_error(MatId m) {
     return m == MAT_A ? clblasInvalidLeadDimA : (m == MAT_B ? clblasInvalidLeadDimB : clblasInvalidLeadDimC);
 }
 
+clblasStatus mem_error(MatId m, bool insufficient) {
+    if (insufficient)
+        return m == MAT_A ? clblasInsufficientMemMatA : (m == MAT_B ? clblasInsufficientMemMatB : clblasInsufficientMemMatC);
+    return m == MAT_A ? clblasInvalidMatA : (m == MAT_B ? clblasInvalidMatB : clblasInvalidMatC);
+}
+
 // Restates checkMatrixSizes (generic/common.c:585-688) for a rows x cols logical matrix:
 // zero dimension -> InvalidDim; ld below the number of elements that are contiguous in
-// memory -> InvalidLeadDim{A,B,C}.  The reference's third outcome, InsufficientMemMat*,
-// compares against CL_MEM_SIZE of the cl_mem; a raw device pointer carries no size, so
-// that code cannot arise here.
+// memory -> InvalidLeadDim{A,B,C}.  The reference's third outcome, InsufficientMemMat*
+// (common.c:644-684), compares offset + footprint against CL_MEM_SIZE of the cl_mem.  A raw
+// device pointer carries no size, so by default that code cannot arise; with the debug switch
+// CLBLAS_AMD_CHECK_MEM=1 the allocation behind `base` is looked up and the same rule applied:
+// (off + (lines - 1) ld + run) sizeof(T) beyond the memory behind the pointer ->
+// InsufficientMemMat{A,B,C}; a pointer that no allocation holds -> InvalidMat{A,B,C} (the
+// reference's answer when clGetMemObjectInfo fails).
 clblasStatus check_matrix_sizes(clblasOrder order, clblasTranspose trans, size_t rows, size_t cols, size_t ld,
-                                MatId which) {
+                                MatId which, const void *base, size_t off, size_t tsize) {
     if (rows == 0 || cols == 0) return clblasInvalidDim;
     const bool rows_contiguous = (order == clblasRowMajor && trans != clblasNoTrans) ||
                                  (order == clblasColumnMajor && trans == clblasNoTrans);
     if (rows_contiguous ? (ld < rows) : (ld < cols)) return lead_dim_error(which);
+    if (cba::knobs().check_mem) {
+        const size_t mem = cba::mem_behind(base);
+        if (mem == 0) return mem_error(which, false);
+        const size_t run = rows_contiguous ? rows : cols, lines = rows_contiguous ? cols : rows;
+        // ((lines - 1) ld + run + off) tsize, refusing anything that leaves 64 bits on the way
+        unsigned __int128 used = (unsigned __int128)(lines - 1) * ld + run + off;
+        used *= tsize;
+        if (used > (unsigned __int128)mem) return mem_error(which, true);
+    }
     return clblasSuccess;
 }
 
@@ -190,6 +300,7 @@ template <typename T, bool NOALLOC = false>
 clblasStatus gemm_front(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M,
                         size_t N, size_t K, T alpha, const T *A, size_t offA, size_t lda, const T *B, size_t offB,
                         size_t ldb, T beta, T *C, size_t offC, size_t ldc, hipStream_t stream) {
+    cba::CallLease lease;  // scratch handed out during this call stays ours until it returns
     // Order of checks follows xgemm.cc:685-706: objects A, B, C; then (K != 0) sizes of A,
     // sizes of B; then sizes of C.
     if (!A) return clblasInvalidMatA;
@@ -198,10 +309,10 @@ clblasStatus gemm_front(clblasOrder order, clblasTranspose transA, clblasTranspo
     if (!valid_order(order) || !valid_trans(transA) || !valid_trans(transB)) return clblasInvalidValue;
     clblasStatus st;
     if (K != 0) {
-        if ((st = check_matrix_sizes(order, transA, M, K, lda, MAT_A)) != clblasSuccess) return st;
-        if ((st = check_matrix_sizes(order, transB, K, N, ldb, MAT_B)) != clblasSuccess) return st;
+        if ((st = check_matrix_sizes(order, transA, M, K, lda, MAT_A, A, offA, sizeof(*A))) != clblasSuccess) return st;
+        if ((st = check_matrix_sizes(order, transB, K, N, ldb, MAT_B, B, offB, sizeof(*B))) != clblasSuccess) return st;
     }
-    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldc, MAT_C, C, offC, sizeof(*C))) != clblasSuccess) return st;
     if (M > kMaxDim || N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
 
     // Real types: ConjTrans is Trans (xgemm.cc:330-335); the real launchers ignore cA / cB.
@@ -235,22 +346,23 @@ template <typename T>
 clblasStatus syrk_front(clblasOrder order, clblasUplo uplo, clblasTranspose transA, size_t N, size_t K, T alpha,
                         const T *A, size_t offA, size_t lda, T beta, T *C, size_t offC, size_t ldc,
                         hipStream_t stream) {
+    cba::CallLease lease;  // scratch handed out during this call stays ours until it returns
     if (!A) return clblasInvalidMatA;
     if (!C) return clblasInvalidMatC;
     if (!valid_order(order) || !valid_trans(transA) || (uplo != clblasUpper && uplo != clblasLower))
         return clblasInvalidValue;
     if (IsComplex<T>::value && transA == clblasConjTrans) return clblasInvalidValue;
     clblasStatus st;
-    if ((st = check_matrix_sizes(order, transA, N, K, lda, MAT_A)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, transA, N, K, lda, MAT_A, A, offA, sizeof(*A))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C, C, offC, sizeof(*C))) != clblasSuccess) return st;
     if (N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
     bool lower = uplo == clblasLower, trans = transA != clblasNoTrans;
     if (order == clblasRowMajor) {
         lower = !lower;
         trans = !trans;
     }
-    return map_hip_error(cba::syrk_colmajor<T>(lower, trans, (int)N, (int)K, alpha, A + offA, (int64_t)lda, beta,
-                                               C + offC, (int64_t)ldc, stream));
+    return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::syrk_colmajor<T>(lower, trans, (int)N, (int)K, alpha, A + offA, (int64_t)lda, beta,
+                                               C + offC, (int64_t)ldc, stream); }));
 }
 
 // TRMM front end.  Checks as doTrmm (src/library/blas/xtrmm.c:47-64), the same as TRSM's;
@@ -259,6 +371,7 @@ template <typename T>
 clblasStatus trmm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
                         clblasDiag diag, size_t M, size_t N, T alpha, const T *A, size_t offA, size_t lda, T *B,
                         size_t offB, size_t ldb, hipStream_t stream) {
+    cba::CallLease lease;  // scratch handed out during this call stays ours until it returns
     if (!A) return clblasInvalidMatA;
     if (!B) return clblasInvalidMatB;
     if (!valid_order(order) || !valid_trans(transA) || (side != clblasLeft && side != clblasRight) ||
@@ -266,8 +379,8 @@ clblasStatus trmm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clb
         return clblasInvalidValue;
     const size_t msize = side == clblasLeft ? M : N;
     clblasStatus st;
-    if ((st = check_matrix_sizes(order, transA, msize, msize, lda, MAT_A)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, transA, msize, msize, lda, MAT_A, A, offA, sizeof(*A))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B, B, offB, sizeof(*B))) != clblasSuccess) return st;
     if (M > kMaxDim || N > kMaxDim) return clblasNotImplemented;
     bool right = side == clblasRight, lower = uplo == clblasLower;
     if (order == clblasRowMajor) {
@@ -275,10 +388,10 @@ clblasStatus trmm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clb
         right = !right;
         lower = !lower;
     }
-    return map_hip_error(cba::trmm_colmajor<T>(right, lower, transA != clblasNoTrans,
+    return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::trmm_colmajor<T>(right, lower, transA != clblasNoTrans,
                                                IsComplex<T>::value && transA == clblasConjTrans, diag == clblasUnit,
                                                (int)M, (int)N, alpha, A + offA, (int64_t)lda, B + offB, (int64_t)ldb,
-                                               stream));
+                                               stream); }));
 }
 
 // SYMM front end.  Checks as doSymm (src/library/blas/xsymm.c:50-71): objects A, B, C; A is
@@ -288,6 +401,7 @@ template <typename T, bool HERM = false>
 clblasStatus symm_front(clblasOrder order, clblasSide side, clblasUplo uplo, size_t M, size_t N, T alpha, const T *A,
                         size_t offA, size_t lda, const T *B, size_t offB, size_t ldb, T beta, T *C, size_t offC,
                         size_t ldc, hipStream_t stream) {
+    cba::CallLease lease;  // scratch handed out during this call stays ours until it returns
     if (!A) return clblasInvalidMatA;
     if (!B) return clblasInvalidMatB;
     if (!C) return clblasInvalidMatC;
@@ -296,9 +410,9 @@ clblasStatus symm_front(clblasOrder order, clblasSide side, clblasUplo uplo, siz
         return clblasInvalidValue;
     const size_t msize = side == clblasLeft ? M : N;
     clblasStatus st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, msize, msize, lda, MAT_A)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, msize, msize, lda, MAT_A, A, offA, sizeof(*A))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B, B, offB, sizeof(*B))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldc, MAT_C, C, offC, sizeof(*C))) != clblasSuccess) return st;
     if (M > kMaxDim || N > kMaxDim) return clblasNotImplemented;
     bool right = side == clblasRight, lower = uplo == clblasLower;
     if (order == clblasRowMajor) {
@@ -307,11 +421,11 @@ clblasStatus symm_front(clblasOrder order, clblasSide side, clblasUplo uplo, siz
         lower = !lower;
     }
     if constexpr (HERM)  // HEMM goes through doSymm as well (xhemm.c:69-73), same checks and folding
-        return map_hip_error(cba::hemm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
-                                                   B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+        return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::hemm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
+                                                   B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream); }));
     else
-        return map_hip_error(cba::symm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
-                                                   B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+        return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::symm_colmajor<T>(right, lower, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
+                                                   B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream); }));
 }
 
 // SYR2K front end.  Checks as doSyr2k (src/library/blas/xsyr2k.c:58-76): objects A, B, C;
@@ -321,6 +435,7 @@ template <typename T>
 clblasStatus syr2k_front(clblasOrder order, clblasUplo uplo, clblasTranspose transAB, size_t N, size_t K, T alpha,
                          const T *A, size_t offA, size_t lda, const T *B, size_t offB, size_t ldb, T beta, T *C,
                          size_t offC, size_t ldc, hipStream_t stream) {
+    cba::CallLease lease;  // scratch handed out during this call stays ours until it returns
     if (!A) return clblasInvalidMatA;
     if (!B) return clblasInvalidMatB;
     if (!C) return clblasInvalidMatC;
@@ -328,17 +443,17 @@ clblasStatus syr2k_front(clblasOrder order, clblasUplo uplo, clblasTranspose tra
         return clblasInvalidValue;
     if (IsComplex<T>::value && transAB == clblasConjTrans) return clblasInvalidValue;
     clblasStatus st;
-    if ((st = check_matrix_sizes(order, transAB, N, K, lda, MAT_A)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, transAB, N, K, ldb, MAT_B)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, transAB, N, K, lda, MAT_A, A, offA, sizeof(*A))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, transAB, N, K, ldb, MAT_B, B, offB, sizeof(*B))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C, C, offC, sizeof(*C))) != clblasSuccess) return st;
     if (N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
     bool lower = uplo == clblasLower, trans = transAB != clblasNoTrans;
     if (order == clblasRowMajor) {
         lower = !lower;
         trans = !trans;
     }
-    return map_hip_error(cba::syr2k_colmajor<T>(lower, trans, (int)N, (int)K, alpha, A + offA, (int64_t)lda, B + offB,
-                                                (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+    return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::syr2k_colmajor<T>(lower, trans, (int)N, (int)K, alpha, A + offA, (int64_t)lda, B + offB,
+                                                (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream); }));
 }
 
 // HERK / HER2K front end (B == nullptr with `two` false: HERK).  Checks as doHerk / doHer2k
@@ -350,6 +465,7 @@ template <typename R>
 clblasStatus herk_front(bool two, clblasOrder order, clblasUplo uplo, clblasTranspose trans, size_t N, size_t K,
                         cba::Cx<R> alpha, const cba::Cx<R> *A, size_t offA, size_t lda, const cba::Cx<R> *B,
                         size_t offB, size_t ldb, R beta, cba::Cx<R> *C, size_t offC, size_t ldc, hipStream_t stream) {
+    cba::CallLease lease;  // scratch handed out during this call stays ours until it returns
     if (!A) return clblasInvalidMatA;
     if (two && !B) return clblasInvalidMatB;
     if (!C) return clblasInvalidMatC;
@@ -357,9 +473,9 @@ clblasStatus herk_front(bool two, clblasOrder order, clblasUplo uplo, clblasTran
         return clblasInvalidValue;
     if (trans == clblasTrans) return clblasInvalidValue;
     clblasStatus st;
-    if ((st = check_matrix_sizes(order, trans, N, K, lda, MAT_A)) != clblasSuccess) return st;
-    if (two && (st = check_matrix_sizes(order, trans, N, K, ldb, MAT_B)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, trans, N, K, lda, MAT_A, A, offA, sizeof(*A))) != clblasSuccess) return st;
+    if (two && (st = check_matrix_sizes(order, trans, N, K, ldb, MAT_B, B, offB, sizeof(*B))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, N, N, ldc, MAT_C, C, offC, sizeof(*C))) != clblasSuccess) return st;
     if (N > kMaxDim || K > kMaxDim) return clblasNotImplemented;
     bool lower = uplo == clblasLower, ctrans = trans != clblasNoTrans;
     if (order == clblasRowMajor) {
@@ -368,10 +484,10 @@ clblasStatus herk_front(bool two, clblasOrder order, clblasUplo uplo, clblasTran
         alpha.im = -alpha.im;
     }
     if (!two)
-        return map_hip_error(cba::herk_colmajor<R>(lower, ctrans, (int)N, (int)K, alpha.re, A + offA, (int64_t)lda,
-                                                   beta, C + offC, (int64_t)ldc, stream));
-    return map_hip_error(cba::her2k_colmajor<R>(lower, ctrans, (int)N, (int)K, alpha, A + offA, (int64_t)lda,
-                                                B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+        return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::herk_colmajor<R>(lower, ctrans, (int)N, (int)K, alpha.re, A + offA, (int64_t)lda,
+                                                   beta, C + offC, (int64_t)ldc, stream); }));
+    return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::her2k_colmajor<R>(lower, ctrans, (int)N, (int)K, alpha, A + offA, (int64_t)lda,
+                                                B + offB, (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream); }));
 }
 
 static_assert(sizeof(FloatComplex) == sizeof(cba::Cx<float>) && sizeof(DoubleComplex) == sizeof(cba::Cx<double>),
@@ -388,6 +504,7 @@ template <typename T>
 clblasStatus trsm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clblasTranspose transA,
                         clblasDiag diag, size_t M, size_t N, T alpha, const T *A, size_t offA, size_t lda, T *B,
                         size_t offB, size_t ldb, hipStream_t stream) {
+    cba::CallLease lease;  // scratch handed out during this call stays ours until it returns
     // Order of checks follows doTrsm (functor_xtrsm.cc:57-75): objects, A (msize^2), B (M x N).
     if (!A) return clblasInvalidMatA;
     if (!B) return clblasInvalidMatB;
@@ -396,8 +513,8 @@ clblasStatus trsm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clb
         return clblasInvalidValue;
     const size_t msize = side == clblasLeft ? M : N;
     clblasStatus st;
-    if ((st = check_matrix_sizes(order, transA, msize, msize, lda, MAT_A)) != clblasSuccess) return st;
-    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B)) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, transA, msize, msize, lda, MAT_A, A, offA, sizeof(*A))) != clblasSuccess) return st;
+    if ((st = check_matrix_sizes(order, clblasNoTrans, M, N, ldb, MAT_B, B, offB, sizeof(*B))) != clblasSuccess) return st;
     if (M > kMaxDim || N > kMaxDim) return clblasNotImplemented;
 
     bool right = side == clblasRight, lower = uplo == clblasLower;
@@ -409,9 +526,9 @@ clblasStatus trsm_front(clblasOrder order, clblasSide side, clblasUplo uplo, clb
         right = !right;
         lower = !lower;
     }
-    return map_hip_error(cba::trsm_colmajor<T>(right, lower, transA != clblasNoTrans, transA == clblasConjTrans,
+    return map_hip_error(cba::with_workspaces_secured(stream, [&] { return cba::trsm_colmajor<T>(right, lower, transA != clblasNoTrans, transA == clblasConjTrans,
                                                diag == clblasUnit, (int)M, (int)N, alpha, A + offA, (int64_t)lda,
-                                               B + offB, (int64_t)ldb, stream));
+                                               B + offB, (int64_t)ldb, stream); }));
 }
 
 }  // namespace
@@ -451,7 +568,9 @@ clblasStatus clblasSetup(void) {
     return clblasSuccess;
 }
 
-void clblasTeardown(void) { cba::workspace_release_all(); }
+// Synchronises every device that holds scratch buffers, then frees them (buffers of a device that
+// cannot be synchronised - one of its streams is being captured - stay until the next call).
+void clblasTeardown(void) { (void)cba::workspace_release_all(); }
 
 void clblasAmdReloadDebugEnv(void) { cba::reload_knobs(); }
 
@@ -473,6 +592,16 @@ clblasStatus clblasAmdReleaseStream(hipStream_t stream) {
     if (hipGetDevice(&dev) != hipSuccess) {
         (void)hipGetLastError();
         return clblasInvalidDevice;
+    }
+    // The buffers go back to the device at once, so everything the stream was given has to be through
+    // with them: wait for the stream first.  A stream under capture cannot be waited for (and the
+    // graph would keep pointers into the buffers): refuse.
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone) return clblasInvalidOperation;
+    (void)hipGetLastError();
+    if (hipStreamSynchronize(stream) != hipSuccess) {
+        (void)hipGetLastError();
+        return clblasInvalidCommandQueue;
     }
     cba::ws_release_stream(dev, stream);
     return clblasSuccess;

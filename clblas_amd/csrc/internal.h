@@ -11,6 +11,15 @@
 
 namespace cba {
 
+// Dry run of a call's launch sequence on the calling thread: while one is active, launch_kernel
+// launches nothing and workspace_get only records how much scratch of each kind was asked for.
+// Routines made of several launches use it on a stream under graph capture to secure every buffer
+// before the first kernel is enqueued (see with_workspaces_secured).
+struct DryRun {
+    size_t need[3] = {0, 0, 0};
+};
+DryRun *&dry_run_slot();  // thread-local; nullptr: launches are real
+
 // Launches `fn` and returns the status of THIS launch.  (The <<<>>> form reports through the
 // thread's sticky error, which would also pick up - and clear - an error that unrelated code of
 // the caller left there.)
@@ -24,6 +33,7 @@ template <typename... KArgs, typename... Args>
 inline hipError_t launch_kernel(void (*fn)(KArgs...), dim3 grid, dim3 block, size_t smem, hipStream_t stream,
                                 Args &&...args) {
     static_assert(sizeof...(KArgs) == sizeof...(Args), "argument count");
+    if (dry_run_slot()) return hipSuccess;
     std::tuple<KArgs...> t(static_cast<KArgs>(args)...);
     return launch_kernel_impl(fn, grid, block, smem, stream, t, std::index_sequence_for<KArgs...>());
 }
@@ -37,8 +47,11 @@ template <typename R> struct Cx { R re, im; };
 //   CLBLAS_AMD_GEMM_TILE (index into the per-type tile table, -1: model's choice), _SPLIT_MODEL,
 //   _SPLITS, _TAIL, _GROUP_M (0: default), _XCD, _STAGGER: see the tile choice in gemm_launch.hpp;
 //   CLBLAS_AMD_LOG=1: one line per kernel launch on stderr.
+//   CLBLAS_AMD_CHECK_MEM=1: every operand is looked up among the device allocations and a matrix that
+//   does not fit behind its pointer is refused with clblasInsufficientMemMat{A,B,C}.
 struct DebugKnobs {
     int gemm_tile = -1, split_model = 1, splits = 0, tail = 1, group_m = 0, xcd = 1, stagger = 1, log = 0;
+    int check_mem = 0;
     int wide_ld = 0;       // CLBLAS_AMD_GEMM_WIDE_LD=1: the wide-ld kernels whatever the leading dimensions (tests)
     int deep_panels = 1;   // CLBLAS_AMD_GEMM_DEEP: 0 never the deep-panel variant of a tile, 1 by the rule, 2 wherever built, more: from that depth of a K range
 };
@@ -63,9 +76,37 @@ DispatchRecord &dispatch_record();  // thread-local
 // hipErrorOutOfMemory if the allocation fails; hipErrorStreamCaptureUnsupported if `stream`
 // is being captured into a graph and the buffer would have to be allocated now.
 hipError_t workspace_get(hipStream_t stream, size_t bytes, int kind, void **out);
-void workspace_release_all();
+bool workspace_release_all();  // false: some device could not be synchronised and keeps its buffers
 void ws_release_stream(int device, hipStream_t stream);
 void ws_stats(size_t *streams, size_t *bytes);
+
+// Holds the calling thread's claim on the scratch buffers it is handed between the first
+// workspace_get of an API call and the end of that call: while the claim stands the buffers of
+// that (device, stream) are not given up to make room for another stream (a thread that has its
+// pointer but has not enqueued its kernels yet would otherwise launch on freed memory).  One per
+// extern "C" entry point, on the stack.
+struct CallLease {
+    CallLease();
+    ~CallLease();
+    CallLease(const CallLease &) = delete;
+    CallLease &operator=(const CallLease &) = delete;
+    bool held = false;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    CallLease *outer = nullptr;
+};
+
+// Runs `body` (a sequence of launches on `stream`).  On a stream that is being captured into a graph
+// the sequence is first walked dry, and every scratch buffer it will ask for is secured before the
+// first kernel is enqueued: a call that would have to allocate fails with
+// hipErrorStreamCaptureUnsupported and leaves its operands untouched, instead of failing half-way.
+template <typename F> hipError_t with_workspaces_secured(hipStream_t stream, F &&body);
+
+// Bytes from `ptr` to the end of the device allocation that holds it; 0 if no allocation is known
+// to hold it.  The default asks the HIP runtime; tests put their own table in its place.
+typedef size_t (*MemProbe)(const void *ptr);
+void set_mem_probe(MemProbe probe);  // nullptr: back to the HIP lookup
+size_t mem_behind(const void *ptr);
 
 // Caller-supplied scratch that replaces workspace_get for one call (the entry point that
 // must not allocate): requests beyond `bytes` fail with hipErrorOutOfMemory.
@@ -156,5 +197,24 @@ hipError_t hemm_colmajor(bool right, bool lower, int M, int N, T alpha, const T 
 template <typename T>
 hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool conj, bool unit, int M, int N, T alpha, const T *A,
                          int64_t lda, T *B, int64_t ldb, hipStream_t stream);
+
+template <typename F> hipError_t with_workspaces_secured(hipStream_t stream, F &&body) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (dry_run_slot() || hipStreamIsCapturing(stream, &cap) != hipSuccess || cap == hipStreamCaptureStatusNone)
+        return body();
+    DryRun dry;
+    const DispatchRecord kept = dispatch_record();
+    dry_run_slot() = &dry;
+    hipError_t e = body();
+    dry_run_slot() = nullptr;
+    dispatch_record() = kept;
+    if (e != hipSuccess) return e;
+    for (int kind = 0; kind < 3; ++kind) {
+        if (!dry.need[kind]) continue;
+        void *p = nullptr;
+        if ((e = workspace_get(stream, dry.need[kind], kind, &p)) != hipSuccess) return e;
+    }
+    return body();
+}
 
 }  // namespace cba

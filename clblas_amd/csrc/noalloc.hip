@@ -22,7 +22,7 @@ namespace {
 constexpr size_t kScratchBytes = CLBLAS_AMD_NOALLOC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
-constexpr int kMaxDevices = 64;
+constexpr int kMaxDevices = 64;  // device ordinals beyond this are refused (hipErrorInvalidDevice)
 std::mutex g_mutex;
 void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, once looked up
 
@@ -52,6 +52,25 @@ hipError_t sgemm_colmajor_noalloc(bool transA, bool transB, int M, int N, int K,
                                   int64_t lda, const float *B, int64_t ldb, float beta, float *C, int64_t ldc,
                                   hipStream_t stream) {
     FixedScratch fixed;
+    fixed.ptr = nullptr;
+    {
+        // The address is looked up once per device.  That lookup may load the code object, which is
+        // not something to do in the middle of a stream capture: a first call per device that finds
+        // its stream being captured is refused (clblasSetup, or one call outside a capture, comes first).
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        bool known = false;
+        if (dev >= 0 && dev < kMaxDevices) {
+            std::lock_guard<std::mutex> lock(g_mutex);
+            known = g_scratch_ptr[dev] != nullptr;
+        }
+        if (!known) {
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+                return hipErrorStreamCaptureUnsupported;
+        }
+    }
     hipError_t e = noalloc_scratch(&fixed.ptr);
     if (e != hipSuccess) return e;
     fixed.bytes = kScratchBytes;

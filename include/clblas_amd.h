@@ -109,12 +109,16 @@ typedef struct DoubleComplex_ { double s[2]; } __attribute__((aligned(16))) Doub
 clblasStatus clblasGetVersion(unsigned int *major, unsigned int *minor, unsigned int *patch);
 
 /* Replaces clblasSetup (src/clBLAS.h:196-197, src/library/blas/init.c:43-223).
- * Checks that a gfx950 device is current and its code object loads.  GEMM and TRSM
- * do not require it (the reference's GEMM path does not check it either). */
+ * Checks that a gfx950 device is current and its code object loads.  No routine of this library
+ * requires it: where the reference's S/C/Z TRSM return clblasNotInitialized without it
+ * (src/library/blas/functor/functor_xtrsm.cc:57-59), these run (as the reference's GEMM and
+ * DTRSM paths do, which never ask).  clblasNotInitialized is never returned. */
 clblasStatus clblasSetup(void);
 
 /* Replaces clblasTeardown (src/clBLAS.h:208-209, src/library/blas/init.c:232-263).
- * Releases the library-owned device workspace. */
+ * Waits for every device that holds library-owned scratch buffers (hipDeviceSynchronize) and
+ * frees them; buffers of a device that cannot be waited for (one of its streams is being
+ * captured) are kept. */
 void clblasTeardown(void);
 
 /* Replaces clblasSgemm (src/clBLAS.h:7382-7405, src/library/blas/xgemm.cc:667-723).
@@ -137,7 +141,10 @@ clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTransp
  * A call that would need more scratch than that (small C with very deep K: K ranges x N x M
  * rounded up to 64, x 4 bytes) returns clblasOutOfResources and enqueues nothing; calls that
  * need no scratch (the large ones) have no size limit.  All calls on one GPU share the array:
- * calls in order on one stream are safe, calls that overlap in time on one GPU race. */
+ * calls in order on one stream are safe, calls that overlap in time on one GPU race.
+ * The array's device address is looked up once per GPU, by clblasSetup or by the first call on
+ * that GPU; that first call must not be made on a stream that is being captured (it returns
+ * clblasInvalidOperation then): call clblasSetup, or make one call outside a capture, first. */
 #define CLBLAS_AMD_NOALLOC_SCRATCH_BYTES (32u << 20)
 clblasStatus clblasSgemmNoAlloc(clblasOrder order, clblasTranspose transA, clblasTranspose transB,
                                 size_t M, size_t N, size_t K, float alpha,
@@ -329,23 +336,35 @@ clblasStatus clblasZhemm(clblasOrder order, clblasSide side, clblasUplo uplo, si
  * logs nothing; this library keeps scratch buffers per (device, stream) and lets the caller
  * manage them. ---- */
 
-/* Frees the scratch buffers kept for `stream` on the current device.  Call it after the stream's
- * work has completed and before destroying the stream.  Without it a process still holds a
- * bounded amount: at most 32 streams per device keep buffers, the least recently used one is
- * evicted (after a device synchronisation) when another appears. */
+/* Waits for `stream` (hipStreamSynchronize) and frees the scratch buffers kept for it on the current
+ * device.  Call it before destroying the stream.  clblasInvalidOperation, and nothing freed, if the
+ * stream is being captured.  Without it a process still holds a bounded amount: at most 32 streams per
+ * device keep buffers, the least recently used one is evicted (after a device synchronisation; none if
+ * that fails) when another appears - never one that a running call has been handed buffers of, nor
+ * one whose buffers were handed out while the stream was being captured.
+ * A HIP graph captured from calls of this library holds raw pointers into its stream's buffers: do not
+ * call this for that stream, nor clblasTeardown, while such a graph can still be launched. */
 clblasStatus clblasAmdReleaseStream(hipStream_t stream);
 
 /* Makes sure the scratch buffers of `stream` on the current device are at least this large
- * (bytes; 0 leaves a buffer alone): gemm_bytes for GEMM-shaped calls that cut K into ranges
- * (ranges x M x N elements, M rounded up to 64) or slice their last round of tiles (at most 256
- * tiles of 256 x 128 elements), trmm_bytes for TRMM's copy of B (M x N elements), trsm_bytes
- * for TRSM's packed diagonal blocks (real types: 135 168 elements per 512 rows of the triangle or
- * part thereof; complex types: 104 448 real elements per 256 rows).  A later call on the stream whose needs fit allocates nothing,
- * so it can be the first thing recorded into a HIP graph.  A call that would have to allocate
- * while its stream is being captured returns clblasInvalidOperation and leaves the capture valid. */
+ * (bytes; 0 leaves a buffer alone):
+ *   gemm_bytes  GEMM-shaped calls (every routine of this library ends in them) that cut K into
+ *               ranges (ranges x M x N elements, M rounded up to 64, at most 512 ranges) or slice
+ *               their last round of tiles (at most 256 tiles of 256 x 128 elements);
+ *   trmm_bytes  TRMM's copy of B (M x N elements, M rounded up to 64), and the full N x N product
+ *               (N rounded up to 64, times N elements) of a rank-k update - SYRK, SYR2K, HERK,
+ *               HER2K - of a small C with a deep K (N <= 704 and K >= 4096), which also takes
+ *               gemm_bytes for its K ranges;
+ *   trsm_bytes  TRSM's packed diagonal blocks (real types: 135 168 elements per 512 rows of the
+ *               triangle or part thereof; complex types: 104 448 real elements per 256 rows).
+ * A later call on the stream whose needs fit allocates nothing, so it can be the first thing recorded
+ * into a HIP graph.  A call that would have to allocate while its stream is being captured returns
+ * clblasInvalidOperation, enqueues nothing - routines made of several launches find out before the
+ * first one - and leaves the capture valid. */
 clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, size_t trmm_bytes, size_t trsm_bytes);
 
-/* Number of streams that hold scratch buffers, and the bytes of their current buffers. */
+/* Number of streams that hold scratch buffers, and the bytes of their buffers (current ones plus
+ * outgrown ones that are parked until the stream is released). */
 void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes);
 
 /* Describes the last GEMM kernel the calling thread launched (kernel family, tile, transposes,

@@ -133,6 +133,47 @@ int main() {
         EXPECT(clblasCher2k(o, clblasUpper, clblasNoTrans, 6, 0, c1, C, 0, 8, C, 0, 8, 0.f, C, 0, 8, nullptr), clblasInvalidDim);
         EXPECT(clblasZher2k(o, clblasUpper, clblasConjTrans, 6, 4, z1, Z, 0, 3, Z, 0, 8, 0.0, Z, 0, 8, nullptr), clblasInvalidLeadDimA);
     }
+    // CLBLAS_AMD_CHECK_MEM=1: the allocation behind every operand is looked up and the reference's rule
+    // (generic/common.c:644-684; src/tests/functional/func-error.cpp:58-104 makes a matrix larger than its
+    // buffer and expects clblasInsufficientMemMatA / MatB) applies: offset + footprint beyond the buffer.
+    // The lookup is replaced by a table: F holds 64 floats, D2 64 doubles, anything else is unknown.
+    setenv("CLBLAS_AMD_CHECK_MEM", "1", 1);
+    clblasAmdReloadDebugEnv();
+    double *D2 = reinterpret_cast<double *>(0x3000);  // (F and D2 above are one address)
+    static const void *known_f = F, *known_d = D2;
+    cba::set_mem_probe([](const void *ptr) -> size_t {
+        if (ptr == known_f) return 64 * sizeof(float);
+        if (ptr == known_d) return 64 * sizeof(double);
+        return 0;
+    });
+    float *G = reinterpret_cast<float *>(0x2000);  // no allocation holds it
+    for (clblasOrder o : orders)
+        for (clblasTranspose ta : transes)
+            for (clblasTranspose tb : transes) {
+                // 9 x 8 elements with ld 9 need 72 > 64; 8 x 8 fits exactly until an offset of one pushes it out
+                EXPECT(clblasSgemm(o, ta, tb, 9, 8, 8, 1.f, F, 0, 9, F, 0, 9, 0.f, F, 0, 9, nullptr), clblasInsufficientMemMatA);
+                EXPECT(clblasSgemm(o, ta, tb, 8, 8, 8, 1.f, F, 1, 8, F, 0, 8, 0.f, F, 0, 8, nullptr), clblasInsufficientMemMatA);
+                EXPECT(clblasSgemm(o, ta, tb, 8, 8, 8, 1.f, F, 0, 8, F, 1, 8, 0.f, F, 0, 8, nullptr), clblasInsufficientMemMatB);
+                EXPECT(clblasDgemm(o, ta, tb, 8, 8, 8, 1.0, D2, 0, 8, D2, 0, 8, 0.0, D2, 1, 8, nullptr), clblasInsufficientMemMatC);
+                // a padded leading dimension counts up to the last element only: (7 - 1) 9 + 8 = 62 fits, + 3 does not
+                EXPECT(clblasDgemm(o, ta, tb, 7, 7, 7, 1.0, D2, 0, 9, D2, 0, 9, 0.0, D2, 7, 9, nullptr), clblasInsufficientMemMatC);
+                // the order of the checks is unchanged: leading dimension of A before the memory of B
+                EXPECT(clblasSgemm(o, ta, tb, 8, 8, 8, 1.f, F, 0, 7, F, 9, 8, 0.f, F, 0, 8, nullptr), clblasInvalidLeadDimA);
+                // a pointer that no allocation holds is no matrix at all
+                EXPECT(clblasSgemm(o, ta, tb, 8, 8, 8, 1.f, F, 0, 8, G, 0, 8, 0.f, F, 0, 8, nullptr), clblasInvalidMatB);
+                // an offset that wraps round 64 bits does not pass for a small one
+                EXPECT(clblasSgemm(o, ta, tb, 8, 8, 8, 1.f, F, (size_t)-60, 8, F, 0, 8, 0.f, F, 0, 8, nullptr), clblasInsufficientMemMatA);
+            }
+    for (clblasOrder o : orders) {
+        EXPECT(clblasStrsm(o, clblasLeft, clblasLower, clblasNoTrans, clblasNonUnit, 9, 4, 1.f, F, 0, 9, F, 0, 9, nullptr), clblasInsufficientMemMatA);
+        EXPECT(clblasDtrsm(o, clblasRight, clblasUpper, clblasTrans, clblasUnit, 4, 8, 1.0, D2, 0, 8, D2, 40, 8, nullptr), clblasInsufficientMemMatB);
+        EXPECT(clblasSsyrk(o, clblasLower, clblasNoTrans, 8, 8, 1.f, F, 0, 8, 0.f, F, 2, 8, nullptr), clblasInsufficientMemMatC);
+        EXPECT(clblasDtrmm(o, clblasLeft, clblasLower, clblasNoTrans, clblasNonUnit, 8, 8, 1.0, D2, 0, 8, D2, 1, 8, nullptr), clblasInsufficientMemMatB);
+        EXPECT(clblasSsymm(o, clblasLeft, clblasLower, 8, 8, 1.f, F, 1, 8, F, 0, 8, 0.f, F, 0, 8, nullptr), clblasInsufficientMemMatA);
+    }
+    cba::set_mem_probe(nullptr);
+    unsetenv("CLBLAS_AMD_CHECK_MEM");
+    clblasAmdReloadDebugEnv();
     clblasTeardown();
     if (failures) { std::printf("%d failures\n", failures); return 1; }
     std::puts("ok");

@@ -25,7 +25,8 @@ static void t_release(int, void *p) {
     live_bytes -= sizes[p];
     std::free(p);
 }
-static void t_sync(int) { ++syncs; }
+static bool sync_ok = true;
+static bool t_sync(int) { ++syncs; return sync_ok; }
 
 #define CHECK(c) do { if (!(c)) { std::printf("FAILED line %d: %s\n", __LINE__, #c); return 1; } } while (0)
 
@@ -82,8 +83,46 @@ int main() {
         CHECK(c.get(0, keep, WS_TRMM, (size_t)64 << 20, true, &err));  // 1.5 x 60 MiB refused, 64 MiB fits
         CHECK(c.get(0, keep, WS_TRMM, (size_t)65 << 20, true, &err) == nullptr && err == WS_NO_MEMORY);
         fail_big = false;
-        c.release_all();
+        const size_t syncs_before = syncs;
+        CHECK(c.release_all());
+        CHECK(syncs == syncs_before + 2);  // once per device that held buffers
         CHECK(live.empty() && live_bytes == 0 && c.stream_count() == 0);
+    }
+    {
+        // outgrown buffers count in the statistics until they are freed
+        WorkspaceCache c(a, 4);
+        WorkspaceError err;
+        const void *s1 = (const void *)0x10;
+        CHECK(c.get(0, s1, WS_GEMM, (size_t)2 << 20, true, &err));
+        CHECK(c.get(0, s1, WS_GEMM, (size_t)8 << 20, true, &err));
+        CHECK(c.bytes_held() == ((size_t)2 << 20) + ((size_t)8 << 20) && c.allocations() == 2);
+        CHECK(c.release_all() && live.empty());
+    }
+    {
+        // leases and pins keep an entry from eviction; a failed synchronisation evicts nothing
+        WorkspaceCache c(a, 2);
+        WorkspaceError err;
+        const void *s1 = (const void *)0x10, *s2 = (const void *)0x20, *s3 = (const void *)0x30, *s4 = (const void *)0x40;
+        void *p1 = c.get(0, s1, WS_GEMM, 10, true, &err);
+        CHECK(!c.lease(0, s3));                       // no entry: nothing to hold
+        CHECK(c.lease(0, s1));
+        void *p2 = c.get(0, s2, WS_GEMM, 10, true, &err);
+        CHECK(p1 && p2);
+        CHECK(c.get(0, s3, WS_GEMM, 10, true, &err));  // s1 is the oldest but leased: s2 goes
+        CHECK(c.get(0, s1, WS_GEMM, 10, false, &err) == p1);
+        CHECK(c.get(0, s2, WS_GEMM, 10, false, &err) == nullptr);
+        c.unlease(0, s1);
+        c.pin(0, s1);
+        CHECK(c.pinned(0, s1) && !c.pinned(0, s3));
+        CHECK(c.get(0, s4, WS_GEMM, 10, true, &err));  // s1 pinned: s3 goes
+        CHECK(c.get(0, s1, WS_GEMM, 10, false, &err) == p1);
+        CHECK(c.get(0, s3, WS_GEMM, 10, false, &err) == nullptr);
+        sync_ok = false;
+        CHECK(c.get(0, s2, WS_GEMM, 10, true, &err));  // cannot synchronise: nobody is evicted, the quota is exceeded
+        CHECK(c.stream_count() == 3);
+        CHECK(!c.release_all() && c.stream_count() == 3);
+        sync_ok = true;
+        CHECK(c.release_all() && live.empty() && c.stream_count() == 0);
     }
     std::puts("ok");
     return 0;

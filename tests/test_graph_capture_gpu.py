@@ -37,7 +37,9 @@ def test_calls_replay_from_a_hip_graph():
     # STRMM 300 x 200 and SSYRK 300 x 64
     ma, mb = dev(oracle.uniform(300 * 300, 9, f32)), dev(oracle.uniform(300 * 200, 10, f32))
     sa, sc = dev(oracle.uniform(300 * 64, 11, f32)), dev(oracle.uniform(300 * 300, 12, f32))
-    ins = [c1, c2, tb, mb, sc]
+    # SSYRK 200 x 8192: a small C with a deep K runs as a K-split GEMM into a library buffer + a triangle pass
+    da, dc = dev(oracle.uniform(200 * 8192, 13, f32)), dev(oracle.uniform(200 * 200, 14, f32))
+    ins = [c1, c2, tb, mb, sc, dc]
     keep = [x.clone() for x in ins]
 
     def sequence():
@@ -47,8 +49,9 @@ def test_calls_replay_from_a_hip_graph():
                clblas_amd.dgemm(COL, NOTRANS, TRANS, 1100, 1000, 520, 0.75, a2, 0, 1100, b2, 0, 1000, 0.5, c2, 0, 1100),
                clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, 300, 2.0, ta, 0, n, tb, 0, n),
                clblas_amd.trmm("S", COL, LEFT, LOWER, NOTRANS, NONUNIT, 300, 200, 1.5, ma, 0, 300, mb, 0, 300),
-               clblas_amd.syrk("S", COL, LOWER, NOTRANS, 300, 64, 1.0, sa, 0, 300, 0.5, sc, 0, 300)]
-        assert sts == [0] * 5, sts
+               clblas_amd.syrk("S", COL, LOWER, NOTRANS, 300, 64, 1.0, sa, 0, 300, 0.5, sc, 0, 300),
+               clblas_amd.syrk("S", COL, LOWER, NOTRANS, 200, 8192, 0.25, da, 0, 200, 0.5, dc, 0, 200)]
+        assert sts == [0] * 6, sts
 
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -149,3 +152,74 @@ def test_capture_needs_buffers_that_exist_and_reserve_provides_them():
     # 3. releasing the stream gives its buffers back
     assert clblas_amd.release_stream(stream.cuda_stream) == 0
     assert clblas_amd.workspace_stats()[0] == streams_before
+
+
+def test_a_routine_of_several_launches_is_refused_before_its_first_launch():
+    """DTRSM under capture with its packing buffer reserved but not the buffer its update GEMMs cut K
+    into: the call must find that out before the packing pass and the first leaves - which overwrite B
+    in place - are enqueued.  It returns clblasInvalidOperation, the capture stays usable and a replay
+    leaves B as it was.  The same for a deep rank-k update (a GEMM into a library buffer followed by a
+    triangle pass) with only one of its two buffers reserved."""
+    import torch
+    import clblas_amd
+    assert clblas_amd.setup() == 0
+    INVALID_OPERATION = -59
+    f32, f64 = np.float32, np.float64
+
+    def dev(x):
+        return torch.from_numpy(x).cuda()
+
+    n, nrhs = 1100, 100     # leaves of 512, 512, 76 rows; the last update is 76 x 100 x 1024: few tiles, deep K
+    ta, tb = dev(oracle.triangular(n, n, True, 7, f64)), dev(oracle.uniform(n * nrhs, 8, f64))
+    tb_keep = tb.clone()
+    da, dc = dev(oracle.uniform(200 * 8192, 13, f32)), dev(oracle.uniform(200 * 200, 14, f32))
+    dc_keep = dc.clone()
+    probe = torch.zeros(16, device="cuda")
+
+    def trsm():
+        return clblas_amd.dtrsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, nrhs, 2.0, ta, 0, n, tb, 0, n)
+
+    def deep_syrk():
+        return clblas_amd.syrk("S", COL, LOWER, NOTRANS, 200, 8192, 0.25, da, 0, 200, 0.5, dc, 0, 200)
+
+    # eager, on the default stream: what the calls compute, and that they do ask for a GEMM buffer
+    assert trsm() == 0 and deep_syrk() == 0
+    torch.cuda.synchronize()
+    want_tb, want_dc = tb.clone(), dc.clone()
+    assert not torch.equal(want_tb, tb_keep)
+    tb.copy_(tb_keep); dc.copy_(dc_keep)
+
+    stream = torch.cuda.Stream()
+    assert clblas_amd.reserve_workspace(0, 1 << 20, 4 << 20, stream=stream.cuda_stream) == 0   # no GEMM buffer
+    stats = clblas_amd.workspace_stats()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        st_trsm = trsm()
+        st_syrk = deep_syrk()
+        probe.add_(1.0)          # the capture is still alive after the refusals
+    assert st_trsm == INVALID_OPERATION, st_trsm
+    assert st_syrk == INVALID_OPERATION, st_syrk
+    assert clblas_amd.workspace_stats() == stats
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(tb, tb_keep), "the refused DTRSM must not have touched B"
+    assert torch.equal(dc, dc_keep), "the refused SYRK must not have touched C"
+    assert float(probe[0]) == 1.0
+    del graph
+
+    # with the missing buffer reserved the same capture goes through and replays to the eager results
+    assert clblas_amd.reserve_workspace(8 << 20, 0, 0, stream=stream.cuda_stream) == 0
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        sts = [trsm(), deep_syrk()]
+    assert sts == [0, 0], sts
+    for _ in range(2):
+        tb.copy_(tb_keep); dc.copy_(dc_keep)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(tb, want_tb) and torch.equal(dc, want_dc)
+    del graph
+    assert clblas_amd.release_stream(stream.cuda_stream) == 0

@@ -102,10 +102,13 @@ def test_noalloc_can_be_the_first_thing_in_a_graph():
     torch.cuda.synchronize()
     s = torch.cuda.Stream()
     g = torch.cuda.CUDAGraph()
+    stats = clblas_amd.workspace_stats()
     with torch.cuda.stream(s):
         with torch.cuda.graph(g, stream=s):
             st = clblas_amd.sgemm_noalloc(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 0.0, C, 0, M, stream=s)
     assert st == 0
+    assert "splits=1 " not in clblas_amd.last_dispatch()[0] + " ", "the case is meant to use the scratch array"
+    assert clblas_amd.workspace_stats() == stats, "the entry point must not touch the per-stream buffers"
     for _ in range(3):
         C.fill_(-1.0)
         g.replay()
