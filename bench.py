@@ -641,11 +641,11 @@ def main():
             B = gen_uniform(torch, offs[1] + ldb * cb, seed + 1, torch.float32)
             C = gen_uniform(torch, offs[2] + ldc * N, seed + 2, torch.float32)
 
+            bound = clblas_amd.bind("clblasSgemm", COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc)
+
             def call():
-                st = clblas_amd.sgemm(COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2],
-                                      ldc)
-                if st != 0:
-                    raise RuntimeError("clblasSgemm returned %d" % st)
+                if bound() != 0:
+                    raise RuntimeError("clblasSgemm failed")
             return timed_batch(torch, call, 20 if 2.0 * M * N * K > 1e10 else 100, 5)
 
         ms = sgemm_case(1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0), SEEDS["sgemm_config1"])
@@ -706,11 +706,13 @@ def main():
                 A.diagonal().copy_(torch.rand(m, device="cuda", dtype=dt, generator=gen) + 1)
                 B = torch.rand(m, m, device="cuda", dtype=dt, generator=gen)
 
+                # (arguments converted once: at 512 the Python wrapper's share of a call would be a third of it)
+                bound = clblas_amd.bind("clblas" + name.capitalize(), COL, LEFT, LOWER, NOTRANS, NONUNIT, m, m, 1.0, A, 0, m, B, 0, m)
+
                 def call():
-                    st = fn(COL, LEFT, LOWER, NOTRANS, NONUNIT, m, m, 1.0, A, 0, m, B, 0, m)
-                    if st != 0:
-                        raise RuntimeError("clblas %s returned %d" % (name, st))
-                ms = timed_batch(torch, call, 20, 3)
+                    if bound() != 0:
+                        raise RuntimeError("clblas %s failed" % name)
+                ms = timed_batch(torch, call, 50, 5)
                 launches = clblas_amd.last_dispatch()[1]
                 call()
                 launches = clblas_amd.last_dispatch()[1] - launches

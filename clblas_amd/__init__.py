@@ -79,7 +79,7 @@ EXPORTED_SYMBOLS = (
 ) + tuple("clblas%s%s" % (t, f) for f in ("syrk", "trmm", "symm", "syr2k") for t in "SDCZ") + tuple(
     "clblas%s%s" % (t, f) for f in ("herk", "her2k", "hemm") for t in "CZ") + (
     "clblasAmdReleaseStream", "clblasAmdReserveWorkspace", "clblasAmdWorkspaceStats", "clblasAmdLastDispatch",
-    "clblasAmdReloadDebugEnv")
+    "clblasAmdReloadDebugEnv", "clblasAmdTrsmPollTimeouts")
 
 _lib = None
 
@@ -153,6 +153,8 @@ def _declare(lib):
     lib.clblasAmdLastDispatch.argtypes = [ctypes.c_char_p, sz]
     lib.clblasAmdReloadDebugEnv.restype = None
     lib.clblasAmdReloadDebugEnv.argtypes = []
+    lib.clblasAmdTrsmPollTimeouts.restype = ctypes.c_int
+    lib.clblasAmdTrsmPollTimeouts.argtypes = [ctypes.POINTER(ctypes.c_uint), ctypes.c_int]
 
 
 def load_library(path=None):
@@ -189,6 +191,31 @@ def _stream(stream):
     return ctypes.c_void_p(stream.cuda_stream)
 
 
+def bind(symbol, *args, stream=None):
+    """A zero-argument callable that makes the call `symbol(*args, stream)` - e.g.
+    bind("clblasDtrsm", order, side, uplo, trans, diag, M, N, alpha, A, offA, lda, B, offB, ldb) -
+    with the arguments converted to their C types once.  For loops in which the microseconds the
+    wrappers above spend per call (tensor addresses, torch's current stream) would be measured
+    along with the library: benchmarks of small problems.  Tensors must stay alive and in place
+    for as long as the callable is used."""
+    fn = getattr(load_library(), symbol)
+    types = fn.argtypes
+    if len(args) + 1 != len(types):
+        raise TypeError("%s takes %d arguments and a stream" % (symbol, len(types) - 1))
+    conv = []
+    for a, t in zip(args, types):
+        if t is ctypes.c_void_p:
+            conv.append(_ptr(a))
+        elif t in (FloatComplex, DoubleComplex):
+            z = complex(a)
+            conv.append(t(z.real, z.imag))
+        else:
+            conv.append(t(a))
+    conv.append(_stream(stream))
+    conv = tuple(conv)
+    return lambda: fn(*conv)
+
+
 def setup():
     return load_library().clblasSetup()
 
@@ -211,6 +238,16 @@ def workspace_stats():
     a, b = ctypes.c_size_t(), ctypes.c_size_t()
     load_library().clblasAmdWorkspaceStats(ctypes.byref(a), ctypes.byref(b))
     return a.value, b.value
+
+
+def trsm_poll_timeouts(reset=False):
+    """Flag waits of the TRSM substitution leaf that gave up at their poll limit on the current GPU (0 for
+    a working library); blocks until the device is idle enough to be read."""
+    n = ctypes.c_uint(0)
+    st = load_library().clblasAmdTrsmPollTimeouts(ctypes.byref(n), 1 if reset else 0)
+    if st != 0:
+        raise RuntimeError("clblasAmdTrsmPollTimeouts returned %d" % st)
+    return n.value
 
 
 def last_dispatch():

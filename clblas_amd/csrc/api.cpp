@@ -50,6 +50,8 @@ void read_knobs() {
     k.wide_ld = env_int("CLBLAS_AMD_GEMM_WIDE_LD", 0);
     k.log = env_int("CLBLAS_AMD_LOG", 0);
     k.check_mem = env_int("CLBLAS_AMD_CHECK_MEM", 0);
+    k.trsm_leaf = env_int("CLBLAS_AMD_TRSM_LEAF", 0);
+    k.trsm_poll_limit = env_int("CLBLAS_AMD_TRSM_POLL_LIMIT", 0);
     g_knobs = k;
 }
 }  // namespace
@@ -619,6 +621,10 @@ clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, si
 }
 
 void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes) { cba::ws_stats(streams, bytes); }
+
+clblasStatus clblasAmdTrsmPollTimeouts(unsigned int *count, int reset) {
+    return map_hip_error(cba::trsm_poll_timeouts_read(count, reset != 0));
+}
 
 clblasStatus clblasSgemm(clblasOrder order, clblasTranspose transA, clblasTranspose transB, size_t M, size_t N,
                          size_t K, float alpha, const float *A, size_t offA, size_t lda, const float *B, size_t offB,

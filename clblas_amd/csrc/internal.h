@@ -52,6 +52,8 @@ template <typename R> struct Cx { R re, im; };
 struct DebugKnobs {
     int gemm_tile = -1, split_model = 1, splits = 0, tail = 1, group_m = 0, xcd = 1, stagger = 1, log = 0;
     int check_mem = 0;
+    int trsm_poll_limit = 0;  // CLBLAS_AMD_TRSM_POLL_LIMIT: polls after which a flag wait of the substitution leaf gives up (0: 2^22); tests
+    int trsm_leaf = 0;     // CLBLAS_AMD_TRSM_LEAF (real types): 0 substitution over 16-row sub-blocks, 1 inverted 64 x 64 triangles
     int wide_ld = 0;       // CLBLAS_AMD_GEMM_WIDE_LD=1: the wide-ld kernels whatever the leading dimensions (tests)
     int deep_panels = 1;   // CLBLAS_AMD_GEMM_DEEP: 0 never the deep-panel variant of a tile, 1 by the rule, 2 wherever built, more: from that depth of a K range
 };
@@ -197,6 +199,10 @@ hipError_t hemm_colmajor(bool right, bool lower, int M, int N, T alpha, const T 
 template <typename T>
 hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool conj, bool unit, int M, int N, T alpha, const T *A,
                          int64_t lda, T *B, int64_t ldb, hipStream_t stream);
+
+// Flag waits of the TRSM leaf that ran into their poll limit on the current GPU (trsm.hip); waits for
+// the device's copy queue, so not for use between enqueues of a benchmark.
+hipError_t trsm_poll_timeouts_read(unsigned int *count, bool reset);
 
 template <typename F> hipError_t with_workspaces_secured(hipStream_t stream, F &&body) {
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;

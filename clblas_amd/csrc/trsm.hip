@@ -227,10 +227,16 @@ trsm_pack_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool co
 
 template <int N> struct IntC { static constexpr int value = N; };
 
+// Number of flag waits of trsm_diag_kernel that gave up at their poll limit since the library was
+// loaded (per GPU).  A wait that gives up lets its wavefront go on with whatever the slot holds - a
+// wrong result instead of a hang - so this counter staying at zero is what says that no result
+// was ever produced that way.  Only touched on that path; read by clblasAmdTrsmPollTimeouts.
+__device__ unsigned int trsm_poll_timeouts = 0;
+
 template <typename T, bool RIGHT, bool FORWARD, bool WIDE>
 __global__ void __launch_bounds__(TrsmLeaf<T>::THREADS)
 trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk,
-                 int64_t ldb, int nrhs) {
+                 int64_t ldb, int nrhs, int poll_limit) {
     typedef TrsmLeaf<T, RIGHT, WIDE> L;
     typedef typename Elem<T>::Real R;
     typedef Mma16<R> M;
@@ -444,7 +450,8 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
         if (lane == 0) __hip_atomic_store(published + s, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     };
     auto wait_for = [&](int s, bool urgent) {
-        for (int polls = 0; polls < (1 << 22); ++polls) {
+        int polls = 0;
+        for (; polls < poll_limit; ++polls) {
             // (an atomic load: a plain one may be hoisted out of the loop, a volatile one is compiled as
             // a flat access, which also waits for every outstanding global load)
             if (__builtin_amdgcn_readfirstlane(
@@ -452,6 +459,7 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
                 break;
             if (!urgent) __builtin_amdgcn_s_sleep(1);
         }
+        if (polls >= poll_limit && lane == 0) atomicAdd(&trsm_poll_timeouts, 1u);
         asm volatile("" ::: "memory");  // (compiler only) the X_s loads stay behind the flag load
     };
     // Row block h of this wavefront: updates with X_0 .. X_(row-1), then X_row = inv(L_row,row) Y.
@@ -593,6 +601,442 @@ trsm_diag_kernel(const typename Elem<T>::Real *__restrict__ packed, int nb, T al
     static_assert(RW <= 2, "one run_row call per row block");
 }
 
+// ---------------------------------------------------------------------------------------------
+// Real types: diagonal blocks of 512 x 512 solved with explicitly inverted 64 x 64 triangles.
+//
+// The reference inverts its diagonal blocks by doubling - 16 x 16 triangles by substitution, then
+// inv21 = -inv22 (A21 inv11) for 32, 64 and 128 (trtri/diag_dtrtri_lower_128_16.cpp:60-160,
+// trtri/triple_dgemm_update_128_16_PART1_L.cpp:44-160, ..._32_PART1_L.cpp, ..._64_PART1_L.cpp) - and
+// multiplies by the inverses.  The same here up to 64 x 64 ("super-blocks" of four sub-block rows):
+// the packing pass files, for sub-block row r = 4S + i, the sub-blocks -L(r, q) for q < 4S and the
+// sub-blocks Inv_S(i, j), j <= i, of the inverted triangle at q = 4S + j - one uniform row of
+// MFMA "A" operands - and the solve of a diagonal block is eight steps
+//     X_S = Inv_S Y_S ;   Y_r += (-L(r, 4S..4S+3)) X_S   for every sub-block row r beyond S.
+// Substitution over 16-row sub-blocks needs 32 dependent steps whose latencies (flag, X out of LDS, four
+// dependent MFMAs, X into LDS) do not overlap with the bulk of the MFMA work; with the inverses the
+// serial part of a step is one product per owner and everything else is work for all sixteen
+// wavefronts between two barriers.
+//
+// Workgroup: one diagonal block x 16 NBK right-hand sides, 16 wavefronts, wavefront w owning sub-block
+// rows w and w + 16 (accumulators, as above); super-block S is owned by four consecutive
+// wavefronts, one per SIMD.  Step S:
+//   A  the four owners: X_r = sum_{j<=i} Inv_S(i, j) Y_(4S+j), the Y of the other owners out of LDS
+//      (written at the end of the step before); X_r to LDS and to memory.           barrier
+//   B  every wavefront, each row beyond S it owns: four products with the X of S; then the row's
+//      coefficients of the next step are requested; owners of S + 1 file their Y.      barrier
+// The schedule is fixed, so results are reproducible bit for bit.
+template <typename R> struct TrsmBlock {
+    static constexpr int IB = 16, WAVES = 8, RW = 4, NB = WAVES * IB * RW, NBLK = NB / IB;
+    static constexpr int SBR = 4, SB = SBR * IB, NS = NB / SB;  // sub-block rows per super-block, its order, super-blocks
+    static constexpr int THREADS = 64 * WAVES;
+    static constexpr int SUB_REALS = IB * IB;
+    static constexpr int N_EBLK = NBLK * (NBLK + 1) / 2;
+    static constexpr int PACK_REALS = N_EBLK * SUB_REALS;
+    static constexpr int PACK_CHUNK = 8;                        // sub-blocks per copying workgroup of the packing pass
+    static constexpr int COPY_GROUPS = NBLK * (NBLK / PACK_CHUNK);
+    typedef double Work;                                        // the inversion runs in FP64 for both types
+    static constexpr size_t PACK_SMEM = (size_t)(2 * SB * SB + SB) * sizeof(Work);
+};
+
+// Packing pass of the above.  blockIdx.y: diagonal block.  blockIdx.x < COPY_GROUPS: workgroup
+// (bi, chunk) negates and files up to PACK_CHUNK sub-blocks (bi, bj), bj < 4 (bi / 4), of sub-block row bi;
+// blockIdx.x >= COPY_GROUPS: super-block S = blockIdx.x - COPY_GROUPS is inverted and its ten sub-blocks filed.
+// Only the referenced triangle is read, and no diagonal when `unit`; rows past the end of a short
+// block count as rows of the identity.
+template <typename T, bool FORWARD>
+__global__ void __launch_bounds__(256)
+trsm_pack_inv_kernel(const T *__restrict__ A, int64_t lda, int n, bool teff, bool unit, T *__restrict__ pack) {
+    typedef TrsmBlock<T> L;
+    typedef Mma16<T> M;
+    typedef typename L::Work W;
+    constexpr int IB = L::IB, SB = L::SB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pack_smem[];
+    const int tid = threadIdx.x;
+    const int i0 = blockIdx.y * L::NB;
+    const int nb = n - i0 < L::NB ? n - i0 : L::NB;
+    const T *Ablk = A + i0 + (int64_t)i0 * lda;
+    T *out_blk = pack + (int64_t)blockIdx.y * L::PACK_REALS;
+    auto coef = [&](int P, int Q) -> T {  // Q <= P < nb
+        const int ip = FORWARD ? P : nb - 1 - P, iq = FORWARD ? Q : nb - 1 - Q;
+        return teff ? Ablk[iq + (int64_t)ip * lda] : Ablk[ip + (int64_t)iq * lda];
+    };
+    if ((int)blockIdx.x < L::COPY_GROUPS) {
+        constexpr int CHUNKS = L::NBLK / L::PACK_CHUNK;
+        const int bi = blockIdx.x / CHUNKS, chunk = blockIdx.x % CHUNKS;
+        if (bi * IB >= nb) return;
+        const int below = (bi / L::SBR) * L::SBR;  // sub-block columns left of the row's super-block
+        const int bj_lo = chunk * L::PACK_CHUNK;
+        const int bj_hi = bj_lo + L::PACK_CHUNK < below ? bj_lo + L::PACK_CHUNK : below;
+        T *out = out_blk + (int64_t)(bi * (bi + 1) / 2) * L::SUB_REALS;
+        for (int e = bj_lo * IB * IB + tid; e < bj_hi * IB * IB; e += 256) {
+            const int bj = e / (IB * IB), w = e % (IB * IB);
+            const int lane = w / 4, c = w % 4;
+            const int P = bi * IB + M::arow(lane % 16), Q = bj * IB + M::krow(lane / 16, c);
+            out[bj * L::SUB_REALS + packed_at<T>(lane, c)] = (P < nb) ? -coef(P, Q) : (T)0;
+        }
+        return;
+    }
+    const int sb = blockIdx.x - L::COPY_GROUPS;
+    const int P0 = sb * SB;
+    if (P0 >= nb) return;
+    W(*Ls)[SB] = reinterpret_cast<W(*)[SB]>(pack_smem);                       // the triangle, later A21 inv11
+    W(*Iv)[SB] = reinterpret_cast<W(*)[SB]>(pack_smem + sizeof(W) * SB * SB);  // its inverse
+    W *Rd = reinterpret_cast<W *>(pack_smem + 2 * sizeof(W) * SB * SB);        // reciprocals of the diagonal
+    for (int e = tid; e < SB * SB; e += 256) {
+        const int p = e / SB, q = e % SB;
+        const int P = P0 + p, Q = P0 + q;
+        W v = 0;
+        if (p == q) v = (unit || P >= nb) ? (W)1 : (W)coef(P, P);
+        else if (q < p && P < nb) v = (W)coef(P, Q);
+        Ls[p][q] = v;
+        Iv[p][q] = 0;
+    }
+    __syncthreads();
+    if (tid < SB) Rd[tid] = (W)1 / Ls[tid][tid];
+    __syncthreads();
+    // the four 16 x 16 triangles on the diagonal, by substitution: thread (d, zc) solves L_dd z = e_zc
+    if (tid < SB) {
+        const int d = tid / IB, zc = tid % IB, o = d * IB;
+        W z[IB];
+#pragma unroll
+        for (int p = 0; p < IB; ++p) {
+            W acc = (p == zc) ? (W)1 : (W)0;
+#pragma unroll
+            for (int q = 0; q < IB; ++q)
+                if (q < p) acc -= Ls[o + p][o + q] * z[q];
+            z[p] = (p < zc) ? (W)0 : acc * Rd[o + p];
+        }
+#pragma unroll
+        for (int p = 0; p < IB; ++p) Iv[o + p][o + zc] = z[p];
+    }
+    __syncthreads();
+    // doubling: with inv11 (h x h at offset c0) and inv22 (h x h at c0 + h) known,
+    //   T = A21 inv11 (into the place of A21), then inv21 = -inv22 T.
+    // (The sums run over all h terms - the triangular factors hold their zeros - so that the loops
+    // have fixed lengths and their LDS reads are issued back to back.)
+    auto level = [&](auto hc) {
+        constexpr int h = decltype(hc)::value;
+        constexpr int PER = h / 8;  // all the A21 of one level: SB / (2h) pairs of h x h elements, h / 8 per thread
+        W t[PER];
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int o = tid + 256 * u;
+            const int pr = o / (h * h), i = (o % (h * h)) / h, j = o % h;
+            const int c0 = pr * 2 * h, r0 = c0 + h;
+            W acc = 0;
+#pragma unroll
+            for (int k = 0; k < h; ++k) acc += Ls[r0 + i][c0 + k] * Iv[c0 + k][c0 + j];
+            t[u] = acc;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int o = tid + 256 * u;
+            const int pr = o / (h * h), i = (o % (h * h)) / h, j = o % h;
+            Ls[pr * 2 * h + h + i][pr * 2 * h + j] = t[u];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int o = tid + 256 * u;
+            const int pr = o / (h * h), i = (o % (h * h)) / h, j = o % h;
+            const int c0 = pr * 2 * h, r0 = c0 + h;
+            W acc = 0;
+#pragma unroll
+            for (int k = 0; k < h; ++k) acc += Iv[r0 + i][r0 + k] * Ls[r0 + k][c0 + j];
+            t[u] = -acc;
+        }
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int o = tid + 256 * u;
+            const int pr = o / (h * h), i = (o % (h * h)) / h, j = o % h;
+            Iv[pr * 2 * h + h + i][pr * 2 * h + j] = t[u];
+        }
+        __syncthreads();
+    };
+    level(IntC<16>{});
+    level(IntC<32>{});
+    static_assert(SB == 64, "two doubling levels");
+    // the ten sub-blocks (4 sb + i, 4 sb + j), j <= i, in MFMA operand order
+    for (int o = tid; o < 10 * IB * IB; o += 256) {
+        const int blk = o / (IB * IB), w = o % (IB * IB);
+        const int i = blk < 1 ? 0 : blk < 3 ? 1 : blk < 6 ? 2 : 3, j = blk - i * (i + 1) / 2;
+        const int lane = w / 4, c = w % 4;
+        const int r = sb * L::SBR + i, q = sb * L::SBR + j;
+        out_blk[(int64_t)(r * (r + 1) / 2 + q) * L::SUB_REALS + packed_at<T>(lane, c)] =
+            (T)Iv[i * IB + M::arow(lane % 16)][j * IB + M::krow(lane / 16, c)];
+    }
+}
+
+template <typename T, bool RIGHT, bool FORWARD, int NBK>
+__global__ void __launch_bounds__(TrsmBlock<T>::THREADS)
+trsm_block_kernel(const T *__restrict__ packed, int nb, T alpha, T *__restrict__ Bblk, int64_t ldb, int nrhs) {
+    typedef TrsmBlock<T> L;
+    typedef T R;
+    typedef Mma16<R> M;
+    typedef typename M::Acc Acc;
+    constexpr int IB = L::IB, WAVES = L::WAVES, RW = L::RW, SBR = L::SBR, NS = L::NS, CW = 16 * NBK;
+    static_assert(WAVES == 2 * SBR && RW * WAVES * IB == L::NB, "two sets of SBR owners, RW rows each");
+    constexpr int V = 16 / (int)sizeof(R);  // reals per 16 bytes
+    constexpr int CH = 4 / V;               // 16-byte pieces of an accumulator block
+    typedef R VT __attribute__((ext_vector_type(V)));
+    // LDS: X of the last two steps (step S in half S % 2) and the Y that the owners of the coming step
+    // exchange; one accumulator block per (sub-block row of the super-block, block of 16 right-hand
+    // sides), in per-lane order.
+    __shared__ __attribute__((aligned(16))) R Xb[2][SBR * NBK * 256];
+    __shared__ __attribute__((aligned(16))) R Yb[SBR * NBK * 256];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int own_i = wave % SBR;  // the wavefront owns row own_i of the super-blocks SET, SET + 2, ... (SET = wave / SBR)
+    const int g = lane >> 4, jj = lane & 15;
+    const int64_t j0 = (int64_t)blockIdx.x * CW;
+    const int nsteps = (nb + IB - 1) / IB;        // sub-block rows that exist
+    const int nsuper = (nb + L::SB - 1) / L::SB;  // super-blocks that exist
+
+    // The two sets of owners run different programs (their turns alternate), each in straight-line code:
+    // the body is instantiated per set and a wavefront enters the one of its set.  Both instances execute
+    // the same number of barriers.
+    auto body = [&](auto setc) __attribute__((always_inline)) {
+        constexpr int SET = decltype(setc)::value;
+        // Row h of this wavefront: sub-block row (2h + set) SBR + own_i.  Its packed sub-blocks are consecutive.
+        auto row_of = [&](int h) __attribute__((always_inline)) { return (2 * h + SET) * SBR + own_i; };
+        // (Addresses are kept as a wavefront-uniform pointer plus a 32-bit lane offset, so that they live in
+        // scalar registers.)
+        const uint32_t lane_off = (uint32_t)lane * V;
+        // Sub-blocks first .. first + 3 of row h (clamped to the row's own sub-blocks) into four register blocks.
+        auto fetch4 = [&](int h, int first, R (&dst)[SBR][4]) __attribute__((always_inline)) {
+            const int row = row_of(h);
+            const R *rowp = packed + (int64_t)(row * (row + 1) / 2) * L::SUB_REALS;
+    #pragma unroll
+            for (int q = 0; q < SBR; ++q) {
+                int sidx = first + q;
+                sidx = sidx < 0 ? 0 : (sidx < row ? sidx : row);
+                const R *src = rowp + sidx * L::SUB_REALS;
+    #pragma unroll
+                for (int c = 0; c < 4; c += V) {
+                    const VT t = *reinterpret_cast<const VT *>(src + (c / V) * (64 * V) + lane_off);
+    #pragma unroll
+                    for (int x = 0; x < V; ++x) dst[q][c + x] = t[x];
+                }
+            }
+        };
+        // Coefficients in flight: for the wavefront's next turn as an owner the sub-blocks of its near update
+        // (ecn) and of the inverse (eca); for its far updates one step's sub-blocks of the rows 1 .. 3 (row 0 of a
+        // wavefront lies in super-block 0 or 1 and takes no far update).
+        // FP64 has no registers for both sets of the owner's sub-blocks: there the inverse is requested into
+        // the near update's registers as soon as that update's MFMAs are issued.
+        constexpr bool TWO_CRIT = sizeof(R) == 4;
+        R ecn[SBR][4], eca_own[TWO_CRIT ? SBR : 1][4], ef[RW - 1][SBR][4];
+        R(&eca)[SBR][4] = *reinterpret_cast<R(*)[SBR][4]>(TWO_CRIT ? &eca_own[0] : &ecn[0]);
+        // first turn: super-block `set`, row 0
+        if constexpr (TWO_CRIT) {
+            fetch4(0, (SET - 1) * SBR, ecn);
+            fetch4(0, SET * SBR, eca);
+        } else {
+            fetch4(0, 0, ecn);  // set 0: its inverse; set 1: its near update with X_0
+        }
+    #pragma unroll
+        for (int h = 1; h < RW; ++h) fetch4(h, 0, ef[h - 1]);
+
+        // ---- right-hand sides into the accumulator layout (as in trsm_diag_kernel) ----
+        Acc y[RW][NBK];
+        auto mem_row = [&](int P) __attribute__((always_inline)) { return FORWARD ? P : nb - 1 - P; };
+        auto at = [&](int P, int64_t j) __attribute__((always_inline)) -> int64_t {
+            return RIGHT ? j + (int64_t)mem_row(P) * ldb : (int64_t)mem_row(P) + j * ldb;
+        };
+        constexpr bool ROWS4 = !RIGHT;
+        typedef R rx4u_t __attribute__((ext_vector_type(4), aligned(sizeof(R))));
+    #pragma unroll
+        for (int h = 0; h < RW; ++h)
+    #pragma unroll
+            for (int k = 0; k < NBK; ++k) {
+                const int64_t j = j0 + 16 * k + jj;
+                const int P0 = row_of(h) * IB + M::krow(g, 0);
+                if (ROWS4 && P0 + 3 < nb && j < nrhs) {
+                    if constexpr (ROWS4) {
+                        const rx4u_t t = *reinterpret_cast<const rx4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j)));
+    #pragma unroll
+                        for (int v = 0; v < 4; ++v) y[h][k][v] = alpha * t[FORWARD ? v : 3 - v];
+                    }
+                } else {
+    #pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int P = P0 + v;
+                        const bool have = P < nb && j < nrhs;
+                        const T b = Bblk[have ? at(P, j) : 0];
+                        y[h][k][v] = have ? alpha * b : (T)0;
+                    }
+                }
+            }
+        auto store_row = [&](int h) __attribute__((always_inline)) {
+    #pragma unroll
+            for (int k = 0; k < NBK; ++k) {
+                const int64_t j = j0 + 16 * k + jj;
+                const int P0 = row_of(h) * IB + M::krow(g, 0);
+                if (ROWS4 && P0 + 3 < nb && j < nrhs) {
+                    if constexpr (ROWS4) {
+                        rx4u_t t;
+    #pragma unroll
+                        for (int v = 0; v < 4; ++v) t[FORWARD ? v : 3 - v] = y[h][k][v];
+                        *reinterpret_cast<rx4u_t *>(Bblk + (FORWARD ? at(P0, j) : at(P0 + 3, j))) = t;
+                    }
+                } else {
+    #pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int P = P0 + v;
+                        if (P < nb && j < nrhs) Bblk[at(P, j)] = y[h][k][v];
+                    }
+                }
+            }
+        };
+        // An accumulator block in LDS: 16-byte pieces, each piece of all 64 lanes together.
+        auto blk_put = [&](R *buf, int i, int k, const Acc &a) __attribute__((always_inline)) {
+    #pragma unroll
+            for (int ch = 0; ch < CH; ++ch) {
+                VT t;
+    #pragma unroll
+                for (int x = 0; x < V; ++x) t[x] = a[ch * V + x];
+                *reinterpret_cast<VT *>(buf + (((i * NBK + k) * CH + ch) * 64 + lane) * V) = t;
+            }
+        };
+        auto blk_get = [&](const R *buf, int i, int k) __attribute__((always_inline)) -> Acc {
+            Acc a;
+    #pragma unroll
+            for (int ch = 0; ch < CH; ++ch) {
+                const VT t = *reinterpret_cast<const VT *>(buf + (((i * NBK + k) * CH + ch) * 64 + lane) * V);
+    #pragma unroll
+                for (int x = 0; x < V; ++x) a[ch * V + x] = t[x];
+            }
+            return a;
+        };
+        // out += E in for one sub-block E (this lane's values) and NBK blocks in MFMA "B" operand order
+        auto block_mma = [&](const R (&ev)[4], const Acc (&in)[NBK], Acc (&out)[NBK]) {
+    #pragma unroll
+            for (int c = 0; c < 4; ++c)
+    #pragma unroll
+                for (int k = 0; k < NBK; ++k) out[k] = M::run(ev[c], in[k][c], out[k]);
+        };
+        // Far update with the X of step s (in half s % 2 of Xb): rows HMIN .. RW-1 of this wavefront take
+        // y += (-L(row, 4s .. 4s+3)) X_s, the rows in the inner loop so that consecutive MFMAs are independent;
+        // then each row's sub-blocks of step s + 1 are requested.
+        auto far = [&](auto sc, auto hminc) __attribute__((always_inline)) {
+            constexpr int s = decltype(sc)::value, HMIN = decltype(hminc)::value;
+            if constexpr (HMIN < RW && s >= 0) {
+                const R *X = Xb[s % 2];
+    #pragma unroll
+                for (int q = 0; q < SBR; ++q) {
+                    Acc in[NBK];
+    #pragma unroll
+                    for (int k = 0; k < NBK; ++k) in[k] = blk_get(X, q, k);
+    #pragma unroll
+                    for (int c = 0; c < 4; ++c)
+    #pragma unroll
+                        for (int h = HMIN; h < RW; ++h) {
+                            if (row_of(h) < nsteps) {
+    #pragma unroll
+                                for (int k = 0; k < NBK; ++k) y[h][k] = M::run(ef[h - 1][q][c], in[k][c], y[h][k]);
+                            }
+                        }
+                }
+                // (The requests for the next step's sub-blocks stay behind this step's MFMAs: hoisted above
+                // them they would need a second set of registers.)
+    #pragma unroll
+                for (int h = HMIN; h < RW; ++h)
+    #pragma unroll
+                    for (int k = 0; k < NBK; ++k) asm volatile("" : "+v"(y[h][k]) : : "memory");
+    #pragma unroll
+                for (int h = HMIN; h < RW; ++h) fetch4(h, (s + 1) * SBR, ef[h - 1]);
+            }
+        };
+
+        if constexpr (SET == 0) {  // owners of super-block 0 file their Y
+    #pragma unroll
+            for (int k = 0; k < NBK; ++k) blk_put(Yb, own_i, k, y[0][k]);
+        }
+        __syncthreads();
+        // Step S, two halves with a barrier after each:
+        //   first   owners of S (set S % 2, their row S / 2):  A  X = sum_{j <= i} Inv(i, j) Y_j
+        //           the other set:                              far update with X_(S-1) on all its unsolved rows
+        //   second  owners of S:                                X to memory; far update with X_(S-1) on the rows beyond S + 1
+        //           the other set (owners of S + 1):            N  near update of its row of S + 1 with X_S; Y filed
+        // Every row thus takes the X of an earlier super-block of its own set's one half-step after it appears
+        // and the X of the other set's three half-steps after, always in the same order.
+        auto step = [&](auto Sc) __attribute__((always_inline)) {
+            constexpr int S = decltype(Sc)::value;
+            constexpr int HO = S / 2;        // the owners' row
+            constexpr int HN = (S + 1) / 2;  // the row of S + 1 in the other set
+            constexpr bool mine = SET == S % 2;
+            if constexpr (mine) {
+                if (row_of(HO) < nsteps) {
+                    Acc x[NBK];
+    #pragma unroll
+                    for (int k = 0; k < NBK; ++k) x[k] = Acc{0, 0, 0, 0};
+    #pragma unroll
+                    for (int q = 0; q < SBR; ++q) {
+                        if (q < own_i) {
+                            Acc in[NBK];
+    #pragma unroll
+                            for (int k = 0; k < NBK; ++k) in[k] = blk_get(Yb, q, k);
+                            block_mma(eca[q], in, x);
+                        } else if (q == own_i) {
+                            block_mma(eca[q], y[HO], x);
+                        }
+                    }
+    #pragma unroll
+                    for (int k = 0; k < NBK; ++k) {
+                        y[HO][k] = x[k];
+                        blk_put(Xb[S % 2], own_i, k, x[k]);
+                    }
+                }
+                // the coefficients of the next turn as an owner: super-block S + 2, row HO + 1
+                if constexpr (HO + 1 < RW) {
+    #pragma unroll
+                    for (int k = 0; k < NBK; ++k) asm volatile("" : "+v"(y[HO][k]) : : "memory");
+                    fetch4(HO + 1, (S + 1) * SBR, ecn);
+                    if constexpr (TWO_CRIT) fetch4(HO + 1, (S + 2) * SBR, eca);
+                }
+            } else {
+                far(IntC<S - 1>{}, IntC<(S + 1) / 2>{});
+            }
+            __syncthreads();
+            if constexpr (mine) {
+                if (row_of(HO) < nsteps) store_row(HO);
+                far(IntC<S - 1>{}, IntC<S / 2 + 1>{});
+            } else if constexpr (HN < RW && S + 1 < NS) {
+                if (row_of(HN) < nsteps) {
+    #pragma unroll
+                    for (int q = 0; q < SBR; ++q) {
+                        Acc in[NBK];
+    #pragma unroll
+                        for (int k = 0; k < NBK; ++k) in[k] = blk_get(Xb[S % 2], q, k);
+                        block_mma(ecn[q], in, y[HN]);
+                    }
+                    if constexpr (!TWO_CRIT) {
+    #pragma unroll
+                        for (int k = 0; k < NBK; ++k) asm volatile("" : "+v"(y[HN][k]) : : "memory");
+                        fetch4(HN, (S + 1) * SBR, ecn);
+                    }
+    #pragma unroll
+                    for (int k = 0; k < NBK; ++k) blk_put(Yb, own_i, k, y[HN][k]);
+                }
+            }
+            __syncthreads();
+        };
+        if (0 < nsuper) step(IntC<0>{});
+        if (1 < nsuper) step(IntC<1>{});
+        if (2 < nsuper) step(IntC<2>{});
+        if (3 < nsuper) step(IntC<3>{});
+        if (4 < nsuper) step(IntC<4>{});
+        if (5 < nsuper) step(IntC<5>{});
+        if (6 < nsuper) step(IntC<6>{});
+        if (7 < nsuper) step(IntC<7>{});
+    };
+    if (wave / SBR == 0) body(IntC<0>{}); else body(IntC<1>{});
+    static_assert(NS == 8, "one step call per super-block");
+}
+
 template <typename T> struct TrsmDriver {
     typedef typename Elem<T>::Real R;
     static constexpr int NBL = TrsmLeaf<T>::NB;
@@ -604,6 +1048,7 @@ template <typename T> struct TrsmDriver {
     int64_t ldb;
     hipStream_t stream;
     const R *pack;  // packed diagonal blocks, TrsmLeaf<T>::PACK_REALS each
+    bool inv_leaf;  // real types: the block solve with inverted 64 x 64 triangles (else substitution over 16-row sub-blocks)
 
     static T minus_one() { return el_scale_host(-1); }
     static T el_scale_host(int v) {
@@ -613,9 +1058,28 @@ template <typename T> struct TrsmDriver {
 
     // Packs every diagonal block of the triangle (one launch per call).
     hipError_t prepare() {
-        typedef TrsmLeaf<T> L;
         const int n = right ? N : M;
         const int nblk = (n + NBL - 1) / NBL;
+        void *wv = nullptr;
+        if constexpr (!Elem<T>::CPLX) {
+            if (!inv_leaf) return prepare_substitution(n, nblk);
+            typedef TrsmBlock<T> L;
+            hipError_t we = workspace_get(stream, (size_t)nblk * L::PACK_REALS * sizeof(R), 2, &wv);
+            if (we != hipSuccess) return we;
+            pack = (const R *)wv;
+            void (*fn)(const T *, int64_t, int, bool, bool, T *) =
+                forward ? trsm_pack_inv_kernel<T, true> : trsm_pack_inv_kernel<T, false>;
+            hipError_t e = ensure_dynamic_lds((const void *)fn, L::PACK_SMEM);
+            if (e != hipSuccess) return e;
+            dispatch_record().launches++;
+            return launch_kernel(fn, dim3(L::COPY_GROUPS + L::NS, nblk), dim3(256), L::PACK_SMEM, stream, A, lda, n, teff, unit,
+                                 (T *)wv);
+        } else {
+            return prepare_substitution(n, nblk);
+        }
+    }
+    hipError_t prepare_substitution(int n, int nblk) {
+        typedef TrsmLeaf<T> L;
         void *wv = nullptr;
         hipError_t we = workspace_get(stream, (size_t)nblk * L::PACK_REALS * sizeof(R), 2, &wv);
         if (we != hipSuccess) return we;
@@ -629,12 +1093,29 @@ template <typename T> struct TrsmDriver {
                              conj, unit, w);
     }
 
+    // Real types: the block solve with inverted 64 x 64 triangles, NBK blocks of 16 right-hand sides per workgroup.
+    template <bool RIGHT, int NBK> hipError_t block_side(int i0, int nb, T alpha) {
+        if constexpr (!Elem<T>::CPLX) {
+            typedef TrsmBlock<T> L;
+            const int nrhs = RIGHT ? M : N;
+            T *Bblk = RIGHT ? B + (int64_t)i0 * ldb : B + i0;
+            const T *packed = pack + (int64_t)(i0 / NBL) * L::PACK_REALS;
+            void (*fn)(const T *, int, T, T *, int64_t, int) =
+                forward ? trsm_block_kernel<T, RIGHT, true, NBK> : trsm_block_kernel<T, RIGHT, false, NBK>;
+            dim3 grid((unsigned)((nrhs + 16 * NBK - 1) / (16 * NBK))), block(L::THREADS);
+            dispatch_record().launches++;
+            return launch_kernel(fn, grid, block, 0, stream, packed, nb, alpha, Bblk, ldb, nrhs);
+        } else {
+            return hipErrorNotSupported;
+        }
+    }
+
     template <bool RIGHT, bool WIDE> hipError_t leaf_side(int i0, int nb, T alpha) {
         typedef TrsmLeaf<T, RIGHT, WIDE> L;
         const int nrhs = RIGHT ? M : N;
         T *Bblk = RIGHT ? B + (int64_t)i0 * ldb : B + i0;
         const R *packed = pack + (int64_t)(i0 / NBL) * L::PACK_REALS;
-        void (*fn)(const R *, int, T, T *, int64_t, int) =
+        void (*fn)(const R *, int, T, T *, int64_t, int, int) =
             forward ? trsm_diag_kernel<T, RIGHT, true, WIDE> : trsm_diag_kernel<T, RIGHT, false, WIDE>;
         if (L::SMEM > 64 * 1024) {
             hipError_t e = ensure_dynamic_lds((const void *)fn, L::SMEM);
@@ -642,20 +1123,30 @@ template <typename T> struct TrsmDriver {
         }
         dim3 grid((unsigned)((nrhs + L::CW - 1) / L::CW)), block(L::THREADS);
         dispatch_record().launches++;
-        return launch_kernel(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs);
+        // (2^22 polls: far beyond any wait of a leaf that works, short enough that a mistake ends in seconds)
+        const int poll_limit = knobs().trsm_poll_limit > 0 ? knobs().trsm_poll_limit : (1 << 22);
+        return launch_kernel(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs, poll_limit);
     }
-    // Right-hand sides per workgroup.  16 gives a launch twice the workgroups; 32 (real types) gives each
-    // sub-block of coefficients twice the work and is taken when 16 would make more than one round of
-    // workgroups anyway (more than 256 x 16 right-hand sides), and for FP32 with side = right, whose
-    // right-hand sides are rows of B: 16 floats are too short a run of memory.
+    // Right-hand sides per workgroup.  Real types: 16, or 32 for FP32 (each sub-block of coefficients is then
+    // used twice) when 16 would make more than one round of workgroups anyway (more than 256 x 16
+    // right-hand sides) or with side = right, whose right-hand sides are rows of B: 16 floats are too
+    // short a run of memory.
     hipError_t leaf(int i0, int nb, T alpha) {
-        constexpr bool CAN_WIDEN = !Elem<T>::CPLX;
         const int nrhs = right ? M : N;
-        const bool wide = CAN_WIDEN && (nrhs > 256 * 16 || (right && sizeof(R) == 4));
-        if constexpr (CAN_WIDEN) {
-            if (wide) return right ? leaf_side<true, true>(i0, nb, alpha) : leaf_side<false, true>(i0, nb, alpha);
+        if constexpr (!Elem<T>::CPLX) {
+            if (!inv_leaf) {
+                const bool wide = nrhs > 256 * 16 || (right && sizeof(R) == 4);
+                if (wide) return right ? leaf_side<true, true>(i0, nb, alpha) : leaf_side<false, true>(i0, nb, alpha);
+                return right ? leaf_side<true, false>(i0, nb, alpha) : leaf_side<false, false>(i0, nb, alpha);
+            }
+            const bool two = sizeof(R) == 4 && (nrhs > 256 * 16 || right);
+            if constexpr (sizeof(R) == 4) {
+                if (two) return right ? block_side<true, 2>(i0, nb, alpha) : block_side<false, 2>(i0, nb, alpha);
+            }
+            return right ? block_side<true, 1>(i0, nb, alpha) : block_side<false, 1>(i0, nb, alpha);
+        } else {
+            return right ? leaf_side<true, false>(i0, nb, alpha) : leaf_side<false, false>(i0, nb, alpha);
         }
-        return right ? leaf_side<true, false>(i0, nb, alpha) : leaf_side<false, false>(i0, nb, alpha);
     }
 
     // Off-diagonal update of the block range `dst` (length nd, start d0) with the solved
@@ -702,9 +1193,22 @@ hipError_t trsm_colmajor(bool right, bool lower, bool trans, bool conj, bool uni
     d.forward = right ? (lower == trans) : (lower != trans);
     d.teff = trans != right;
     d.M = M; d.N = N; d.A = A; d.lda = lda; d.B = B; d.ldb = ldb; d.stream = stream;
+    d.inv_leaf = !Elem<T>::CPLX && knobs().trsm_leaf != 0;
     hipError_t e = d.prepare();
     if (e != hipSuccess) return e;
     return d.solve(0, right ? N : M, alpha);
+}
+
+hipError_t trsm_poll_timeouts_read(unsigned int *count, bool reset) {
+    unsigned int v = 0;
+    hipError_t e = hipMemcpyFromSymbol(&v, HIP_SYMBOL(trsm_poll_timeouts), sizeof v);
+    if (e != hipSuccess) return e;
+    if (count) *count = v;
+    if (reset && v != 0) {
+        const unsigned int zero = 0;
+        e = hipMemcpyToSymbol(HIP_SYMBOL(trsm_poll_timeouts), &zero, sizeof zero);
+    }
+    return e;
 }
 
 template hipError_t trsm_colmajor<float>(bool, bool, bool, bool, bool, int, int, float, const float *, int64_t, float *,

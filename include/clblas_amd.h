@@ -367,6 +367,14 @@ clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, si
  * outgrown ones that are parked until the stream is released). */
 void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes);
 
+/* The TRSM kernel that solves a diagonal block by substitution synchronises its wavefronts through
+ * flags in LDS; a wait for a flag gives up after a bounded number of polls (so that a mistake in the
+ * library would end in a wrong result, not in a hung GPU).  This reads, for the current GPU, how many
+ * waits have ever given up since the library was loaded - zero unless the library is broken or the
+ * debugging variable CLBLAS_AMD_TRSM_POLL_LIMIT makes the bound tiny - and, with reset != 0, sets the
+ * count back to zero.  It waits for the device (a blocking copy).  No counterpart in the reference. */
+clblasStatus clblasAmdTrsmPollTimeouts(unsigned int *count, int reset);
+
 /* Describes the last GEMM kernel the calling thread launched (kernel family, tile, transposes,
  * sizes, grid, K ranges), as text; returns the number of kernel launches the thread has issued
  * through this library.  With CLBLAS_AMD_LOG=1 in the environment every launch also prints

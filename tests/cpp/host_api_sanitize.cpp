@@ -35,6 +35,7 @@ hipError_t trsm_colmajor(bool, bool, bool, bool, bool, int, int, T, const T *, i
 hipError_t sgemm_colmajor_noalloc(bool, bool, int, int, int, float, const float *, int64_t, const float *, int64_t, float,
                                   float *, int64_t, hipStream_t) { reached("sgemm_noalloc"); }
 hipError_t noalloc_scratch(void **) { return hipErrorNoDevice; }
+hipError_t trsm_poll_timeouts_read(unsigned int *count, bool) { if (count) *count = 0; return hipSuccess; }
 
 #define INST(T)                                                                                                         \
     template hipError_t launch_gemm<T>(bool, bool, bool, bool, int, int, int, T, const T *, int64_t, const T *, int64_t, T, \
