@@ -259,13 +259,13 @@ TILE_MODEL_SHAPES = (
 )
 
 
-def tile_model_block(torch, clblas_amd, gen):
+def tile_model_block(torch, clblas_amd, gen, keep_forced=False):
     """Default tile choice against every forced tile (debug switch CLBLAS_AMD_GEMM_TILE), SGEMM and DGEMM,
     column-major NN, alpha = beta = 1.  Per shape: [default TFLOP/s, default tile, best forced TFLOP/s, best
     tile]; `mispicks` lists the shapes where the default runs more than 3 % behind a different, forced tile."""
     out = {}
     for name, dt, fn, ntiles in (("sgemm", torch.float32, clblas_amd.sgemm, 5), ("dgemm", torch.float64, clblas_amd.dgemm, 2)):
-        rows, mispicks, worst = {}, [], 1.0
+        rows, mispicks, worst, forced = {}, [], 1.0, {}
         for (M, N, K) in TILE_MODEL_SHAPES:
             if name == "dgemm" and M * N * K > 6.5e10:
                 continue
@@ -281,27 +281,36 @@ def tile_model_block(torch, clblas_amd, gen):
             ms_default = timed_batch(torch, call, reps, 2, batches=3)
             import re
             default_tile = re.search(r"<\w,(\d+x\d+)x", clblas_amd.last_dispatch()[0]).group(1)
-            best, best_tile, best_dims = None, -1, ""
+            default_desc = clblas_amd.last_dispatch()[0]
+            best, best_tile, best_dims, per_tile = None, -1, "", []
             for tile in range(ntiles):
                 os.environ["CLBLAS_AMD_GEMM_TILE"] = str(tile)
                 clblas_amd.reload_debug_env()
                 try:
                     ms = timed_batch(torch, call, reps, 2, batches=3)
-                    dims = re.search(r"<\w,(\d+x\d+)x", clblas_amd.last_dispatch()[0]).group(1)
+                    desc = clblas_amd.last_dispatch()[0]
+                    dims = re.search(r"<\w,(\d+x\d+)x", desc).group(1)
                 finally:
                     os.environ.pop("CLBLAS_AMD_GEMM_TILE", None)
                     clblas_amd.reload_debug_env()
+                # [milliseconds, K ranges, tail slices] of the forced tile: what clblas_amd/fit_tile_model.py fits to
+                per_tile.append([round(ms, 5), int(re.search(r"splits=(\d+)", desc).group(1)),
+                                 int(re.search(r"tail_slices=(\d+)", desc).group(1))])
                 if best is None or ms < best:
                     best, best_tile, best_dims = ms, tile, dims
             tf = lambda ms: round(2.0 * M * N * K / ms / 1e9, 1)
             key = "%dx%dx%d" % (M, N, K)
             rows[key] = [tf(ms_default), default_tile, tf(best), best_dims]
+            forced[key] = {"default_ms": round(ms_default, 5), "default_splits": int(re.search(r"splits=(\d+)", default_desc).group(1)),
+                           "tiles": per_tile}
             ratio = best / ms_default if best_dims != default_tile else 1.0   # the same tile twice: timing noise
             worst = min(worst, ratio)
             if ratio < 0.97:
                 mispicks.append(key)
             del A, B, C
         out[name] = {"shapes": rows, "mispicks": mispicks, "worst_default_over_best": round(worst, 3)}
+        if keep_forced:
+            out[name]["forced_ms"] = forced
     return out
 
 
@@ -772,7 +781,8 @@ def main():
     # ---- The tile choice against the best forced tile, on shapes that are not whole rounds of any tile:
     #      tracks how well the cost model in the launcher (choose_tile) fits the kernels as they are now. ----
     if args.only in ("", "tilemodel"):
-        extra["tile_model"] = tile_model_block(torch, clblas_amd, gen)
+        # (--only tilemodel also keeps every forced tile's time: the input of clblas_amd/fit_tile_model.py)
+        extra["tile_model"] = tile_model_block(torch, clblas_amd, gen, keep_forced=args.only == "tilemodel")
 
     # ---- Yardstick: the vendor BLAS that torch calls (rocBLAS / hipBLASLt) on the same box, same sizes.
     #      Not the reference and not a target of the parity tests: it shows what the part gives a

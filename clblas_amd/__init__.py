@@ -79,7 +79,7 @@ EXPORTED_SYMBOLS = (
 ) + tuple("clblas%s%s" % (t, f) for f in ("syrk", "trmm", "symm", "syr2k") for t in "SDCZ") + tuple(
     "clblas%s%s" % (t, f) for f in ("herk", "her2k", "hemm") for t in "CZ") + (
     "clblasAmdReleaseStream", "clblasAmdReserveWorkspace", "clblasAmdWorkspaceStats", "clblasAmdLastDispatch",
-    "clblasAmdReloadDebugEnv", "clblasAmdTrsmPollTimeouts")
+    "clblasAmdReloadDebugEnv", "clblasAmdTrsmPollTimeouts", "clblasAmdTileModelQuery", "clblasAmdTileModelParam")
 
 _lib = None
 
@@ -153,6 +153,12 @@ def _declare(lib):
     lib.clblasAmdLastDispatch.argtypes = [ctypes.c_char_p, sz]
     lib.clblasAmdReloadDebugEnv.restype = None
     lib.clblasAmdReloadDebugEnv.argtypes = []
+    lib.clblasAmdTileModelQuery.restype = ctypes.c_int
+    lib.clblasAmdTileModelQuery.argtypes = [ctypes.c_char, sz, sz, sz, ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_int),
+                                            ctypes.POINTER(ctypes.c_int), ctypes.POINTER(ctypes.c_double),
+                                            ctypes.POINTER(ctypes.c_int), ctypes.c_int]
+    lib.clblasAmdTileModelParam.restype = ctypes.c_int
+    lib.clblasAmdTileModelParam.argtypes = [ctypes.c_char, ctypes.c_int, ctypes.c_int, ctypes.POINTER(ctypes.c_double), ctypes.c_int]
     lib.clblasAmdTrsmPollTimeouts.restype = ctypes.c_int
     lib.clblasAmdTrsmPollTimeouts.argtypes = [ctypes.POINTER(ctypes.c_uint), ctypes.c_int]
 
@@ -238,6 +244,34 @@ def workspace_stats():
     a, b = ctypes.c_size_t(), ctypes.c_size_t()
     load_library().clblasAmdWorkspaceStats(ctypes.byref(a), ctypes.byref(b))
     return a.value, b.value
+
+
+TILE_PARAMS = ("eff", "alone", "k0", "tail_extra", "deep_gain")
+
+
+def tile_model_query(type_letter, M, N, K):
+    """The tile choice for a plain product, without launching: dict with the chosen tile's index, its K
+    ranges and tail slices, and per tile of the table its dimensions "BMxBNxBK" and the model's cost
+    (None: not offered).  type_letter: "s" or "d"."""
+    n = 16
+    tile, splits, tail = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    costs, dims = (ctypes.c_double * n)(), (ctypes.c_int * (3 * n))()
+    nt = load_library().clblasAmdTileModelQuery(type_letter.encode(), M, N, K, ctypes.byref(tile), ctypes.byref(splits),
+                                                ctypes.byref(tail), costs, dims, n)
+    if nt < 0:
+        raise ValueError("clblasAmdTileModelQuery refused (%r, %d, %d, %d)" % (type_letter, M, N, K))
+    return {"tile": tile.value, "splits": splits.value, "tail_slices": tail.value,
+            "tiles": ["%dx%dx%d" % tuple(dims[3 * i:3 * i + 3]) for i in range(nt)],
+            "costs": [costs[i] if costs[i] >= 0 else None for i in range(nt)]}
+
+
+def tile_model_param(type_letter, tile, name, value=None):
+    """Reads (value is None) or sets parameter `name` (one of TILE_PARAMS) of tile `tile`'s choice model."""
+    v = ctypes.c_double(0.0 if value is None else float(value))
+    if load_library().clblasAmdTileModelParam(type_letter.encode(), tile, TILE_PARAMS.index(name), ctypes.byref(v),
+                                              0 if value is None else 1) != 0:
+        raise ValueError("no parameter %r of tile %d for type %r" % (name, tile, type_letter))
+    return v.value
 
 
 def trsm_poll_timeouts(reset=False):

@@ -622,6 +622,23 @@ clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, si
 
 void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes) { cba::ws_stats(streams, bytes); }
 
+int clblasAmdTileModelQuery(char type, size_t M, size_t N, size_t K, int *tile, int *splits, int *tail_slices,
+                            double *costs, int *dims, int max_tiles) {
+    if (!tile || !splits || !tail_slices || !costs || !dims || max_tiles < 1) return -1;
+    if (M == 0 || N == 0 || K == 0 || M > kMaxDim || N > kMaxDim || K > kMaxDim) return -1;
+    if (type == 's') return cba::sgemm_model_query((int)M, (int)N, (int)K, tile, splits, tail_slices, costs, max_tiles, dims);
+    if (type == 'd') return cba::dgemm_model_query((int)M, (int)N, (int)K, tile, splits, tail_slices, costs, max_tiles, dims);
+    return -1;
+}
+
+int clblasAmdTileModelParam(char type, int tile, int which, double *value, int set) {
+    double *p = type == 's' ? cba::sgemm_model_param(tile, which) : type == 'd' ? cba::dgemm_model_param(tile, which) : nullptr;
+    if (!p || !value) return -1;
+    if (set) *p = *value;
+    else *value = *p;
+    return 0;
+}
+
 clblasStatus clblasAmdTrsmPollTimeouts(unsigned int *count, int reset) {
     return map_hip_error(cba::trsm_poll_timeouts_read(count, reset != 0));
 }

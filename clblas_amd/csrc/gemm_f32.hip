@@ -23,8 +23,9 @@ namespace cba {
 //      depth 16, 8192 x 64 x 8192: 106-112 against 91-94); with panels of depth 64 where a workgroup's K
 //      range is at least 1024 (1024^3 95.4 -> 99.0 TFLOP/s, 1024 x 1024 x 2048 109 -> 115, 960 x 960 x 2048
 //      96 -> 101, 512 x 512 x 4096 85 -> 90)
-static const TileEntry<float> *f32_tiles(int *n) {
-    static const TileEntry<float> tab[] = {
+// (Not const: clblasAmdTileModelParam lets the fitting script vary the model's parameters; the launch path only reads.)
+static TileEntry<float> *f32_tiles(int *n) {
+    static TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.12),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0),
@@ -41,6 +42,18 @@ hipError_t sgemm_colmajor(bool transA, bool transB, int M, int N, int K, float a
     int n;
     const TileEntry<float> *tab = f32_tiles(&n);
     return run_gemm_colmajor<float>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, tri, fixed);
+}
+
+int sgemm_model_query(int M, int N, int K, int *tile, int *splits, int *tail_slices, double *costs, int max_costs, int *dims) {
+    int n;
+    const TileEntry<float> *tab = f32_tiles(&n);
+    model_query<float>(tab, n, M, N, K, tile, splits, tail_slices, costs, max_costs);
+    for (int i = 0; i < n && i < max_costs; ++i) { dims[3 * i] = tab[i].bm; dims[3 * i + 1] = tab[i].bn; dims[3 * i + 2] = tab[i].bk; }
+    return n;
+}
+double *sgemm_model_param(int tile, int which) {
+    int n;
+    return model_param<float>(f32_tiles(&n), n, tile, which);
 }
 
 }  // namespace cba

@@ -13,8 +13,9 @@ namespace cba {
 //      1024 x 1024 x 2048 59.8 -> 64.2, 960 x 960 x 2048 50.9 -> 53.4).
 //   Short K on large C goes to the 64x64 tiles through the fixed-time term (k0 = 95 and 68):
 //   4096 x 4096 x 64 31.9 -> 38.9 TFLOP/s, x 128 45.5 -> 52.2, x 256 57.5 -> 61.6, 3000 x 3000 x 640 59.2 -> 64.3.
-static const TileEntry<double> *f64_tiles(int *n) {
-    static const TileEntry<double> tab[] = {
+// (Not const: clblasAmdTileModelParam lets the fitting script vary the model's parameters; the launch path only reads.)
+static TileEntry<double> *f64_tiles(int *n) {
+    static TileEntry<double> tab[] = {
         make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 95.0),
         make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32, true>(0.90, 0.85, 0.84, 68.0),
     };
@@ -28,6 +29,18 @@ hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double 
     int n;
     const TileEntry<double> *tab = f64_tiles(&n);
     return run_gemm_colmajor<double>(tab, n, transA, transB, false, false, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, tri);
+}
+
+int dgemm_model_query(int M, int N, int K, int *tile, int *splits, int *tail_slices, double *costs, int max_costs, int *dims) {
+    int n;
+    const TileEntry<double> *tab = f64_tiles(&n);
+    model_query<double>(tab, n, M, N, K, tile, splits, tail_slices, costs, max_costs);
+    for (int i = 0; i < n && i < max_costs; ++i) { dims[3 * i] = tab[i].bm; dims[3 * i + 1] = tab[i].bn; dims[3 * i + 2] = tab[i].bk; }
+    return n;
+}
+double *dgemm_model_param(int tile, int which) {
+    int n;
+    return model_param<double>(f64_tiles(&n), n, tile, which);
 }
 
 }  // namespace cba

@@ -247,7 +247,7 @@ template <typename T> static double split_overhead_cost(int M, int N, int K, int
 
 template <typename T>
 static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, int force, bool need_tri, int tri_c,
-                        bool tri_operand, bool tail_ok, int *tile_out, int *splits_out) {
+                        bool tri_operand, bool tail_ok, int *tile_out, int *splits_out, double *costs_out = nullptr) {
     const int64_t kCUs = 256;
     int pick = ntab - 1;  // table is ordered large -> small
     bool pick_split = true;
@@ -288,6 +288,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             double cost = rounds * tab[i].bm * tab[i].bn / eff;
             if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             cost *= 1.0 + tab[i].k0 / K;
+            if (costs_out) costs_out[i] = cost;
             if (!have || cost < best) { best = cost; pick = i; have = true; }
             // Small C, deep K: the larger tiles with a K split, ranges of at least 512 and 32 panels.
             if (split_model && tab[i].has_splitk && i != ntab - 1) {
@@ -525,6 +526,34 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
         }
     }
     return err;
+}
+
+// The tile choice as a function of the shape alone (plain product, no forced tile), with the cost the
+// model puts on every tile in one range (negative where a tile is not offered): what
+// clblasAmdTileModelQuery reports and the fitting script (clblas_amd/fit_tile_model.py) evaluates.
+template <typename T>
+static void model_query(const TileEntry<T> *tab, int ntab, int M, int N, int K, int *tile, int *splits, int *tail_slices,
+                        double *costs, int max_costs) {
+    double c[16];
+    for (int i = 0; i < 16; ++i) c[i] = -1.0;
+    choose_tile(tab, ntab, M, N, K, -1, false, 0, false, knobs().tail != 0, tile, splits, c);
+    for (int i = 0; i < max_costs && i < ntab && i < 16; ++i) costs[i] = c[i];
+    const TileEntry<T> &e = tab[*tile];
+    const int64_t ntiles = ceil_div64(M, e.bm) * ceil_div64(N, e.bn);
+    *tail_slices = (*splits <= 1 && e.tri[0]) ? tail_slices_for(ntiles, K, e.bk, knobs().tail != 0) : 1;
+}
+
+// One parameter of the choice model of tile `i`: 0 eff, 1 alone, 2 k0, 3 tail_extra, 4 deep_gain.
+template <typename T> static double *model_param(TileEntry<T> *tab, int ntab, int i, int which) {
+    if (i < 0 || i >= ntab) return nullptr;
+    switch (which) {
+        case 0: return &tab[i].eff;
+        case 1: return &tab[i].alone;
+        case 2: return &tab[i].k0;
+        case 3: return &tab[i].tail_extra;
+        case 4: return &tab[i].deep_gain;
+        default: return nullptr;
+    }
 }
 
 }  // namespace cba

@@ -148,6 +148,14 @@ hipError_t dgemm_colmajor(bool transA, bool transB, int M, int N, int K, double 
                           int64_t lda, const double *B, int64_t ldb, double beta, double *C, int64_t ldc,
                           hipStream_t stream, const GemmTri *tri = nullptr);
 
+// The tile choice model of SGEMM / DGEMM from outside (diagnostics, clblasAmdTileModelQuery / ...Param):
+// the choice for a plain M x N x K product, the model's cost of every tile of the table in one K range
+// (negative: not offered), the tiles' dimensions (bm, bn, bk per tile); returns the number of tiles.
+int sgemm_model_query(int M, int N, int K, int *tile, int *splits, int *tail_slices, double *costs, int max_costs, int *dims);
+int dgemm_model_query(int M, int N, int K, int *tile, int *splits, int *tail_slices, double *costs, int max_costs, int *dims);
+double *sgemm_model_param(int tile, int which);  // nullptr: no such tile / parameter
+double *dgemm_model_param(int tile, int which);
+
 // Complex variants: conjA / conjB conjugate the elements of op(A) / op(B) (clblasConjTrans).
 hipError_t cgemm_colmajor(bool transA, bool transB, bool conjA, bool conjB, int M, int N, int K, Cx<float> alpha,
                           const Cx<float> *A, int64_t lda, const Cx<float> *B, int64_t ldb, Cx<float> beta,

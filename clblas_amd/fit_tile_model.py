@@ -1,0 +1,108 @@
+#!/usr/bin/env python3
+"""Refits the parameters of the SGEMM / DGEMM tile choice model to measured times.
+
+    python bench.py --only tilemodel --no-cpu > tilemodel.json        (on the GPU: every tile forced on 40 shapes)
+    python -m clblas_amd.fit_tile_model tilemodel.json                 (anywhere: needs no GPU)
+
+The launcher (clblas_amd/csrc/gemm_launch.hpp, choose_tile) prices every tile of a type's table for a
+product and takes the cheapest; each tile carries four fitted numbers: `eff` (share of the MFMA peak it
+is credited with), `alone` (factor when a workgroup has its CU to itself), `k0` (fixed time per
+workgroup, as a depth) and `tail_extra` (price of a sliced last round, in rounds).  This script takes the
+times of every forced tile on every shape from bench.py, evaluates the library's own model through
+clblasAmdTileModelQuery with trial parameters set through clblasAmdTileModelParam - the model is not
+restated here - and searches, one parameter at a time over a grid around its present value, for the
+setting with the least regret
+
+    regret = sum over shapes of  time(tile the model picks) / time(best tile) - 1,
+
+counting a pick that is more than 3 % behind the best as one extra percent each (those are what
+bench.py reports as mispicks).  Shapes whose forced runs cut K into ranges are left out of the fit (a
+forced tile splits by rule, the model's own pick by price: their times do not say what the model's pick
+would cost) and listed separately.  Prints the table before and after and the parameters as the
+arguments of make_tile_entry in gemm_f32.hip / gemm_f64.hip; it changes no file.
+"""
+import json
+import sys
+
+import clblas_amd
+
+GRIDS = {"eff": [-0.06, -0.04, -0.03, -0.02, -0.01, 0.01, 0.02, 0.03, 0.04, 0.06],
+         "alone": [-0.1, -0.05, -0.03, 0.03, 0.05, 0.1],
+         "k0": [-40, -20, -10, 10, 20, 40],
+         "tail_extra": [-0.1, -0.05, -0.02, 0.02, 0.05, 0.1, 0.2]}
+LIMITS = {"eff": (0.6, 1.0), "alone": (0.5, 1.0), "k0": (0.0, 300.0), "tail_extra": (0.0, 1.0)}
+
+
+def shapes_of(block):
+    """[(M, N, K, [ms per tile]), ...] for the shapes that can be fitted, and the keys of the others."""
+    fit, skipped = [], []
+    for key, rec in block["forced_ms"].items():
+        M, N, K = (int(x) for x in key.split("x"))
+        if rec["default_splits"] > 1 or any(t[1] > 1 for t in rec["tiles"]):
+            skipped.append(key)
+            continue
+        fit.append((M, N, K, [t[0] for t in rec["tiles"]]))
+    return fit, skipped
+
+
+def regret(letter, shapes, detail=False):
+    total, rows = 0.0, []
+    for M, N, K, ms in shapes:
+        q = clblas_amd.tile_model_query(letter, M, N, K)
+        pick = q["tile"]
+        r = ms[pick] / min(ms) - 1.0
+        total += r + (0.01 if r > 0.03 else 0.0)
+        if detail:
+            rows.append(("%dx%dx%d" % (M, N, K), q["tiles"][pick], q["tiles"][ms.index(min(ms))], r))
+    return (total, rows) if detail else total
+
+
+def fit(letter, shapes, ntiles, sweeps=4):
+    for _ in range(sweeps):
+        improved = False
+        for tile in range(ntiles):
+            for name, steps in GRIDS.items():
+                here = clblas_amd.tile_model_param(letter, tile, name)
+                best_v, best_r = here, regret(letter, shapes)
+                for d in steps:
+                    v = min(max(here + d, LIMITS[name][0]), LIMITS[name][1])
+                    clblas_amd.tile_model_param(letter, tile, name, v)
+                    r = regret(letter, shapes)
+                    if r < best_r - 1e-9:
+                        best_v, best_r, improved = v, r, True
+                clblas_amd.tile_model_param(letter, tile, name, best_v)
+        if not improved:
+            break
+
+
+def main(path):
+    data = json.load(open(path))
+    model = data["extra"]["tile_model"] if "extra" in data else data
+    for letter, name in (("s", "sgemm"), ("d", "dgemm")):
+        if name not in model or "forced_ms" not in model[name]:
+            print("%s: no forced-tile times in %s (run bench.py --only tilemodel)" % (name, path))
+            continue
+        shapes, skipped = shapes_of(model[name])
+        ntiles = len(shapes[0][3])
+        before, rows_before = regret(letter, shapes, detail=True)
+        params_before = [[clblas_amd.tile_model_param(letter, t, p) for p in GRIDS] for t in range(ntiles)]
+        fit(letter, shapes, ntiles)
+        after, rows_after = regret(letter, shapes, detail=True)
+        print("== %s: %d shapes fitted, %d left out (K ranges: %s)" % (name, len(shapes), len(skipped), ", ".join(skipped)))
+        print("   regret %.4f -> %.4f; picks more than 3 %% behind the best tile: %d -> %d" % (
+            before, after, sum(r[3] > 0.03 for r in rows_before), sum(r[3] > 0.03 for r in rows_after)))
+        for b, a in zip(rows_before, rows_after):
+            if b[1] != a[1] or a[3] > 0.015:
+                print("   %-18s before %-11s (%+5.1f %%)   after %-11s (%+5.1f %%)   best %s" % (
+                    b[0], b[1], 100 * b[3], a[1], 100 * a[3], a[2]))
+        q = clblas_amd.tile_model_query(letter, 1024, 1024, 1024)
+        print("   parameters (eff, alone, k0, tail_extra), before -> after:")
+        for t in range(ntiles):
+            now = [clblas_amd.tile_model_param(letter, t, p) for p in GRIDS]
+            print("     tile %d %-11s %s -> %s" % (t, q["tiles"][t], ["%.3g" % v for v in params_before[t]], ["%.3g" % v for v in now]))
+
+
+if __name__ == "__main__":
+    if len(sys.argv) != 2:
+        sys.exit(__doc__)
+    main(sys.argv[1])

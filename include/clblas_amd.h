@@ -367,6 +367,22 @@ clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, si
  * outgrown ones that are parked until the stream is released). */
 void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes);
 
+/* The tile choice of clblasSgemm (type 's') / clblasDgemm ('d') for a plain M x N x K product, as a
+ * function that launches nothing: the chosen tile (index into the type's tile table), its number of K
+ * ranges and tail slices, the cost the choice model puts on every tile in one K range (negative: tile not
+ * offered) and the tiles' dimensions (bm, bn, bk per tile, 3 ints each; `costs` and `dims` hold max_tiles
+ * entries).  Returns the number of tiles in the table, -1 for bad arguments.
+ * clblasAmdTileModelParam reads (set == 0) or sets one parameter of one tile's model - which: 0 the
+ * efficiency credited to the tile, 1 the factor for a workgroup alone on its CU, 2 the fixed time per
+ * workgroup as a depth, 3 the price of a sliced tail in rounds, 4 the credit of the deep-panel form -
+ * returning 0, or -1 for no such tile or parameter.  Both exist for clblas_amd/fit_tile_model.py, which
+ * refits the parameters to measured times; setting parameters while another thread is inside a GEMM call
+ * is not supported.  No counterpart in the reference (its selection table is generated at build time,
+ * src/library/blas/AutoGemm/KernelSelection.py). */
+int clblasAmdTileModelQuery(char type, size_t M, size_t N, size_t K, int *tile, int *splits, int *tail_slices,
+                            double *costs, int *dims, int max_tiles);
+int clblasAmdTileModelParam(char type, int tile, int which, double *value, int set);
+
 /* The TRSM kernel that solves a diagonal block by substitution synchronises its wavefronts through
  * flags in LDS; a wait for a flag gives up after a bounded number of polls (so that a mistake in the
  * library would end in a wrong result, not in a hung GPU).  This reads, for the current GPU, how many

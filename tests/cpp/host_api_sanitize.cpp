@@ -36,6 +36,10 @@ hipError_t sgemm_colmajor_noalloc(bool, bool, int, int, int, float, const float 
                                   float *, int64_t, hipStream_t) { reached("sgemm_noalloc"); }
 hipError_t noalloc_scratch(void **) { return hipErrorNoDevice; }
 hipError_t trsm_poll_timeouts_read(unsigned int *count, bool) { if (count) *count = 0; return hipSuccess; }
+int sgemm_model_query(int, int, int, int *, int *, int *, double *, int, int *) { return 0; }
+int dgemm_model_query(int, int, int, int *, int *, int *, double *, int, int *) { return 0; }
+double *sgemm_model_param(int, int) { return nullptr; }
+double *dgemm_model_param(int, int) { return nullptr; }
 
 #define INST(T)                                                                                                         \
     template hipError_t launch_gemm<T>(bool, bool, bool, bool, int, int, int, T, const T *, int64_t, const T *, int64_t, T, \
