@@ -11,13 +11,16 @@ namespace cba {
 //      .84) and with .84 where an operand is triangular (DTRMM / DSYMM 6144 lose 2-3 % with .90).
 //      With panels of depth 32 where a workgroup's K range is at least 1024 (1024^3 54.9 -> 58.5 TFLOP/s,
 //      1024 x 1024 x 2048 59.8 -> 64.2, 960 x 960 x 2048 50.9 -> 53.4).
-//   Short K on large C goes to the 64x64 tiles through the fixed-time term (k0 = 95 and 68):
+//   Last refit (clblas_amd/fit_tile_model.py on bench.py --only tilemodel): k0 of the 128x128 tile 95 -> 85, a
+//   sliced tail of the 64x64 tiles priced at 0.35 rounds instead of 0.05 (4480 x 4480 x 2000, 2500 x 7000 x 1200,
+//   8192 x 8192 x 512: the 128x128 tile 0.5-0.9 % ahead).
+//   Short K on large C goes to the 64x64 tiles through the fixed-time term (k0 = 85 and 68):
 //   4096 x 4096 x 64 31.9 -> 38.9 TFLOP/s, x 128 45.5 -> 52.2, x 256 57.5 -> 61.6, 3000 x 3000 x 640 59.2 -> 64.3.
 // (Not const: clblasAmdTileModelParam lets the fitting script vary the model's parameters; the launch path only reads.)
 static TileEntry<double> *f64_tiles(int *n) {
     static TileEntry<double> tab[] = {
-        make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 95.0),
-        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32, true>(0.90, 0.85, 0.84, 68.0),
+        make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 85.0),
+        make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32, true>(0.90, 0.85, 0.84, 68.0, 0.35),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;

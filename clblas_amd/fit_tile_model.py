@@ -26,10 +26,12 @@ import sys
 
 import clblas_amd
 
-GRIDS = {"eff": [-0.06, -0.04, -0.03, -0.02, -0.01, 0.01, 0.02, 0.03, 0.04, 0.06],
+# (k0 and tail_extra first: they say where a tile loses - short K, a sliced last round - and leave its
+# credit on long, whole rounds alone; eff moves only where those two cannot explain the times)
+GRIDS = {"k0": [-40, -20, -10, 10, 20, 40, 80],
+         "tail_extra": [-0.1, -0.05, -0.02, 0.02, 0.05, 0.1, 0.2],
          "alone": [-0.1, -0.05, -0.03, 0.03, 0.05, 0.1],
-         "k0": [-40, -20, -10, 10, 20, 40],
-         "tail_extra": [-0.1, -0.05, -0.02, 0.02, 0.05, 0.1, 0.2]}
+         "eff": [-0.04, -0.03, -0.02, -0.01, 0.01, 0.02, 0.03, 0.04]}
 LIMITS = {"eff": (0.6, 1.0), "alone": (0.5, 1.0), "k0": (0.0, 300.0), "tail_extra": (0.0, 1.0)}
 
 
@@ -64,7 +66,7 @@ def fit(letter, shapes, ntiles, sweeps=4):
             for name, steps in GRIDS.items():
                 here = clblas_amd.tile_model_param(letter, tile, name)
                 best_v, best_r = here, regret(letter, shapes)
-                for d in steps:
+                for d in sorted(steps, key=abs):   # the smallest change that gives the least regret
                     v = min(max(here + d, LIMITS[name][0]), LIMITS[name][1])
                     clblas_amd.tile_model_param(letter, tile, name, v)
                     r = regret(letter, shapes)
@@ -96,7 +98,7 @@ def main(path):
                 print("   %-18s before %-11s (%+5.1f %%)   after %-11s (%+5.1f %%)   best %s" % (
                     b[0], b[1], 100 * b[3], a[1], 100 * a[3], a[2]))
         q = clblas_amd.tile_model_query(letter, 1024, 1024, 1024)
-        print("   parameters (eff, alone, k0, tail_extra), before -> after:")
+        print("   parameters (%s), before -> after:" % ", ".join(GRIDS))
         for t in range(ntiles):
             now = [clblas_amd.tile_model_param(letter, t, p) for p in GRIDS]
             print("     tile %d %-11s %s -> %s" % (t, q["tiles"][t], ["%.3g" % v for v in params_before[t]], ["%.3g" % v for v in now]))
