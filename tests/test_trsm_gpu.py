@@ -156,3 +156,38 @@ def test_config5_dtrsm_8192(gpu):
     assert oracle.trsm_blocked(COL, LEFT, LOWER, NOTRANS, NONUNIT, k, nc, 1.0, Asub, 0, k, sub, 0, k) == 0
     want = sub.reshape(nc, k).T
     assert np.abs(X[:k, :nc] - want).max() <= 32 * k * np.finfo(np.float64).eps * np.abs(want).max()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("order", [ROW, COL])
+def test_inverted_triangle_leaf_behind_its_switch(gpu, dtype, order):
+    """The other way of solving a diagonal block (real types): 64 x 64 triangles inverted by doubling in the
+    packing pass - as the reference inverts its 128 x 128 ones - and a leaf of eight steps between barriers
+    (CLBLAS_AMD_TRSM_LEAF=1).  Same bars as test_all_variants, nothing widened, on a spread of the variants
+    and sizes (short last blocks, 16 and 32 right-hand sides per workgroup, both sides); bit-identical
+    when repeated."""
+    eps = np.finfo(dtype).eps
+    sizes = [(5, 3), (130, 17), (257, 64), (513, 40), (48, 1030), (1100, 530), (37, 4130), (4130, 29)]
+    with gpu.debug_env(CLBLAS_AMD_TRSM_LEAF=1):
+        for vi, (side, uplo, tA, diag) in enumerate(VARIANTS):
+            for (M, N) in sizes[vi % 2::2]:
+                alpha = 0.75
+                A, lda, B, ldb = make_inputs(order, side, uplo, diag, M, N, dtype, 13)
+                want = B.copy()
+                assert oracle.trsm_blocked(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, want, 7, ldb) == 0
+                st, got = gpu.trsm(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, B, 7, ldb)
+                assert st == 0
+                n = M if side == LEFT else N
+                Xg = logical_view(got, order, NOTRANS, M, N, 7, ldb)
+                assert not np.isnan(Xg).any(), "poisoned triangle or unit diagonal was read (%d,%d)" % (M, N)
+                be = backward_error(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, B, got, 7, ldb)
+                assert be <= 2 * n * eps, ((M, N), be)
+                Xw = logical_view(want, order, NOTRANS, M, N, 7, ldb)
+                assert np.abs(Xg - Xw).max() <= 32 * n * eps * np.abs(Xw).max(), (M, N)
+                mask = np.ones(B.size, dtype=bool)
+                logical_view(mask, order, NOTRANS, M, N, 7, ldb)[:] = False
+                np.testing.assert_array_equal(got[mask], B[mask])
+                if vi % 5 == 0:
+                    st, again = gpu.trsm(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, B, 7, ldb)
+                    assert st == 0
+                    np.testing.assert_array_equal(again, got)
