@@ -851,6 +851,18 @@ def main():
                  for _ in range(3))
         others["config1_sgemm_1024"] = {"value": round(2.0 * m1 ** 3 / dt / 1e12, 5), "unit": "TFLOP/s",
                                         "sample": "config 1 in full: SGEMM NN 1024^3, beta=0, best of 3 calls, %.3f s" % dt}
+        # The reference's own CPU code for this operation - the naive gemm its kernel-test tool checks device
+        # results against (src/library/tools/ktest/naive/naive_blas.cpp, compiled from the reference tree by
+        # oracle/Makefile) - on config 1 in full: one thread, a plain triple loop.
+        try:
+            cr = c.copy()
+            dt_ref = clock(lambda: oracle.ref_gemm(COL, NOTRANS, NOTRANS, m1, m1, m1, 1.0, a, m1, b, m1, 0.0, cr, m1))
+            others["config1_sgemm_1024_reference_naive_blas"] = {
+                "value": round(2.0 * m1 ** 3 / dt_ref / 1e12, 6), "unit": "TFLOP/s", "cores": 1, "kind": "reference",
+                "sample": "config 1 in full through the reference's naive_blas.cpp gemm<float>, one call, %.1f s" % dt_ref}
+            del cr
+        except Exception as e:   # the checker library is only there when it was built from the reference tree
+            others["config1_sgemm_1024_reference_naive_blas"] = {"value": None, "sample": "not available: %s" % e}
         m4 = min(n, 2048)               # config 4 on its leading 2048^3 problem (flops scale with M N K: x%d for the whole)
         a = oracle.normal(m4 * m4, SEEDS["dgemm"], np.float64)
         b = oracle.normal(m4 * m4, SEEDS["dgemm"] + 1, np.float64)
