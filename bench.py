@@ -257,6 +257,9 @@ TILE_MODEL_SHAPES = (
     (16384, 128, 2048), (128, 16384, 2048), (4096, 4096, 64), (4096, 4096, 256), (8192, 8192, 128), (6144, 6144, 6144),
     (5120, 5120, 5120), (2048, 2048, 2048), (4096, 4096, 4096), (1536, 1536, 1536),
     (8192, 8192, 8192), (8192, 8192, 2048), (8192, 8192, 512),      # the headline shape and its shorter relatives
+    # beyond 8192: tens of rounds of tiles, edges that are no multiples of a tile, odd leading dimensions
+    (10000, 10000, 10000), (9000, 9000, 9000), (12000, 12000, 4096), (16000, 16000, 2048), (20000, 20000, 8192),
+    (11111, 9999, 5000), (8320, 8320, 8192),
 )
 
 
@@ -268,7 +271,7 @@ def tile_model_block(torch, clblas_amd, gen, keep_forced=False):
     for name, dt, fn, ntiles in (("sgemm", torch.float32, clblas_amd.sgemm, 5), ("dgemm", torch.float64, clblas_amd.dgemm, 2)):
         rows, mispicks, worst, forced = {}, [], 1.0, {}
         for (M, N, K) in TILE_MODEL_SHAPES:
-            if name == "dgemm" and M * N * K > 6.5e10 and M != 8192:
+            if name == "dgemm" and M * N * K > 6.5e10 and M not in (8192, 9000, 10000, 12000):
                 continue
             A = torch.rand(M * K, device="cuda", dtype=dt, generator=gen) * 2 - 1
             B = torch.rand(K * N, device="cuda", dtype=dt, generator=gen) * 2 - 1
@@ -299,6 +302,10 @@ def tile_model_block(torch, clblas_amd, gen, keep_forced=False):
                                  int(re.search(r"tail_slices=(\d+)", desc).group(1))])
                 if best is None or ms < best:
                     best, best_tile, best_dims = ms, tile, dims
+                if desc == default_desc:
+                    # the very launch the default makes, timed a second time: the better of the two counts for
+                    # the default (the first measurement of a shape runs right behind its allocations)
+                    ms_default = min(ms_default, ms)
             tf = lambda ms: round(2.0 * M * N * K / ms / 1e9, 1)
             key = "%dx%dx%d" % (M, N, K)
             rows[key] = [tf(ms_default), default_tile, tf(best), best_dims]

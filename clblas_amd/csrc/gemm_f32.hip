@@ -21,9 +21,12 @@ namespace cba {
 //      7-9 % slower with them).
 //   The parameters of the choice model (efficiency, fixed time per workgroup as a depth k0, price of a sliced
 //   tail) were last refitted with clblas_amd/fit_tile_model.py on bench.py --only tilemodel: the 256x128 tile
-//   got k0 = 80 (on large C with K of a few hundred the 128x128 tile is ahead: 8192 x 8192 x 128 +3.5 %,
+//   has a k0 (on large C with K of a few hundred the 128x128 tile is ahead: 8192 x 8192 x 128 +3.5 %,
 //   4096 x 4096 x 64 +1.3 %), the 128x128 tile's sliced tail 0.12 -> 0.07, the 64x64 tile .86 -> .88
-//   (5000 x 1000 x 1000 +7 %, 4200 x 1700 x 900 +3 %).
+//   (5000 x 1000 x 1000 +7 %, 4200 x 1700 x 900 +3 %).  With shapes beyond 8192 in the set (tens of rounds of
+//   tiles, edges that are no multiples of a tile) the 256x128 tile went from (.942, k0 80, tail .05) to
+//   (.952, 40, .03): 10000^3, 16000 x 16000 x 2048 and 20000 x 20000 x 8192 had been given 128x64 tiles
+//   and ran 8-11 % behind (its credit for plain products only: the triangular forms keep .942).
 //   4:  64x64x32,  wave 32x32, split-K capable (small / deep-K problems; 1024^3: 94 against 86 with
 //      depth 16, 8192 x 64 x 8192: 106-112 against 91-94); with panels of depth 64 where a workgroup's K
 //      range is at least 1024 (1024^3 95.4 -> 99.0 TFLOP/s, 1024 x 1024 x 2048 109 -> 115, 960 x 960 x 2048
@@ -31,7 +34,7 @@ namespace cba {
 // (Not const: clblasAmdTileModelParam lets the fitting script vary the model's parameters; the launch path only reads.)
 static TileEntry<float> *f32_tiles(int *n) {
     static TileEntry<float> tab[] = {
-        make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.942, 0.85, -1.0, 80.0),
+        make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.952, 0.85, 0.942, 40.0, 0.03, 0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.07),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0),
         make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.97, 0.0),

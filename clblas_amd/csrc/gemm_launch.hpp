@@ -302,7 +302,10 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         // The smallest tile, when even it cannot give every CU a workgroup, takes the number of ranges
         // that the same model prices lowest, one range included (short K: the pass that adds the
         // ranges up costs more than the idle CUs; 960 x 960 x 256 FP64 22 -> 14 us, 512^3 18 -> 15 us).
-        // A larger tile is split only where the model puts it 3 % ahead of what would run otherwise.
+        // A larger tile is split only where the model puts it 8 % ahead of what would run otherwise (the model
+        // is hard on one round of unsplit small tiles over a deep K: DGEMM 1024 x 1024 x 8192 and 2048 x 512 x 8192
+        // run 69.1 TFLOP/s on 256 tiles of 64x64 and 66.6 on 128x128 tiles in 8 ranges, which it had 7 % ahead;
+        // 896 x 896 x 8192, 60.4 against 53.1 the other way, it has further ahead than that).
         const int last = ntab - 1;
         int last_splits = -1;  // -1: the rule without the model
         if (split_model && pick == last && tab[last].has_splitk) {
@@ -321,7 +324,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             }
         }
         if (pick_of_split >= 0) {
-            if (best_split * 1.03 < best) pick = pick_of_split;
+            if (best_split * 1.08 < best) pick = pick_of_split;
             else pick_of_split = -1;
         }
         pick_split = pick == last || pick == pick_of_split;
