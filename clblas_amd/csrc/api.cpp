@@ -51,6 +51,7 @@ void read_knobs() {
     k.log = env_int("CLBLAS_AMD_LOG", 0);
     k.check_mem = env_int("CLBLAS_AMD_CHECK_MEM", 0);
     k.trsm_leaf = env_int("CLBLAS_AMD_TRSM_LEAF", 0);
+    k.trsm_wide = env_int("CLBLAS_AMD_TRSM_WIDE", -1);
     k.trsm_poll_limit = env_int("CLBLAS_AMD_TRSM_POLL_LIMIT", 0);
     g_knobs = k;
 }

@@ -1133,15 +1133,24 @@ template <typename T> struct TrsmDriver {
         const int poll_limit = knobs().trsm_poll_limit > 0 ? knobs().trsm_poll_limit : (1 << 22);
         return launch_kernel(fn, grid, block, L::SMEM, stream, packed, nb, alpha, Bblk, ldb, nrhs, poll_limit);
     }
-    // Right-hand sides per workgroup.  Real types: 16, or 32 for FP32 (each sub-block of coefficients is then
-    // used twice) when 16 would make more than one round of workgroups anyway (more than 256 x 16
-    // right-hand sides) or with side = right, whose right-hand sides are rows of B: 16 floats are too
-    // short a run of memory.
+    // Right-hand sides per workgroup.  Real types: 16, or 32 (each sub-block of coefficients is then
+    // used twice) where that makes the launch shorter, or for FP32 with side = right, whose right-hand sides
+    // are rows of B: 16 floats are too short a run of memory.  A leaf kernel has a CU to itself and lasts
+    // about as long whatever the number of workgroups in its round, so a launch costs rounds x time per
+    // round: FP64 30 us with 16 and 52 us with 32 right-hand sides per workgroup, FP32 21 and 34.  One round
+    // of 32 beats two of 16 (4097 .. 8192 right-hand sides), two rounds of 32 lose against three of 16
+    // (8193 .. 12288: DTRSM 9216 64.0 -> 66.6 TFLOP/s), and so on.
+    static bool wide_leaf_pays(int nrhs) {
+        const int64_t rounds16 = ((int64_t)(nrhs + 15) / 16 + 255) / 256, rounds32 = ((int64_t)(nrhs + 31) / 32 + 255) / 256;
+        const double wide_over_narrow = sizeof(R) == 8 ? 52.0 / 30.0 : 34.0 / 21.0;
+        return (double)rounds32 * wide_over_narrow < (double)rounds16;
+    }
     hipError_t leaf(int i0, int nb, T alpha) {
         const int nrhs = right ? M : N;
         if constexpr (!Elem<T>::CPLX) {
             if (!inv_leaf) {
-                const bool wide = nrhs > 256 * 16 || (right && sizeof(R) == 4);
+                bool wide = wide_leaf_pays(nrhs) || (right && sizeof(R) == 4);
+                if (knobs().trsm_wide >= 0) wide = knobs().trsm_wide != 0;
                 if (wide) return right ? leaf_side<true, true>(i0, nb, alpha) : leaf_side<false, true>(i0, nb, alpha);
                 return right ? leaf_side<true, false>(i0, nb, alpha) : leaf_side<false, false>(i0, nb, alpha);
             }

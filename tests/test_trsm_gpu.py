@@ -159,6 +159,39 @@ def test_config5_dtrsm_8192(gpu):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_several_rounds_of_leaf_workgroups(gpu, dtype):
+    """More right-hand sides than one round of leaf workgroups takes, in the ranges where the launch is priced
+    for 16 per workgroup (8193 .. 12288: three rounds) and for 32 (12289 .. 16384: two rounds), both sides,
+    a diagonal block and a half; and each width forced on the other's range (CLBLAS_AMD_TRSM_WIDE).  Same
+    bars as test_all_variants."""
+    eps = np.finfo(dtype).eps
+    cases = [(LEFT, 40, 8300), (LEFT, 530, 8300), (RIGHT, 8300, 40), (RIGHT, 8300, 530), (LEFT, 40, 12500),
+             (RIGHT, 12500, 40)]
+    for ci, (side, M, N) in enumerate(cases):
+        uplo, tA, diag = [(LOWER, NOTRANS, NONUNIT), (UPPER, TRANS, NONUNIT), (UPPER, NOTRANS, UNIT)][ci % 3]
+        order = COL if ci % 2 == 0 else ROW
+        alpha = 0.75
+        A, lda, B, ldb = make_inputs(order, side, uplo, diag, M, N, dtype, 17)
+        want = B.copy()
+        assert oracle.trsm_blocked(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, want, 7, ldb) == 0
+        n = M if side == LEFT else N
+        Xw = logical_view(want, order, NOTRANS, M, N, 7, ldb)
+        for forced in (None, 0, 1):
+            env = {} if forced is None else {"CLBLAS_AMD_TRSM_WIDE": forced}
+            with gpu.debug_env(**env):
+                st, got = gpu.trsm(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, B, 7, ldb)
+            assert st == 0
+            Xg = logical_view(got, order, NOTRANS, M, N, 7, ldb)
+            assert not np.isnan(Xg).any(), "poisoned triangle or unit diagonal was read (%d,%d)" % (M, N)
+            be = backward_error(order, side, uplo, tA, diag, M, N, alpha, A, 5, lda, B, got, 7, ldb)
+            assert be <= 2 * n * eps, ((M, N), forced, be)
+            assert np.abs(Xg - Xw).max() <= 32 * n * eps * np.abs(Xw).max(), (M, N, forced)
+            mask = np.ones(B.size, dtype=bool)
+            logical_view(mask, order, NOTRANS, M, N, 7, ldb)[:] = False
+            np.testing.assert_array_equal(got[mask], B[mask])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("order", [ROW, COL])
 def test_inverted_triangle_leaf_behind_its_switch(gpu, dtype, order):
     """The other way of solving a diagonal block (real types): 64 x 64 triangles inverted by doubling in the
