@@ -259,7 +259,7 @@ TILE_MODEL_SHAPES = (
     (8192, 8192, 8192), (8192, 8192, 2048), (8192, 8192, 512),      # the headline shape and its shorter relatives
     # beyond 8192: tens of rounds of tiles, edges that are no multiples of a tile, odd leading dimensions
     (10000, 10000, 10000), (9000, 9000, 9000), (12000, 12000, 4096), (16000, 16000, 2048), (20000, 20000, 8192),
-    (11111, 9999, 5000), (8320, 8320, 8192),
+    (11111, 9999, 5000), (8320, 8320, 8192), (20000, 20000, 256), (12000, 12000, 512), (16000, 16000, 128),
 )
 
 

@@ -26,7 +26,9 @@ namespace cba {
 //   (5000 x 1000 x 1000 +7 %, 4200 x 1700 x 900 +3 %).  With shapes beyond 8192 in the set (tens of rounds of
 //   tiles, edges that are no multiples of a tile) the 256x128 tile went from (.942, k0 80, tail .05) to
 //   (.952, 40, .03): 10000^3, 16000 x 16000 x 2048 and 20000 x 20000 x 8192 had been given 128x64 tiles
-//   and ran 8-11 % behind (its credit for plain products only: the triangular forms keep .942).
+//   and ran 8-11 % behind (its credit for plain products only: the triangular forms keep .942); and the
+//   128x64 / 64x128 tiles got k0 = 10 (20000 x 20000 x 256 and 16000 x 16000 x 128 ran 3.5 and 8 % behind the
+//   128x128 tile with them, 6000 x 6000 x 640 2.8 %).
 //   4:  64x64x32,  wave 32x32, split-K capable (small / deep-K problems; 1024^3: 94 against 86 with
 //      depth 16, 8192 x 64 x 8192: 106-112 against 91-94); with panels of depth 64 where a workgroup's K
 //      range is at least 1024 (1024^3 95.4 -> 99.0 TFLOP/s, 1024 x 1024 x 2048 109 -> 115, 960 x 960 x 2048
@@ -36,8 +38,8 @@ static TileEntry<float> *f32_tiles(int *n) {
     static TileEntry<float> tab[] = {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.952, 0.85, 0.942, 40.0, 0.03, 0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.07),
-        make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0),
-        make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.97, 0.0),
+        make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.97, 0.0, 10.0),
+        make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.97, 0.0, 10.0),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64, true>(0.88, 0.95),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

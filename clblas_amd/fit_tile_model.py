@@ -10,8 +10,8 @@ is credited with), `alone` (factor when a workgroup has its CU to itself), `k0` 
 workgroup, as a depth) and `tail_extra` (price of a sliced last round, in rounds).  This script takes the
 times of every forced tile on every shape from bench.py, evaluates the library's own model through
 clblasAmdTileModelQuery with trial parameters set through clblasAmdTileModelParam - the model is not
-restated here - and searches, one parameter at a time over a grid around its present value, for the
-setting with the least regret
+restated here - and searches, one step of one parameter at a time over a grid around its present value
+(always the step that helps most), for the setting with the least regret
 
     regret = sum over shapes of  time(tile the model picks) / time(best tile) - 1,
 
@@ -59,22 +59,45 @@ def regret(letter, shapes, detail=False):
     return (total, rows) if detail else total
 
 
-def fit(letter, shapes, ntiles, sweeps=4):
+def twins(letter, ntiles):
+    """Tiles that are each other's transpose (128x64 and 64x128) and carry the same parameters are moved
+    together: changing one of a pair alone only hands its picks to the other.  {first tile: [tiles]}."""
+    dims = [tuple(int(x) for x in d.split("x")) for d in clblas_amd.tile_model_query(letter, 1024, 1024, 1024)["tiles"]]
+    params = [[clblas_amd.tile_model_param(letter, t, p) for p in GRIDS] for t in range(ntiles)]
+    groups, seen = {}, set()
+    for t in range(ntiles):
+        if t in seen:
+            continue
+        groups[t] = [u for u in range(t, ntiles) if u == t or (params[u] == params[t] and dims[u][:2] == dims[t][1::-1]
+                                                                 and dims[u][2] == dims[t][2])]
+        seen.update(groups[t])
+    return groups
+
+
+def fit(letter, shapes, ntiles, sweeps=12):
+    """Steepest descent over single steps: every round tries each step of each parameter of each tile
+    (twins together) from where the model stands, takes the one that lowers the regret most - the smaller
+    step on a tie - and stops when none lowers it.  So the parameters move as little as the times ask for."""
+    groups = twins(letter, ntiles)
     for _ in range(sweeps):
-        improved = False
-        for tile in range(ntiles):
+        base = regret(letter, shapes)
+        best = None  # (regret, relative size of the step, group, name, value)
+        for tile, group in groups.items():
             for name, steps in GRIDS.items():
                 here = clblas_amd.tile_model_param(letter, tile, name)
-                best_v, best_r = here, regret(letter, shapes)
-                for d in sorted(steps, key=abs):   # the smallest change that gives the least regret
+                for d in steps:
                     v = min(max(here + d, LIMITS[name][0]), LIMITS[name][1])
-                    clblas_amd.tile_model_param(letter, tile, name, v)
-                    r = regret(letter, shapes)
-                    if r < best_r - 1e-9:
-                        best_v, best_r, improved = v, r, True
-                clblas_amd.tile_model_param(letter, tile, name, best_v)
-        if not improved:
+                    for t in group:
+                        clblas_amd.tile_model_param(letter, t, name, v)
+                    cand = (regret(letter, shapes), abs(d) / max(abs(x) for x in steps), group, name, v)
+                    if cand[0] < base - 1e-9 and (best is None or cand[:2] < best[:2]):
+                        best = cand
+                for t in group:
+                    clblas_amd.tile_model_param(letter, t, name, here)
+        if best is None:
             break
+        for t in best[2]:
+            clblas_amd.tile_model_param(letter, t, best[3], best[4])
 
 
 def main(path):
