@@ -260,6 +260,9 @@ TILE_MODEL_SHAPES = (
     # beyond 8192: tens of rounds of tiles, edges that are no multiples of a tile, odd leading dimensions
     (10000, 10000, 10000), (9000, 9000, 9000), (12000, 12000, 4096), (16000, 16000, 2048), (20000, 20000, 8192),
     (11111, 9999, 5000), (8320, 8320, 8192), (20000, 20000, 256), (12000, 12000, 512), (16000, 16000, 128),
+    # one or two rows / columns of tiles over a deep K: the operand that is streamed from HBM is read once
+    (10000, 100, 10000), (100, 10000, 10000), (12000, 100, 3000), (16384, 64, 10000), (5000, 200, 8192),
+    (100, 5000, 20000), (7000, 300, 5000), (30000, 40, 3000), (9000, 130, 9000), (50000, 50, 5000), (20000, 200, 4096),
 )
 
 

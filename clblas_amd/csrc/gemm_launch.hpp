@@ -22,6 +22,7 @@ template <typename T> struct TileEntry {
     // round of workgroups: see where the variant is chosen).
     int bk_deep;
     double deep_gain;  // factor on `eff` where the deep form runs (plain products, K range from 1024)
+    double split_gain; // factor on `eff` in a launch that cuts K into ranges (the 64x128 FP32 tile: 4-6 % ahead of 128x64 there, behind it everywhere else)
     size_t smem_deep[4];
     void (*plain_deep[4])(const GemmParams<T>);
     void (*splitk_deep[4])(const GemmParams<T>);
@@ -60,6 +61,7 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
     typedef GemmCfg<T, BM, BN, BK, WM, WN, false, false> Cfg;
     TileEntry<T> e;
     e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK;
+    e.split_gain = 1.0;
     e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri; e.k0 = k0; e.tail_extra = tail_extra;
     e.eff_tri_c = eff_tri_c < 0 ? eff : eff_tri_c;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
@@ -257,10 +259,15 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
     } else {
         // Cost of tile i with its depth cut into s ranges: the ranges fill the CUs that the tiles
         // alone leave idle, at the price of the pass that adds them up.
+        // Operands beyond the 256 MB of the memory-side cache are streamed from HBM, and a workgroup alone on
+        // its CU then has too few loads in flight for the latency: SGEMM 16384 x 64 x 10000 (655 MB of A, one
+        // 64x64 tile per CU) runs at 105 TFLOP/s where 1024 x 1024 x 8192 (64 MB, the same 256 tiles) runs at 125.
+        const bool streamed = ((double)M * K + (double)K * N) * sizeof(T) > 256e6;
+        const double lone_stream = streamed ? 0.85 : 1.0;
         auto split_cost = [&](int i, int64_t t, int s) {
-            const double alone = t * s <= kCUs ? tab[i].alone : 1.0;
+            const double alone = t * s <= kCUs ? tab[i].alone * lone_stream : 1.0;
             const double deep = (tab[i].bk_deep > 0 && (K / s >= 1024 || (K / s >= 512 && t * s <= kCUs))) ? tab[i].deep_gain : 1.0;
-            return (double)ceil_div64(t * s, kCUs) * tab[i].bm * tab[i].bn / (s * tab[i].eff * deep * alone) +
+            return (double)ceil_div64(t * s, kCUs) * tab[i].bm * tab[i].bn / (s * tab[i].eff * tab[i].split_gain * deep * alone) +
                    split_overhead_cost<T>(M, N, K, s);
         };
         const bool split_model = knobs().split_model != 0 && !need_tri;
@@ -275,7 +282,15 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
             // A sliced tail round lasts 1 / ts of a round plus what does not shrink with the depth of a slice
             // (its first loads, the partial tiles written and added up by a second pass): about 120 deep.
-            if (ts > 1) rounds = (double)(t / kCUs) + 1.0 / ts + tab[i].tail_extra + 120.0 / K;
+            if (ts > 1) {
+                // With a single whole round every CU holds one whole tile next to its slice, and once the slice
+                // is done that tile runs at the rate of a workgroup alone - which matters where the operands are
+                // streamed: SGEMM 10000 x 100 x 10000 on 64x64 tiles, 256 whole + 58 x 4 slices, takes 1.25 x the
+                // 0.199 ms of 16384 x 64 x 10000 (one tile per CU), 1.7 rounds at the pair rate, not 1.3;
+                // 5000 x 200 x 8192 (164 MB, each panel of A used by four tiles) takes the 1.3.
+                const double lone = (streamed && t / kCUs == 1) ? (tab[i].alone < 0.8 ? tab[i].alone : 0.8) : 1.0;
+                rounds = ((double)(t / kCUs) + 1.0 / ts) / lone + tab[i].tail_extra + 120.0 / K;
+            }
             // A triangular operand makes the tiles differ in depth (half of the full depth on
             // average, started deepest first): the CUs share the total evenly up to a fraction
             // of one full-depth tile, fitted to STRMM / DTRMM 4096 and 8192 (STRMM 4096: 256x128
@@ -286,7 +301,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             // than the deeper panels gain - 2000^3 FP32 128 TFLOP/s with 128x64 tiles, 119 with 64x64)
             if (!need_tri && ts <= 1 && tab[i].bk_deep > 0 && ((K >= 1024 && t <= 3 * kCUs) || (K >= 512 && t <= kCUs))) eff *= tab[i].deep_gain;
             double cost = rounds * tab[i].bm * tab[i].bn / eff;
-            if (t <= kCUs) cost /= tab[i].alone;  // a workgroup alone on its CU cannot keep the MFMA pipes full
+            if (t <= kCUs) cost /= tab[i].alone * lone_stream;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             cost *= 1.0 + tab[i].k0 / K;
             if (costs_out) costs_out[i] = cost;
             if (!have || cost < best) { best = cost; pick = i; have = true; }
@@ -302,7 +317,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         // The smallest tile, when even it cannot give every CU a workgroup, takes the number of ranges
         // that the same model prices lowest, one range included (short K: the pass that adds the
         // ranges up costs more than the idle CUs; 960 x 960 x 256 FP64 22 -> 14 us, 512^3 18 -> 15 us).
-        // A larger tile is split only where the model puts it 8 % ahead of what would run otherwise (the model
+        // A larger tile is split only where the model puts it 10 % ahead of what would run otherwise (the model
         // is hard on one round of unsplit small tiles over a deep K: DGEMM 1024 x 1024 x 8192 and 2048 x 512 x 8192
         // run 69.1 TFLOP/s on 256 tiles of 64x64 and 66.6 on 128x128 tiles in 8 ranges, which it had 7 % ahead;
         // 896 x 896 x 8192, 60.4 against 53.1 the other way, it has further ahead than that).
@@ -324,7 +339,10 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             }
         }
         if (pick_of_split >= 0) {
-            if (best_split * 1.08 < best) pick = pick_of_split;
+            // (the margin is for a split against an unsplit launch; where the smallest tile is itself cut into
+            // ranges both pay the pass that adds them up, and the prices are compared as they are)
+            const double margin = (pick == last && last_splits > 1) ? 1.0 : 1.10;
+            if (best_split * margin < best) pick = pick_of_split;
             else pick_of_split = -1;
         }
         pick_split = pick == last || pick == pick_of_split;
@@ -546,7 +564,13 @@ static void model_query(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
     *tail_slices = (*splits <= 1 && e.tri[0]) ? tail_slices_for(ntiles, K, e.bk, knobs().tail != 0) : 1;
 }
 
-// One parameter of the choice model of tile `i`: 0 eff, 1 alone, 2 k0, 3 tail_extra, 4 deep_gain.
+// A table entry with its credit in launches that cut K set (see TileEntry::split_gain).
+template <typename T> static TileEntry<T> with_split_gain(TileEntry<T> e, double g) {
+    e.split_gain = g;
+    return e;
+}
+
+// One parameter of the choice model of tile `i`: 0 eff, 1 alone, 2 k0, 3 tail_extra, 4 deep_gain, 5 split_gain.
 template <typename T> static double *model_param(TileEntry<T> *tab, int ntab, int i, int which) {
     if (i < 0 || i >= ntab) return nullptr;
     switch (which) {
@@ -555,6 +579,7 @@ template <typename T> static double *model_param(TileEntry<T> *tab, int ntab, in
         case 2: return &tab[i].k0;
         case 3: return &tab[i].tail_extra;
         case 4: return &tab[i].deep_gain;
+        case 5: return &tab[i].split_gain;
         default: return nullptr;
     }
 }

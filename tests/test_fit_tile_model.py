@@ -22,6 +22,7 @@ def synthetic_block(letter):
         assert q["splits"] == 1
         forced["%dx%dx%d" % (M, N, K)] = {"default_splits": 1,
                                           "tiles": [[c * K * 1e-9, 1, 1] for c in q["costs"]]}
+    # (none of these shapes cuts K, so every pick is one of the timed launches)
     return {"forced_ms": forced}
 
 
@@ -66,5 +67,5 @@ def test_main_prints_a_report(tmp_path, capsys, restore_params):
     path.write_text(json.dumps({"extra": {"tile_model": {"sgemm": synthetic_block("s"), "dgemm": synthetic_block("d")}}}))
     fit_tile_model.main(str(path))
     out = capsys.readouterr().out
-    assert "== sgemm: %d shapes fitted" % len(SHAPES) in out and "== dgemm" in out
+    assert "== sgemm: %d shapes" % len(SHAPES) in out and "== dgemm" in out
     assert "regret 0.0000 -> 0.0000" in out
