@@ -490,8 +490,13 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     {
         const int64_t wgs = grid_x * (splits > 1 ? splits : 1);
         const bool whole_rounds = p.tail_slices <= 1 && wgs % 512 == 0;
-        const int mode = knobs().stagger;  // 0: never
-        p.stagger = mode != 0 && wgs > 512 && !(p.tri_a || p.tri_b) && (!whole_rounds || p.k_per_split <= 2048);
+        const int mode = knobs().stagger;  // 0: never, 2: whatever the type
+        // FP64 only: with the sliced tail in place the FP32 kernels gain nothing from it any more (35 shapes, on
+        // against off: within 0.5 % either way) and the 128x64 tile loses 8-10 % with it on TN operands
+        // (3000^3 120 against 131 TFLOP/s, 3072^3 127 against 138, 3328^3 124 against 139), while DGEMM still takes
+        // + 2.4 % at 8192 x 8192 x 512, + 1.3 % at 12000 x 12000 x 512 and + 7 % at 4200 x 1700 x 900 from it.
+        const bool type_gains = sizeof(typename Elem<T>::Real) == 8 || mode == 2;
+        p.stagger = mode != 0 && type_gains && wgs > 512 && !(p.tri_a || p.tri_b) && (!whole_rounds || p.k_per_split <= 2048);
     }
     size_t smem = e.smem_of[idx];
     const int threads = e.threads;
