@@ -483,20 +483,21 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
             fn = wide ? e.splitk_wide[idx] : e.splitk[idx];
         }
     }
-    // The late start that keeps the workgroups of a CU out of lockstep (see the kernel).  Needed when
-    // the launch is not a whole number of rounds of 2 x 256 workgroups (3584^3 FP64: 54 -> 69 TFLOP/s);
-    // with short K ranges it also pays in whole rounds, because the epilogue of one workgroup then
-    // overlaps the K loop of its neighbour (8192 x 8192 x 512 FP64: 66.9 -> 68.2; x 8192: -0.3 %).
+    // The late start that keeps the workgroups of a CU out of lockstep (see the kernel).  It was needed
+    // where a launch is not a whole number of rounds of 2 x 256 workgroups (3584^3 FP64: 54 -> 69 TFLOP/s)
+    // until the sliced tail took that case over; what is left of it is the gain with short K ranges, where
+    // the epilogue of one workgroup overlaps the K loop of its neighbour (8192 x 8192 x 512 FP64: 66.6 -> 68.2).
     {
         const int64_t wgs = grid_x * (splits > 1 ? splits : 1);
-        const bool whole_rounds = p.tail_slices <= 1 && wgs % 512 == 0;
         const int mode = knobs().stagger;  // 0: never, 2: whatever the type
         // FP64 only: with the sliced tail in place the FP32 kernels gain nothing from it any more (35 shapes, on
         // against off: within 0.5 % either way) and the 128x64 tile loses 8-10 % with it on TN operands
         // (3000^3 120 against 131 TFLOP/s, 3072^3 127 against 138, 3328^3 124 against 139), while DGEMM still takes
         // + 2.4 % at 8192 x 8192 x 512, + 1.3 % at 12000 x 12000 x 512 and + 7 % at 4200 x 1700 x 900 from it.
         const bool type_gains = sizeof(typename Elem<T>::Real) == 8 || mode == 2;
-        p.stagger = mode != 0 && type_gains && wgs > 512 && !(p.tri_a || p.tri_b) && (!whole_rounds || p.k_per_split <= 2048);
+        // ... and only with K ranges of up to 2048: beyond that it is neutral or costs a percent (DGEMM 3072^3
+        // 71.4 -> 70.5, 2560^3 68.6 -> 68.0; 3584^3, 3700^3, 5000^3, 6000^3, 6144^3 within 0.3 %).
+        p.stagger = mode != 0 && type_gains && wgs > 512 && !(p.tri_a || p.tri_b) && p.k_per_split <= 2048;
     }
     size_t smem = e.smem_of[idx];
     const int threads = e.threads;
