@@ -384,7 +384,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, trsm, vendor, tiles or copy "
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, big, trsm, vendor, tiles or copy "
                     "(profiling; copy = a plain 1 GiB device copy used to scale the HBM traffic counters; tiles = every tile "
                     "the five configurations use, --steps times each, for the counter profile)")
     args = ap.parse_args()
@@ -713,6 +713,49 @@ def main():
                     "torch_mm_tflops": round(2.0 * M * N * K / vendor_ms / 1e9, 2)}
                 del A, B, C
         extra["small_c_deep_k"] = dk
+
+    # ---- Beyond 8192: the part has 288 GB, and matrices of 16384 .. 32768 are ordinary there (1 .. 8.6 GB each).
+    #      Column-major NN / left-lower-notrans-nonunit, alpha = beta = 1, tight leading dimensions. ----
+    if args.only in ("", "big"):
+        big = {}
+        for name, dt, fn, peak, n, reps in (("sgemm 16384", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, 16384, 3),
+                                            ("dgemm 16384", torch.float64, clblas_amd.dgemm, PEAK_FP64_MATRIX, 16384, 2),
+                                            ("sgemm 32768", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, 32768, 1),
+                                            ("sgemm 20000x20000x8192", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, (20000, 20000, 8192), 3)):
+            M, N, K = n if isinstance(n, tuple) else (n, n, n)
+            A = torch.rand(M * K, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            B = torch.rand(K * N, device="cuda", dtype=dt, generator=gen) * 2 - 1
+            C = torch.zeros(M * N, device="cuda", dtype=dt)
+
+            def call():
+                st = fn(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, C, 0, M)
+                if st != 0:
+                    raise RuntimeError("clblas %s returned %d" % (name, st))
+            ms = timed_batch(torch, call, reps, 1, batches=2)
+            tf = 2.0 * M * N * K / ms / 1e9
+            big[name] = {"ms": round(ms, 3), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
+                         "kernel": clblas_amd.last_dispatch()[0]}
+            del A, B, C
+        for name, dt, fn, peak, n in (("dtrsm 16384", torch.float64, clblas_amd.dtrsm, PEAK_FP64_MATRIX, 16384),
+                                      ("strsm 16384", torch.float32, clblas_amd.strsm, PEAK_FP32_MATRIX, 16384),
+                                      ("dtrsm 12000", torch.float64, clblas_amd.dtrsm, PEAK_FP64_MATRIX, 12000)):
+            A = (torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1) / n
+            A.view(n, n).diagonal().copy_(torch.rand(n, device="cuda", dtype=dt, generator=gen) + 1)
+            B = torch.randn(n * n, device="cuda", dtype=dt, generator=gen)
+
+            def call():
+                st = fn(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, A, 0, n, B, 0, n)
+                if st != 0:
+                    raise RuntimeError("clblas %s returned %d" % (name, st))
+            n0 = clblas_amd.last_dispatch()[1]
+            call()
+            launches = clblas_amd.last_dispatch()[1] - n0
+            ms = timed_batch(torch, call, 2, 0, batches=2)
+            tf = n * (n + 1.0) * n / ms / 1e9
+            big[name] = {"ms": round(ms, 3), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
+                         "kernels_per_call": launches, "finite": bool(torch.isfinite(B).all())}
+            del A, B
+        extra["beyond_8192"] = big
 
     # ---- TRSM below 8192 (left, lower, no transpose, non-unit; square B, alpha = 1): a chain of short
     #      dependent launches (packing pass, leaves of 512 equations, GEMM updates).  Each solve overwrites B
