@@ -577,308 +577,320 @@ def main():
             extra["dtrsm"]["pct_of_dgemm_rate"] = round(100 * t_tflops / d_tflops, 2)
         del A, B, B0
 
-    # ---- CGEMM / ZGEMM at the same size (no BASELINE configuration; the neighbours of the path) ----
-    for name, dt, fn, peak in (("cgemm", torch.complex64, clblas_amd.cgemm, PEAK_FP32_MATRIX),
-                               ("zgemm", torch.complex128, clblas_amd.zgemm, PEAK_FP64_MATRIX)):
-        if args.only not in ("", name):
-            continue
-        rdt = torch.float32 if dt == torch.complex64 else torch.float64
-        A, B, C = (torch.view_as_complex(torch.rand(n * n, 2, device="cuda", dtype=rdt, generator=gen) * 2 - 1)
-                   for _ in range(3))
-
-        def cgemm():
-            st = fn(COL, NOTRANS, NOTRANS, n, n, n, 1.0 + 0.5j, A, 0, n, B, 0, n, 0.5 - 0.25j, C, 0, n)
-            if st != 0:
-                raise RuntimeError("clblas%s returned %d" % (name, st))
-
-        csteps = max(3, steps // 2)
-        wall, ev_ms = timed_calls(torch, cgemm, csteps, 2)
-        c_tflops = 8.0 * n * n * n / (ev_ms * 1e-3) / 1e12
-        extra[name] = {"workload": "%s column-major NN %d^3, alpha=1+0.5i, beta=0.5-0.25i, uniform[-1,1)" % (name.upper(), n),
-                       "tflops": round(c_tflops, 3), "launch_ms": round(ev_ms, 4),
-                       "pct_of_matrix_peak": round(100 * c_tflops / peak, 2)}
-        del A, B, C
-
-    # ---- SYRK / TRMM / SYMM / SYR2K and the complex-only routines at the same size (useful flops only: the reference client's counts) ----
-    if args.only in ("", "level3"):
-        lv = {}
-        for pre, dt, peak in (("S", torch.float32, PEAK_FP32_MATRIX), ("D", torch.float64, PEAK_FP64_MATRIX)):
-            A = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
-            B0 = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
-            B = B0.clone()
-            C = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
-            cases = (
-                ("syrk", float(n) * (n + 1) * n, None,
-                 lambda: clblas_amd.syrk(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, 1.0, C, 0, n)),
-                ("trmm", float(n) * (n + 1) * n, lambda: B.copy_(B0),
-                 lambda: clblas_amd.trmm(pre, COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, A, 0, n, B, 0, n)),
-                ("symm", 2.0 * n * n * n, None,
-                 lambda: clblas_amd.symm(pre, COL, LEFT, LOWER, n, n, 1.0, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
-                ("syr2k", 2.0 * n * n * n + n, None,
-                 lambda: clblas_amd.syr2k(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
-            )
-            for name, fl, before, fn in cases:
-                def call(fn=fn, name=name):
-                    st = fn()
-                    if st != 0:
-                        raise RuntimeError("clblas%s%s returned %d" % (pre, name, st))
-                wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 2, before_each=before)
-                tf = fl / (ev_ms * 1e-3) / 1e12
-                lv[pre.lower() + name] = {"tflops": round(tf, 2), "ms_per_call": round(ev_ms, 4),
-                                          "pct_of_matrix_peak": round(100 * tf / peak, 1)}
-            del A, B, B0, C
-        # complex types: the Hermitian routines and the triangular solve (flop counts of the reference client)
-        for pre, dt, peak in (("C", torch.complex64, PEAK_FP32_MATRIX), ("Z", torch.complex128, PEAK_FP64_MATRIX)):
+    # Everything from here to the CPU baseline is beside the point of the line (the three BASELINE workloads
+    # above are its point): if one of these blocks raises, the blocks after it are skipped, the error is
+    # recorded in `extra.extras_error` and on stderr, and the line is printed all the same.
+    try:
+        # ---- CGEMM / ZGEMM at the same size (no BASELINE configuration; the neighbours of the path) ----
+        for name, dt, fn, peak in (("cgemm", torch.complex64, clblas_amd.cgemm, PEAK_FP32_MATRIX),
+                                   ("zgemm", torch.complex128, clblas_amd.zgemm, PEAK_FP64_MATRIX)):
+            if args.only not in ("", name):
+                continue
             rdt = torch.float32 if dt == torch.complex64 else torch.float64
-            A, B0, C = (torch.view_as_complex(torch.rand(n * n, 2, device="cuda", dtype=rdt, generator=gen) * 2 - 1)
-                        for _ in range(3))
-            B = B0.clone()
-            T = A / n  # well-conditioned triangle: small off-diagonal entries, diagonal in [1, 2)
-            T.view(n, n).diagonal().copy_(torch.rand(n, device="cuda", dtype=rdt, generator=gen) + 1)
-            trsm = clblas_amd.ctrsm if pre == "C" else clblas_amd.ztrsm
-            cases = (
-                ("herk", 4.0 * n * n * (n + 1), None,
-                 lambda: clblas_amd.herk(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, 1.0, C, 0, n)),
-                ("her2k", 8.0 * n * n * n + 2 * n, None,
-                 lambda: clblas_amd.her2k(pre, COL, LOWER, NOTRANS, n, n, 1.0 + 0.5j, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
-                ("hemm", 8.0 * n * n * n, None,
-                 lambda: clblas_amd.hemm(pre, COL, LEFT, LOWER, n, n, 1.0 + 0.5j, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
-                ("trsm", 4.0 * n * (n + 1) * n, lambda: B.copy_(B0),
-                 lambda: trsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, T, 0, n, B, 0, n)),
-            )
-            for name, fl, before, fn in cases:
-                def call(fn=fn, name=name):
-                    st = fn()
-                    if st != 0:
-                        raise RuntimeError("clblas%s%s returned %d" % (pre, name, st))
-                wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 2, before_each=before)
-                tf = fl / (ev_ms * 1e-3) / 1e12
-                lv[pre.lower() + name] = {"tflops": round(tf, 2), "ms_per_call": round(ev_ms, 4),
-                                          "pct_of_matrix_peak": round(100 * tf / peak, 1)}
-            if not bool(torch.isfinite(torch.view_as_real(B)).all().item()):
-                raise RuntimeError("clblas%strsm produced non-finite values" % pre)
-            del A, B, B0, C, T
-        lv["workload"] = "column-major, lower, left, no transpose, N=M=K=%d, alpha=beta=1 (complex: alpha=1+0.5i)" % n
-        extra["level3"] = lv
+            A, B, C = (torch.view_as_complex(torch.rand(n * n, 2, device="cuda", dtype=rdt, generator=gen) * 2 - 1)
+                       for _ in range(3))
 
-    # ---- BASELINE configs 1 and 3: SGEMM 1024^3 and the edge-shape sweep (ld = rows + 3, offsets 5/7/11,
-    #      alpha = 0.7, beta = -1.3, all four transposes).  Each against its own bound: MFMA time and HBM time
-    #      of the algorithmic bytes 4 (MK + KN + 2 MN). ----
-    if args.only in ("", "configs"):
-        shapes = {}
+            def cgemm():
+                st = fn(COL, NOTRANS, NOTRANS, n, n, n, 1.0 + 0.5j, A, 0, n, B, 0, n, 0.5 - 0.25j, C, 0, n)
+                if st != 0:
+                    raise RuntimeError("clblas%s returned %d" % (name, st))
 
-        def sgemm_case(M, N, K, tA, tB, alpha, beta, pad, offs, seed):
-            ra, ca = (K, M) if tA else (M, K)   # rows x columns as stored (column-major)
-            rb, cb = (N, K) if tB else (K, N)
-            lda, ldb, ldc = ra + pad, rb + pad, M + pad
-            A = gen_uniform(torch, offs[0] + lda * ca, seed, torch.float32)
-            B = gen_uniform(torch, offs[1] + ldb * cb, seed + 1, torch.float32)
-            C = gen_uniform(torch, offs[2] + ldc * N, seed + 2, torch.float32)
+            csteps = max(3, steps // 2)
+            wall, ev_ms = timed_calls(torch, cgemm, csteps, 2)
+            c_tflops = 8.0 * n * n * n / (ev_ms * 1e-3) / 1e12
+            extra[name] = {"workload": "%s column-major NN %d^3, alpha=1+0.5i, beta=0.5-0.25i, uniform[-1,1)" % (name.upper(), n),
+                           "tflops": round(c_tflops, 3), "launch_ms": round(ev_ms, 4),
+                           "pct_of_matrix_peak": round(100 * c_tflops / peak, 2)}
+            del A, B, C
 
-            bound = clblas_amd.bind("clblasSgemm", COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc)
+        # ---- SYRK / TRMM / SYMM / SYR2K and the complex-only routines at the same size (useful flops only: the reference client's counts) ----
+        if args.only in ("", "level3"):
+            lv = {}
+            for pre, dt, peak in (("S", torch.float32, PEAK_FP32_MATRIX), ("D", torch.float64, PEAK_FP64_MATRIX)):
+                A = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+                B0 = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+                B = B0.clone()
+                C = torch.rand(n * n, device="cuda", dtype=dt, generator=gen) * 2 - 1
+                cases = (
+                    ("syrk", float(n) * (n + 1) * n, None,
+                     lambda: clblas_amd.syrk(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, 1.0, C, 0, n)),
+                    ("trmm", float(n) * (n + 1) * n, lambda: B.copy_(B0),
+                     lambda: clblas_amd.trmm(pre, COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, A, 0, n, B, 0, n)),
+                    ("symm", 2.0 * n * n * n, None,
+                     lambda: clblas_amd.symm(pre, COL, LEFT, LOWER, n, n, 1.0, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+                    ("syr2k", 2.0 * n * n * n + n, None,
+                     lambda: clblas_amd.syr2k(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+                )
+                for name, fl, before, fn in cases:
+                    def call(fn=fn, name=name):
+                        st = fn()
+                        if st != 0:
+                            raise RuntimeError("clblas%s%s returned %d" % (pre, name, st))
+                    wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 2, before_each=before)
+                    tf = fl / (ev_ms * 1e-3) / 1e12
+                    lv[pre.lower() + name] = {"tflops": round(tf, 2), "ms_per_call": round(ev_ms, 4),
+                                              "pct_of_matrix_peak": round(100 * tf / peak, 1)}
+                del A, B, B0, C
+            # complex types: the Hermitian routines and the triangular solve (flop counts of the reference client)
+            for pre, dt, peak in (("C", torch.complex64, PEAK_FP32_MATRIX), ("Z", torch.complex128, PEAK_FP64_MATRIX)):
+                rdt = torch.float32 if dt == torch.complex64 else torch.float64
+                A, B0, C = (torch.view_as_complex(torch.rand(n * n, 2, device="cuda", dtype=rdt, generator=gen) * 2 - 1)
+                            for _ in range(3))
+                B = B0.clone()
+                T = A / n  # well-conditioned triangle: small off-diagonal entries, diagonal in [1, 2)
+                T.view(n, n).diagonal().copy_(torch.rand(n, device="cuda", dtype=rdt, generator=gen) + 1)
+                trsm = clblas_amd.ctrsm if pre == "C" else clblas_amd.ztrsm
+                cases = (
+                    ("herk", 4.0 * n * n * (n + 1), None,
+                     lambda: clblas_amd.herk(pre, COL, LOWER, NOTRANS, n, n, 1.0, A, 0, n, 1.0, C, 0, n)),
+                    ("her2k", 8.0 * n * n * n + 2 * n, None,
+                     lambda: clblas_amd.her2k(pre, COL, LOWER, NOTRANS, n, n, 1.0 + 0.5j, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+                    ("hemm", 8.0 * n * n * n, None,
+                     lambda: clblas_amd.hemm(pre, COL, LEFT, LOWER, n, n, 1.0 + 0.5j, A, 0, n, B0, 0, n, 1.0, C, 0, n)),
+                    ("trsm", 4.0 * n * (n + 1) * n, lambda: B.copy_(B0),
+                     lambda: trsm(COL, LEFT, LOWER, NOTRANS, NONUNIT, n, n, 1.0, T, 0, n, B, 0, n)),
+                )
+                for name, fl, before, fn in cases:
+                    def call(fn=fn, name=name):
+                        st = fn()
+                        if st != 0:
+                            raise RuntimeError("clblas%s%s returned %d" % (pre, name, st))
+                    wall, ev_ms = timed_calls(torch, call, max(3, steps // 4), 2, before_each=before)
+                    tf = fl / (ev_ms * 1e-3) / 1e12
+                    lv[pre.lower() + name] = {"tflops": round(tf, 2), "ms_per_call": round(ev_ms, 4),
+                                              "pct_of_matrix_peak": round(100 * tf / peak, 1)}
+                if not bool(torch.isfinite(torch.view_as_real(B)).all().item()):
+                    raise RuntimeError("clblas%strsm produced non-finite values" % pre)
+                del A, B, B0, C, T
+            lv["workload"] = "column-major, lower, left, no transpose, N=M=K=%d, alpha=beta=1 (complex: alpha=1+0.5i)" % n
+            extra["level3"] = lv
 
-            def call():
-                if bound() != 0:
-                    raise RuntimeError("clblasSgemm failed")
-            return timed_batch(torch, call, 20 if 2.0 * M * N * K > 1e10 else 100, 5)
+        # ---- BASELINE configs 1 and 3: SGEMM 1024^3 and the edge-shape sweep (ld = rows + 3, offsets 5/7/11,
+        #      alpha = 0.7, beta = -1.3, all four transposes).  Each against its own bound: MFMA time and HBM time
+        #      of the algorithmic bytes 4 (MK + KN + 2 MN). ----
+        if args.only in ("", "configs"):
+            shapes = {}
 
-        ms = sgemm_case(1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0), SEEDS["sgemm_config1"])
-        shapes["config1 1024x1024x1024 NN"] = {"ms": round(ms, 4), "tflops": round(2.0 * 1024 ** 3 / ms / 1e9, 2)}
-        for (M, N, K) in ((4097, 4095, 1031), (65536, 64, 4096), (64, 65536, 4096), (127, 129, 8192)):
-            flops = 2.0 * M * N * K
-            nbytes = 4.0 * (M * K + K * N + 2.0 * M * N)
-            row = {"mfma_bound_ms": round(flops / (PEAK_FP32_MATRIX * 1e12) * 1e3, 4),
-                   "hbm_bound_ms": round(nbytes / 8e12 * 1e3, 4)}
-            for tA, tB, tag in ((NOTRANS, NOTRANS, "NN"), (NOTRANS, TRANS, "NT"), (TRANS, NOTRANS, "TN"),
-                                (TRANS, TRANS, "TT")):
-                ms = sgemm_case(M, N, K, tA, tB, 0.7, -1.3, 3, (5, 7, 11), SEEDS["sgemm_config3"])
-                row[tag] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2),
-                            "GBps": round(nbytes / ms / 1e6, 1)}
-            shapes["config3 %dx%dx%d" % (M, N, K)] = row
-        # What the memory system gives a plain streaming kernel on this box (1 GiB read + 1 GiB written):
-        # the yardstick for the HBM-side figures of the skinny shapes above.
-        src = torch.empty(1 << 28, device="cuda", dtype=torch.float32)
-        dst = torch.empty_like(src)
-        copy_ms = timed_batch(torch, lambda: dst.copy_(src), 5, 2)
-        shapes["plain_device_copy_GBps"] = round(2 * 2 ** 30 / copy_ms / 1e6, 1)
-        del src, dst
-        extra["sgemm_configs_1_and_3"] = shapes
+            def sgemm_case(M, N, K, tA, tB, alpha, beta, pad, offs, seed):
+                ra, ca = (K, M) if tA else (M, K)   # rows x columns as stored (column-major)
+                rb, cb = (N, K) if tB else (K, N)
+                lda, ldb, ldc = ra + pad, rb + pad, M + pad
+                A = gen_uniform(torch, offs[0] + lda * ca, seed, torch.float32)
+                B = gen_uniform(torch, offs[1] + ldb * cb, seed + 1, torch.float32)
+                C = gen_uniform(torch, offs[2] + ldc * N, seed + 2, torch.float32)
 
-    # ---- Small C, deep K: fewer tiles than CUs, so the tile choice cuts K into ranges (column-major NN,
-    #      alpha = beta = 1); the vendor BLAS behind torch.mm on the same product beside it. ----
-    if args.only in ("", "deepk"):
-        dk = {}
-        for name, dt, fn, peak in (("sgemm", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX),
-                                   ("dgemm", torch.float64, clblas_amd.dgemm, PEAK_FP64_MATRIX)):
-            for (M, N, K) in ((1024, 1024, 16384), (768, 768, 16384), (3000, 200, 6000)):
-                A = torch.rand(K, M, device="cuda", dtype=dt, generator=gen) * 2 - 1   # column-major M x K
-                B = torch.rand(N, K, device="cuda", dtype=dt, generator=gen) * 2 - 1   # column-major K x N
-                C = torch.zeros(N, M, device="cuda", dtype=dt)
+                bound = clblas_amd.bind("clblasSgemm", COL, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc)
+
+                def call():
+                    if bound() != 0:
+                        raise RuntimeError("clblasSgemm failed")
+                return timed_batch(torch, call, 20 if 2.0 * M * N * K > 1e10 else 100, 5)
+
+            ms = sgemm_case(1024, 1024, 1024, NOTRANS, NOTRANS, 1.0, 0.0, 0, (0, 0, 0), SEEDS["sgemm_config1"])
+            shapes["config1 1024x1024x1024 NN"] = {"ms": round(ms, 4), "tflops": round(2.0 * 1024 ** 3 / ms / 1e9, 2)}
+            for (M, N, K) in ((4097, 4095, 1031), (65536, 64, 4096), (64, 65536, 4096), (127, 129, 8192)):
+                flops = 2.0 * M * N * K
+                nbytes = 4.0 * (M * K + K * N + 2.0 * M * N)
+                row = {"mfma_bound_ms": round(flops / (PEAK_FP32_MATRIX * 1e12) * 1e3, 4),
+                       "hbm_bound_ms": round(nbytes / 8e12 * 1e3, 4)}
+                for tA, tB, tag in ((NOTRANS, NOTRANS, "NN"), (NOTRANS, TRANS, "NT"), (TRANS, NOTRANS, "TN"),
+                                    (TRANS, TRANS, "TT")):
+                    ms = sgemm_case(M, N, K, tA, tB, 0.7, -1.3, 3, (5, 7, 11), SEEDS["sgemm_config3"])
+                    row[tag] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2),
+                                "GBps": round(nbytes / ms / 1e6, 1)}
+                shapes["config3 %dx%dx%d" % (M, N, K)] = row
+            # What the memory system gives a plain streaming kernel on this box (1 GiB read + 1 GiB written):
+            # the yardstick for the HBM-side figures of the skinny shapes above.
+            src = torch.empty(1 << 28, device="cuda", dtype=torch.float32)
+            dst = torch.empty_like(src)
+            copy_ms = timed_batch(torch, lambda: dst.copy_(src), 5, 2)
+            shapes["plain_device_copy_GBps"] = round(2 * 2 ** 30 / copy_ms / 1e6, 1)
+            del src, dst
+            extra["sgemm_configs_1_and_3"] = shapes
+
+        # ---- Small C, deep K: fewer tiles than CUs, so the tile choice cuts K into ranges (column-major NN,
+        #      alpha = beta = 1); the vendor BLAS behind torch.mm on the same product beside it. ----
+        if args.only in ("", "deepk"):
+            dk = {}
+            for name, dt, fn, peak in (("sgemm", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX),
+                                       ("dgemm", torch.float64, clblas_amd.dgemm, PEAK_FP64_MATRIX)):
+                for (M, N, K) in ((1024, 1024, 16384), (768, 768, 16384), (3000, 200, 6000)):
+                    A = torch.rand(K, M, device="cuda", dtype=dt, generator=gen) * 2 - 1   # column-major M x K
+                    B = torch.rand(N, K, device="cuda", dtype=dt, generator=gen) * 2 - 1   # column-major K x N
+                    C = torch.zeros(N, M, device="cuda", dtype=dt)
+
+                    def call():
+                        st = fn(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, C, 0, M)
+                        if st != 0:
+                            raise RuntimeError("clblas %s returned %d" % (name, st))
+                    ms = timed_batch(torch, call, 20, 3)
+                    vendor_tf, _ = vendor_rate(torch, lambda: torch.mm(B, A, out=C), 20, 3, 2.0 * M * N * K)   # C^T = B^T A^T, row-major
+                    tf = 2.0 * M * N * K / ms / 1e9
+                    dk["%s %dx%dx%d" % (name, M, N, K)] = {
+                        "ms": round(ms, 4), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
+                        "torch_mm_tflops": vendor_tf}
+                    del A, B, C
+            extra["small_c_deep_k"] = dk
+
+        # ---- Beyond 8192: the part has 288 GB, and matrices of 16384 .. 32768 are ordinary there (1 .. 8.6 GB each).
+        #      Column-major NN / left-lower-notrans-nonunit, alpha = beta = 1, tight leading dimensions. ----
+        if args.only in ("", "big"):
+            big = {}
+            for name, dt, fn, peak, dim, reps in (("sgemm 16384", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, 16384, 3),
+                                                ("dgemm 16384", torch.float64, clblas_amd.dgemm, PEAK_FP64_MATRIX, 16384, 2),
+                                                ("sgemm 32768", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, 32768, 1),
+                                                ("sgemm 20000x20000x8192", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, (20000, 20000, 8192), 3)):
+                M, N, K = dim if isinstance(dim, tuple) else (dim, dim, dim)
+                A = torch.rand(M * K, device="cuda", dtype=dt, generator=gen) * 2 - 1
+                B = torch.rand(K * N, device="cuda", dtype=dt, generator=gen) * 2 - 1
+                C = torch.zeros(M * N, device="cuda", dtype=dt)
 
                 def call():
                     st = fn(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, C, 0, M)
                     if st != 0:
                         raise RuntimeError("clblas %s returned %d" % (name, st))
-                ms = timed_batch(torch, call, 20, 3)
-                vendor_tf, _ = vendor_rate(torch, lambda: torch.mm(B, A, out=C), 20, 3, 2.0 * M * N * K)   # C^T = B^T A^T, row-major
+                ms = timed_batch(torch, call, reps, 1, batches=2)
                 tf = 2.0 * M * N * K / ms / 1e9
-                dk["%s %dx%dx%d" % (name, M, N, K)] = {
-                    "ms": round(ms, 4), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
-                    "torch_mm_tflops": vendor_tf}
+                big[name] = {"ms": round(ms, 3), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
+                             "kernel": clblas_amd.last_dispatch()[0]}
                 del A, B, C
-        extra["small_c_deep_k"] = dk
-
-    # ---- Beyond 8192: the part has 288 GB, and matrices of 16384 .. 32768 are ordinary there (1 .. 8.6 GB each).
-    #      Column-major NN / left-lower-notrans-nonunit, alpha = beta = 1, tight leading dimensions. ----
-    if args.only in ("", "big"):
-        big = {}
-        for name, dt, fn, peak, dim, reps in (("sgemm 16384", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, 16384, 3),
-                                            ("dgemm 16384", torch.float64, clblas_amd.dgemm, PEAK_FP64_MATRIX, 16384, 2),
-                                            ("sgemm 32768", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, 32768, 1),
-                                            ("sgemm 20000x20000x8192", torch.float32, clblas_amd.sgemm, PEAK_FP32_MATRIX, (20000, 20000, 8192), 3)):
-            M, N, K = dim if isinstance(dim, tuple) else (dim, dim, dim)
-            A = torch.rand(M * K, device="cuda", dtype=dt, generator=gen) * 2 - 1
-            B = torch.rand(K * N, device="cuda", dtype=dt, generator=gen) * 2 - 1
-            C = torch.zeros(M * N, device="cuda", dtype=dt)
-
-            def call():
-                st = fn(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, C, 0, M)
-                if st != 0:
-                    raise RuntimeError("clblas %s returned %d" % (name, st))
-            ms = timed_batch(torch, call, reps, 1, batches=2)
-            tf = 2.0 * M * N * K / ms / 1e9
-            big[name] = {"ms": round(ms, 3), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
-                         "kernel": clblas_amd.last_dispatch()[0]}
-            del A, B, C
-        for name, dt, fn, peak, dim in (("dtrsm 16384", torch.float64, clblas_amd.dtrsm, PEAK_FP64_MATRIX, 16384),
-                                      ("strsm 16384", torch.float32, clblas_amd.strsm, PEAK_FP32_MATRIX, 16384),
-                                      ("dtrsm 12000", torch.float64, clblas_amd.dtrsm, PEAK_FP64_MATRIX, 12000)):
-            A = (torch.rand(dim * dim, device="cuda", dtype=dt, generator=gen) * 2 - 1) / dim
-            A.view(dim, dim).diagonal().copy_(torch.rand(dim, device="cuda", dtype=dt, generator=gen) + 1)
-            B = torch.randn(dim * dim, device="cuda", dtype=dt, generator=gen)
-
-            def call():
-                st = fn(COL, LEFT, LOWER, NOTRANS, NONUNIT, dim, dim, 1.0, A, 0, dim, B, 0, dim)
-                if st != 0:
-                    raise RuntimeError("clblas %s returned %d" % (name, st))
-            n0 = clblas_amd.last_dispatch()[1]
-            call()
-            launches = clblas_amd.last_dispatch()[1] - n0
-            ms = timed_batch(torch, call, 2, 0, batches=2)
-            tf = dim * (dim + 1.0) * dim / ms / 1e9
-            big[name] = {"ms": round(ms, 3), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
-                         "kernels_per_call": launches, "finite": bool(torch.isfinite(B).all())}
-            del A, B
-        extra["beyond_8192"] = big
-        torch.cuda.empty_cache()   # tens of GB of freed matrices: back to the device, not kept in torch's cache
-
-    # ---- TRSM below 8192 (left, lower, no transpose, non-unit; square B, alpha = 1): a chain of short
-    #      dependent launches (packing pass, leaves of 512 equations, GEMM updates).  Each solve overwrites B
-    #      with a solution of similar size (diagonal 1..2, off-diagonal < 1/n), so calls can be repeated in
-    #      place.  The vendor's torch.linalg.solve_triangular on the same box beside it. ----
-    if args.only in ("", "trsm"):
-        ts = {}
-        for name, dt, fn in (("dtrsm", torch.float64, clblas_amd.dtrsm), ("strsm", torch.float32, clblas_amd.strsm)):
-            for m in (512, 1024, 2048, 4096):
-                A = (torch.rand(m, m, device="cuda", dtype=dt, generator=gen) - 0.5) / m     # column-major
-                A.diagonal().copy_(torch.rand(m, device="cuda", dtype=dt, generator=gen) + 1)
-                B = torch.rand(m, m, device="cuda", dtype=dt, generator=gen)
-
-                # (arguments converted once: at 512 the Python wrapper's share of a call would be a third of it)
-                bound = clblas_amd.bind("clblas" + name.capitalize(), COL, LEFT, LOWER, NOTRANS, NONUNIT, m, m, 1.0, A, 0, m, B, 0, m)
+            for name, dt, fn, peak, dim in (("dtrsm 16384", torch.float64, clblas_amd.dtrsm, PEAK_FP64_MATRIX, 16384),
+                                          ("strsm 16384", torch.float32, clblas_amd.strsm, PEAK_FP32_MATRIX, 16384),
+                                          ("dtrsm 12000", torch.float64, clblas_amd.dtrsm, PEAK_FP64_MATRIX, 12000)):
+                A = (torch.rand(dim * dim, device="cuda", dtype=dt, generator=gen) * 2 - 1) / dim
+                A.view(dim, dim).diagonal().copy_(torch.rand(dim, device="cuda", dtype=dt, generator=gen) + 1)
+                B = torch.randn(dim * dim, device="cuda", dtype=dt, generator=gen)
 
                 def call():
-                    if bound() != 0:
-                        raise RuntimeError("clblas %s failed" % name)
-                ms = timed_batch(torch, call, 50, 5)
-                launches = clblas_amd.last_dispatch()[1]
+                    st = fn(COL, LEFT, LOWER, NOTRANS, NONUNIT, dim, dim, 1.0, A, 0, dim, B, 0, dim)
+                    if st != 0:
+                        raise RuntimeError("clblas %s returned %d" % (name, st))
+                n0 = clblas_amd.last_dispatch()[1]
                 call()
-                launches = clblas_amd.last_dispatch()[1] - launches
-                Lt = torch.tril(A.T).contiguous()      # the same triangle as a row-major torch matrix
-                flops = float(m) * (m + 1) * m
-                vendor_tf, _ = vendor_rate(torch, lambda: torch.linalg.solve_triangular(Lt, B, upper=False), 5, 2, flops)
-                ts["%s %d" % (name, m)] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2), "kernels_per_call": launches,
-                                           "torch_solve_triangular_tflops": vendor_tf}
-                del A, B, Lt
-        extra["trsm_sizes"] = ts
+                launches = clblas_amd.last_dispatch()[1] - n0
+                ms = timed_batch(torch, call, 2, 0, batches=2)
+                tf = dim * (dim + 1.0) * dim / ms / 1e9
+                big[name] = {"ms": round(ms, 3), "tflops": round(tf, 2), "pct_of_matrix_peak": round(100 * tf / peak, 1),
+                             "kernels_per_call": launches, "finite": bool(torch.isfinite(B).all())}
+                del A, B
+            extra["beyond_8192"] = big
+            torch.cuda.empty_cache()   # tens of GB of freed matrices: back to the device, not kept in torch's cache
 
-    # ---- Host time per call: 10 000 back-to-back calls, CPU clock around the enqueue loop only (the device
-    #      is drained before and after, outside the clock).  Calls go straight to the C symbols with
-    #      prebuilt ctypes arguments; `ctypes_floor_us` is the same loop on a call that fails validation
-    #      at once (M = 0), i.e. the cost of getting from Python into the library and back.  When the
-    #      device is slower than the host the loop blocks on the full queue, so `us_per_call` is an upper
-    #      bound on the host cost and never less than the device time per call. ----
-    if args.only in ("", "host"):
-        import ctypes
-        lib = clblas_amd.load_library()
-        sz, vp, dbl = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_double
-        m = 512
-        A = gen_triangular(torch, m, 51, torch.float64)
-        A = torch.nan_to_num(A)
-        B = gen_uniform(torch, m * m, 52, torch.float64)
-        C = torch.zeros(m * m, device="cuda", dtype=torch.float64)
-        stream = vp(torch.cuda.current_stream().cuda_stream)
-        host = {}
+        # ---- TRSM below 8192 (left, lower, no transpose, non-unit; square B, alpha = 1): a chain of short
+        #      dependent launches (packing pass, leaves of 512 equations, GEMM updates).  Each solve overwrites B
+        #      with a solution of similar size (diagonal 1..2, off-diagonal < 1/n), so calls can be repeated in
+        #      place.  The vendor's torch.linalg.solve_triangular on the same box beside it. ----
+        if args.only in ("", "trsm"):
+            ts = {}
+            for name, dt, fn in (("dtrsm", torch.float64, clblas_amd.dtrsm), ("strsm", torch.float32, clblas_amd.strsm)):
+                for m in (512, 1024, 2048, 4096):
+                    A = (torch.rand(m, m, device="cuda", dtype=dt, generator=gen) - 0.5) / m     # column-major
+                    A.diagonal().copy_(torch.rand(m, device="cuda", dtype=dt, generator=gen) + 1)
+                    B = torch.rand(m, m, device="cuda", dtype=dt, generator=gen)
 
-        def loop(f, argv, calls):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(calls):
-                f(*argv)
-            dt = time.perf_counter() - t0
-            torch.cuda.synchronize()
-            return dt / calls * 1e6
+                    # (arguments converted once: at 512 the Python wrapper's share of a call would be a third of it)
+                    bound = clblas_amd.bind("clblas" + name.capitalize(), COL, LEFT, LOWER, NOTRANS, NONUNIT, m, m, 1.0, A, 0, m, B, 0, m)
 
-        def gemm_args(mm):
-            return (COL, NOTRANS, NOTRANS, sz(mm), sz(m), sz(m), dbl(1.0), vp(A.data_ptr()), sz(0), sz(m), vp(B.data_ptr()), sz(0),
-                    sz(m), dbl(0.0), vp(C.data_ptr()), sz(0), sz(m), stream)
+                    def call():
+                        if bound() != 0:
+                            raise RuntimeError("clblas %s failed" % name)
+                    ms = timed_batch(torch, call, 50, 5)
+                    launches = clblas_amd.last_dispatch()[1]
+                    call()
+                    launches = clblas_amd.last_dispatch()[1] - launches
+                    Lt = torch.tril(A.T).contiguous()      # the same triangle as a row-major torch matrix
+                    flops = float(m) * (m + 1) * m
+                    vendor_tf, _ = vendor_rate(torch, lambda: torch.linalg.solve_triangular(Lt, B, upper=False), 5, 2, flops)
+                    ts["%s %d" % (name, m)] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 2), "kernels_per_call": launches,
+                                               "torch_solve_triangular_tflops": vendor_tf}
+                    del A, B, Lt
+            extra["trsm_sizes"] = ts
 
-        def trsm_args(mm):
-            return (COL, LEFT, LOWER, NOTRANS, NONUNIT, sz(mm), sz(m), dbl(1.0), vp(A.data_ptr()), sz(0), sz(m), vp(B.data_ptr()),
-                    sz(0), sz(m), stream)
-        for name, f, mk in (("dgemm_512", lib.clblasDgemm, gemm_args), ("dtrsm_512", lib.clblasDtrsm, trsm_args)):
-            if f(*mk(m)) != 0:
-                raise RuntimeError("%s failed" % name)
-            n0 = clblas_amd.last_dispatch()[1]
-            us = min(loop(f, mk(m), 10000) for _ in range(2))
-            kernels = (clblas_amd.last_dispatch()[1] - n0) / 20000.0
-            floor = loop(f, mk(0), 10000)
-            host[name] = {"us_per_call": round(us, 2), "ctypes_floor_us": round(floor, 2), "kernels_per_call": kernels}
-        del A, B, C
-        extra["host_enqueue_us"] = host
+        # ---- Host time per call: 10 000 back-to-back calls, CPU clock around the enqueue loop only (the device
+        #      is drained before and after, outside the clock).  Calls go straight to the C symbols with
+        #      prebuilt ctypes arguments; `ctypes_floor_us` is the same loop on a call that fails validation
+        #      at once (M = 0), i.e. the cost of getting from Python into the library and back.  When the
+        #      device is slower than the host the loop blocks on the full queue, so `us_per_call` is an upper
+        #      bound on the host cost and never less than the device time per call. ----
+        if args.only in ("", "host"):
+            import ctypes
+            lib = clblas_amd.load_library()
+            sz, vp, dbl = ctypes.c_size_t, ctypes.c_void_p, ctypes.c_double
+            m = 512
+            A = gen_triangular(torch, m, 51, torch.float64)
+            A = torch.nan_to_num(A)
+            B = gen_uniform(torch, m * m, 52, torch.float64)
+            C = torch.zeros(m * m, device="cuda", dtype=torch.float64)
+            stream = vp(torch.cuda.current_stream().cuda_stream)
+            host = {}
 
-    # ---- The tile choice against the best forced tile, on shapes that are not whole rounds of any tile:
-    #      tracks how well the cost model in the launcher (choose_tile) fits the kernels as they are now. ----
-    if args.only in ("", "tilemodel"):
-        # (--only tilemodel also keeps every forced tile's time: the input of clblas_amd/fit_tile_model.py)
-        extra["tile_model"] = tile_model_block(torch, clblas_amd, gen, keep_forced=args.only == "tilemodel")
+            def loop(f, argv, calls):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(calls):
+                    f(*argv)
+                dt = time.perf_counter() - t0
+                torch.cuda.synchronize()
+                return dt / calls * 1e6
 
-    # ---- Yardstick: the vendor BLAS that torch calls (rocBLAS / hipBLASLt) on the same box, same sizes.
-    #      Not the reference and not a target of the parity tests: it shows what the part gives a
-    #      tuned library.  FP32 without TF32-style shortcuts. ----
-    if args.only in ("", "vendor"):
-        torch.backends.cuda.matmul.allow_tf32 = False
-        vy = {}
-        for name, dt, fl in (("sgemm", torch.float32, 2.0), ("dgemm", torch.float64, 2.0),
-                             ("cgemm", torch.complex64, 8.0), ("zgemm", torch.complex128, 8.0)):
-            real = torch.float32 if dt in (torch.float32, torch.complex64) else torch.float64
-            shape = (n, n, 2) if dt.is_complex else (n, n)
-            mk = lambda: torch.rand(shape, device="cuda", dtype=real, generator=gen) * 2 - 1
-            A, B = mk(), mk()
-            if dt.is_complex:
-                A, B = torch.view_as_complex(A), torch.view_as_complex(B)
-            C = torch.empty(n, n, device="cuda", dtype=dt)
-            tf, ms = vendor_rate(torch, lambda: torch.mm(A, B, out=C), 5, 2, fl * n ** 3)
-            vy["torch_mm_" + name] = {"tflops": tf, "ms": ms}
+            def gemm_args(mm):
+                return (COL, NOTRANS, NOTRANS, sz(mm), sz(m), sz(m), dbl(1.0), vp(A.data_ptr()), sz(0), sz(m), vp(B.data_ptr()), sz(0),
+                        sz(m), dbl(0.0), vp(C.data_ptr()), sz(0), sz(m), stream)
+
+            def trsm_args(mm):
+                return (COL, LEFT, LOWER, NOTRANS, NONUNIT, sz(mm), sz(m), dbl(1.0), vp(A.data_ptr()), sz(0), sz(m), vp(B.data_ptr()),
+                        sz(0), sz(m), stream)
+            for name, f, mk in (("dgemm_512", lib.clblasDgemm, gemm_args), ("dtrsm_512", lib.clblasDtrsm, trsm_args)):
+                if f(*mk(m)) != 0:
+                    raise RuntimeError("%s failed" % name)
+                n0 = clblas_amd.last_dispatch()[1]
+                us = min(loop(f, mk(m), 10000) for _ in range(2))
+                kernels = (clblas_amd.last_dispatch()[1] - n0) / 20000.0
+                floor = loop(f, mk(0), 10000)
+                host[name] = {"us_per_call": round(us, 2), "ctypes_floor_us": round(floor, 2), "kernels_per_call": kernels}
             del A, B, C
-        T = torch.tril(torch.rand(n, n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1) / n
-        T.diagonal().copy_(torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) + 1)
-        Bt = torch.randn(n, n, device="cuda", dtype=torch.float64, generator=gen)
-        tf, ms = vendor_rate(torch, lambda: torch.linalg.solve_triangular(T, Bt, upper=False), 3, 1, float(n) * (n + 1) * n)
-        vy["torch_solve_triangular_f64"] = {"tflops": tf, "ms": ms}
-        vy["workload"] = "square, N=%d, row-major torch tensors, no transposes, beta=0" % n
-        del T, Bt
-        extra["vendor_yardstick"] = vy
+            extra["host_enqueue_us"] = host
+
+        # ---- The tile choice against the best forced tile, on shapes that are not whole rounds of any tile:
+        #      tracks how well the cost model in the launcher (choose_tile) fits the kernels as they are now. ----
+        if args.only in ("", "tilemodel"):
+            # (--only tilemodel also keeps every forced tile's time: the input of clblas_amd/fit_tile_model.py)
+            extra["tile_model"] = tile_model_block(torch, clblas_amd, gen, keep_forced=args.only == "tilemodel")
+
+        # ---- Yardstick: the vendor BLAS that torch calls (rocBLAS / hipBLASLt) on the same box, same sizes.
+        #      Not the reference and not a target of the parity tests: it shows what the part gives a
+        #      tuned library.  FP32 without TF32-style shortcuts. ----
+        if args.only in ("", "vendor"):
+            torch.backends.cuda.matmul.allow_tf32 = False
+            vy = {}
+            for name, dt, fl in (("sgemm", torch.float32, 2.0), ("dgemm", torch.float64, 2.0),
+                                 ("cgemm", torch.complex64, 8.0), ("zgemm", torch.complex128, 8.0)):
+                real = torch.float32 if dt in (torch.float32, torch.complex64) else torch.float64
+                shape = (n, n, 2) if dt.is_complex else (n, n)
+                mk = lambda: torch.rand(shape, device="cuda", dtype=real, generator=gen) * 2 - 1
+                A, B = mk(), mk()
+                if dt.is_complex:
+                    A, B = torch.view_as_complex(A), torch.view_as_complex(B)
+                C = torch.empty(n, n, device="cuda", dtype=dt)
+                tf, ms = vendor_rate(torch, lambda: torch.mm(A, B, out=C), 5, 2, fl * n ** 3)
+                vy["torch_mm_" + name] = {"tflops": tf, "ms": ms}
+                del A, B, C
+            T = torch.tril(torch.rand(n, n, device="cuda", dtype=torch.float64, generator=gen) * 2 - 1) / n
+            T.diagonal().copy_(torch.rand(n, device="cuda", dtype=torch.float64, generator=gen) + 1)
+            Bt = torch.randn(n, n, device="cuda", dtype=torch.float64, generator=gen)
+            tf, ms = vendor_rate(torch, lambda: torch.linalg.solve_triangular(T, Bt, upper=False), 3, 1, float(n) * (n + 1) * n)
+            vy["torch_solve_triangular_f64"] = {"tflops": tf, "ms": ms}
+            vy["workload"] = "square, N=%d, row-major torch tensors, no transposes, beta=0" % n
+            del T, Bt
+            extra["vendor_yardstick"] = vy
+
+    except Exception as e:   # noqa: BLE001 - whatever an extra raises must not cost the headline
+        extra["extras_error"] = "%s: %s" % (type(e).__name__, str(e).splitlines()[0][:300] if str(e) else "")
+        sys.stderr.write("bench.py: an extra block failed, the rest of the extras are skipped: %s\n" % extra["extras_error"])
+        try:
+            torch.cuda.synchronize()
+        except Exception:   # noqa: BLE001
+            pass
 
     # ---- CPU baseline: the oracle (port of the reference arithmetic) on the host cores, same seeds as the
     #      GPU legs; config 2 and config 1 in full, configs 4 and 5 on stated sub-problems (the same
