@@ -43,6 +43,7 @@ void read_knobs() {
     k.split_model = env_int("CLBLAS_AMD_GEMM_SPLIT_MODEL", 1);
     k.splits = env_int("CLBLAS_AMD_GEMM_SPLITS", 0);
     k.tail = env_int("CLBLAS_AMD_GEMM_TAIL", 1);
+    k.peel = env_int("CLBLAS_AMD_GEMM_PEEL", 1);
     k.group_m = env_int("CLBLAS_AMD_GEMM_GROUP_M", 0);
     k.xcd = env_int("CLBLAS_AMD_GEMM_XCD", 1);
     k.stagger = env_int("CLBLAS_AMD_GEMM_STAGGER", 1);
@@ -335,8 +336,12 @@ clblasStatus gemm_front(clblasOrder order, clblasTranspose transA, clblasTranspo
         return map_hip_error(cba::sgemm_colmajor_noalloc(tA, tB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb,
                                                          (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
     else
-        return map_hip_error(cba::launch_gemm<T>(tA, tB, cA, cB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb,
-                                                 (int64_t)ldb, beta, C + offC, (int64_t)ldc, stream));
+        // (a product may be made in two or three launches - see run_gemm_colmajor - so under capture every
+        // scratch buffer is secured before the first of them)
+        return map_hip_error(cba::with_workspaces_secured(stream, [&] {
+            return cba::launch_gemm<T>(tA, tB, cA, cB, (int)M, (int)N, (int)K, alpha, pa, (int64_t)lda, pb, (int64_t)ldb, beta,
+                                       C + offC, (int64_t)ldc, stream);
+        }));
 }
 
 template <typename T> struct IsComplex { static const bool value = false; };

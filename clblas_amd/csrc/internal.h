@@ -53,6 +53,7 @@ struct DebugKnobs {
     int gemm_tile = -1, split_model = 1, splits = 0, tail = 1, group_m = 0, xcd = 1, stagger = 1, log = 0;
     int check_mem = 0;
     int trsm_poll_limit = 0;  // CLBLAS_AMD_TRSM_POLL_LIMIT: polls after which a flag wait of the substitution leaf gives up (0: 2^22); tests
+    int peel = 1;          // CLBLAS_AMD_GEMM_PEEL: 0 never splits a strip of rows / columns off a product, 2 always where one exists (tests)
     int trsm_wide = -1;    // CLBLAS_AMD_TRSM_WIDE (real types, substitution leaf): 0 / 1 forces 16 / 32 right-hand sides per workgroup
     int trsm_leaf = 0;     // CLBLAS_AMD_TRSM_LEAF (real types): 0 substitution over 16-row sub-blocks, 1 inverted 64 x 64 triangles
     int wide_ld = 0;       // CLBLAS_AMD_GEMM_WIDE_LD=1: the wide-ld kernels whatever the leading dimensions (tests)

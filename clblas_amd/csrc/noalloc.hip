@@ -74,6 +74,18 @@ hipError_t sgemm_colmajor_noalloc(bool transA, bool transB, int M, int N, int K,
     hipError_t e = noalloc_scratch(&fixed.ptr);
     if (e != hipSuccess) return e;
     fixed.bytes = kScratchBytes;
+    // A product may take two or three launches (a strip of rows or columns as a product of its own): walk the
+    // sequence dry first, so that a part that needs more scratch than the array holds is found before the
+    // first kernel is enqueued.
+    if (!dry_run_slot()) {
+        DryRun dry;
+        const DispatchRecord kept = dispatch_record();
+        dry_run_slot() = &dry;
+        e = sgemm_colmajor(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, nullptr, &fixed);
+        dry_run_slot() = nullptr;
+        dispatch_record() = kept;
+        if (e != hipSuccess) return e;
+    }
     return sgemm_colmajor(transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, stream, nullptr, &fixed);
 }
 
