@@ -560,8 +560,8 @@ static hipError_t run_gemm_whole(const TileEntry<T> *tab, int ntab, bool tA, boo
 // A dimension that is a few rows or columns more than a whole number of tiles costs a whole extra row or
 // column of tiles that compute on padding (SGEMM 8193^3: 138 TFLOP/s against 148 at 8192^3; 10000 = 39 x 256 + 16).
 // Where the model prices it lower, the product is made in two launches instead: the part up to the last
-// multiple of 128, and the strip of at most 32 rows (or columns) as a product of its own - a skinny one, which
-// gets small tiles and a K split.  Both write disjoint parts of C with the same alpha and beta.  The parts
+// multiple of 128, and the strip of at most 64 rows (or columns: one row of the smallest tile) as a product of
+// its own - a skinny one, which gets small tiles and a K split.  Both write disjoint parts of C with the same alpha and beta.  The parts
 // are priced by the same model as the whole (same K, so the costs add); a launch costs about 3 us on top.
 // Plain products only (no triangular structure, no forced tile, no wide leading dimensions).
 template <typename T>
@@ -573,7 +573,7 @@ static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, 
     const bool plain = !(tri && tri->any()) && K > 0 && knobs().gemm_tile < 0 && knobs().wide_ld == 0;
     if (mode != 0 && plain && depth < 2) {
         const int64_t ld_limit = (int64_t)0x7fffffff / (256 * (int64_t)sizeof(T)) - 8;
-        const int kStrip = 32, kEdge = 128, kLeast = 1024;
+        const int kStrip = 64, kEdge = 128, kLeast = 1024;
         const int rm = M % kEdge, rn = N % kEdge;
         const bool can_m = rm > 0 && rm <= kStrip && M - rm >= kLeast, can_n = rn > 0 && rn <= kStrip && N - rn >= kLeast;
         if ((can_m || can_n) && lda <= ld_limit && ldb <= ld_limit) {

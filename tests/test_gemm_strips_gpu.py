@@ -1,5 +1,5 @@
 """clblas{S,D,C,Z}gemm where a product is made in two or three launches: a dimension that is a few rows or columns
-more than a whole number of tiles has its last rows / columns (at most 32) split off as a product of their own
+more than a whole number of tiles has its last rows / columns (at most 64) split off as a product of their own
 when the tile model prices that lower.  The debug switch CLBLAS_AMD_GEMM_PEEL=2 splits wherever a strip exists,
 =0 never does; every result is compared with the CPU oracle on integer data (exact whatever the order of
 summation), so the pieces must tile C exactly, with the right operands, offsets and leading dimensions, in both
@@ -19,8 +19,8 @@ pytestmark = pytest.mark.gpu
 
 TYPES = {"s": np.float32, "d": np.float64, "c": np.complex64, "z": np.complex128}
 FN = {"s": clblas_amd.sgemm, "d": clblas_amd.dgemm, "c": clblas_amd.cgemm, "z": clblas_amd.zgemm}
-# (M, N, K): a strip of rows, of columns, of both, and a strip of the full 32
-SHAPES = [(1030, 1100, 70), (1100, 1027, 130), (1025, 1056, 33), (1056, 1152, 64), (2049, 1025, 40)]
+# (M, N, K): a strip of rows, of columns, of both, and strips of 32 and of the full 64
+SHAPES = [(1030, 1100, 70), (1100, 1027, 130), (1025, 1056, 33), (1056, 1152, 64), (2049, 1025, 40), (1088, 1100, 50)]
 
 
 def _case(t, order, tA, tB, M, N, K, seed, pad, offs, alpha, beta):
