@@ -223,3 +223,60 @@ def test_a_routine_of_several_launches_is_refused_before_its_first_launch():
         assert torch.equal(tb, want_tb) and torch.equal(dc, want_dc)
     del graph
     assert clblas_amd.release_stream(stream.cuda_stream) == 0
+
+
+def test_a_gemm_made_of_several_launches_under_capture():
+    """A GEMM whose last rows are split off as a product of their own (forced here with
+    CLBLAS_AMD_GEMM_PEEL=2) is two launches, the second of which cuts K and needs a scratch buffer: captured
+    on a stream without that buffer it is refused before the first launch - C untouched after a replay - and
+    with the buffer in place it is captured and replays to the eager result bit for bit."""
+    import torch
+    import clblas_amd
+    import gpu_util
+    assert clblas_amd.setup() == 0
+    INVALID_OPERATION = -59
+    f32 = np.float32
+    M, N, K = 1030, 1100, 4096      # 1024 x 1100 x 4096 in whole tiles + a strip of 6 rows: few tiles, deep K
+    a = torch.from_numpy(oracle.uniform(M * K, 31, f32)).cuda()
+    b = torch.from_numpy(oracle.uniform(K * N, 32, f32)).cuda()
+    c = torch.from_numpy(oracle.uniform(M * N, 33, f32)).cuda()
+    keep = c.clone()
+
+    def gemm():
+        return clblas_amd.sgemm(COL, NOTRANS, NOTRANS, M, N, K, 0.5, a, 0, M, b, 0, K, -1.5, c, 0, M)
+
+    with gpu_util.debug_env(CLBLAS_AMD_GEMM_PEEL=2):
+        n0 = clblas_amd.last_dispatch()[1]
+        assert gemm() == 0
+        torch.cuda.synchronize()
+        assert clblas_amd.last_dispatch()[1] - n0 >= 3, "expected the main part, the strip and its reduction pass"
+        eager = c.clone()
+        c.copy_(keep)
+
+        stream = torch.cuda.Stream()        # a stream that has no scratch buffers yet
+        stats = clblas_amd.workspace_stats()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            st = gemm()
+        assert st == INVALID_OPERATION, st
+        assert clblas_amd.workspace_stats() == stats
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(c, keep), "the refused GEMM must not have touched C"
+        del graph
+
+        assert clblas_amd.reserve_workspace(8 << 20, 0, 0, stream=stream.cuda_stream) == 0
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            st = gemm()
+        assert st == 0, st
+        for rep in range(3):
+            c.copy_(keep)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(c, eager), "replay %d differs from the eager result" % rep
+        del graph
+        assert clblas_amd.release_stream(stream.cuda_stream) == 0
