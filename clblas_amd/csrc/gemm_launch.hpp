@@ -561,9 +561,11 @@ static hipError_t run_gemm_whole(const TileEntry<T> *tab, int ntab, bool tA, boo
 // column of tiles that compute on padding (SGEMM 8193^3: 138 TFLOP/s against 148 at 8192^3; 10000 = 39 x 256 + 16).
 // Where the model prices it lower, the product is made in two launches instead: the part up to the last
 // multiple of 128, and the strip of at most 64 rows (or columns: one row of the smallest tile) as a product of
-// its own - a skinny one, which gets small tiles and a K split.  Both write disjoint parts of C with the same alpha and beta.  The parts
-// are priced by the same model as the whole (same K, so the costs add); a launch costs about 3 us on top.
-// Plain products only (no triangular structure, no forced tile, no wide leading dimensions).
+// its own - a skinny one, which gets small tiles and a K split.  Both write disjoint parts of C with the same
+// alpha and beta.  The parts are priced by the same model as the whole (same K, so the costs add); a launch
+// costs about 3 us on top.  Plain products only (no triangular structure, no forced tile, no wide leading
+// dimensions).  (depth: 0 the caller's product, 1 a main part - it may lose a strip of the other dimension -,
+// 2 a strip: made whole.)
 template <typename T>
 static hipError_t run_gemm_colmajor(const TileEntry<T> *tab, int ntab, bool tA, bool tB, bool cA, bool cB, int M,
                                     int N, int K, T alpha, const T *A, int64_t lda, const T *B, int64_t ldb,
