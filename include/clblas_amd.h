@@ -371,7 +371,9 @@ void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes);
  * function that launches nothing: the chosen tile (index into the type's tile table), its number of K
  * ranges and tail slices, the cost the choice model puts on every tile in one K range (negative: tile not
  * offered) and the tiles' dimensions (bm, bn, bk per tile, 3 ints each; `costs` and `dims` hold max_tiles
- * entries).  Returns the number of tiles in the table, -1 for bad arguments.
+ * entries).  Returns the number of tiles in the table, -1 for bad arguments.  (The answer is for the product
+ * as given, in one piece: the launcher may in addition make a strip of up to 64 rows or columns beyond a
+ * multiple of 128 as a product of its own where this same model prices the two pieces lower.)
  * clblasAmdTileModelParam reads (set == 0) or sets one parameter of one tile's model - which: 0 the
  * efficiency credited to the tile, 1 the factor for a workgroup alone on its CU, 2 the fixed time per
  * workgroup as a depth, 3 the price of a sliced tail in rounds, 4 the credit of the deep-panel form, 5 the
