@@ -16,9 +16,11 @@ namespace cba {
 //      Tiles 1 to 3 are split-K capable for small C with deep K, where the 64x64 tile (split or not) loses to
 //      them: 1024 x 1024 x 65536 98 -> 141 TFLOP/s, 1280 x 1280 x 8192 108 -> 125, 768 x 768 x 16384 109 -> 128,
 //      3000 x 200 x 6000 72 -> 87.
-//      Tiles 2 and 3 are not offered to products with a triangular operand: the round model for those
-//      was fitted on the square tiles and picks the oblong ones where they lose (STRMM / SSYMM 3072:
-//      7-9 % slower with them).
+//      Products with a triangular operand (TRMM, SYMM) are offered tile 3 but not tile 2 (STRMM 4000: 120.6
+//      TFLOP/s with 64x128, 111.8 with 128x64, 113.7 with 64x64), and the credits for them were set from STRMM /
+//      SSYMM at 2000 .. 10000 with every tile forced: 64x64 .83 and 64x128 .885 beside .92 and .942 of the two
+//      large tiles, so that 64x64 is taken up to 3000, 64x128 at 4000 .. 6000, 128x128 from there (STRMM 5000
+//      116 -> 124, 6000 116 -> 123, 7000 117 -> 127; SSYMM 5000 118 -> 128, 7000 120 -> 131).
 //   The parameters of the choice model (efficiency, fixed time per workgroup as a depth k0, price of a sliced
 //   tail) were last refitted with clblas_amd/fit_tile_model.py on bench.py --only tilemodel: the 256x128 tile
 //   has a k0 (on large C with K of a few hundred the 128x128 tile is ahead: 8192 x 8192 x 128 +3.5 %,
@@ -46,8 +48,8 @@ static TileEntry<float> *f32_tiles(int *n) {
         make_tile_entry<float, 256, 128, 16, 128, 64, 2, false, true>(0.952, 0.85, 0.942, 40.0, 0.03, 0.942),
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.07),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.9, 0.0, 10.0),
-        with_split_gain(make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.9, 0.0, 10.0), 1.02),
-        make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64, true>(0.88, 0.85, -1.0, 0.0, 0.02),
+        with_split_gain(make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.9, 0.885, 10.0), 1.02),
+        make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64, true>(0.88, 0.85, 0.83, 0.0, 0.02),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
     return tab;
