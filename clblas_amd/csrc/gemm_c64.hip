@@ -10,13 +10,16 @@ namespace cba {
 //   On large C the 64x64 tiles are the faster ones at every depth (8192^3: 73.2 against 72.0 TFLOP/s, 8192 x 8192 x
 //   2048 72.8 / 71.4, x 512 71.6 / 69.4, x 64 53.3 / 48.8, 4096 x 4096 x 32 38.5 / 32.4), so they are credited with
 //   .945 against .93 and with the smaller fixed time (k0 = 35 and 44 from T(K) = T_inf K / (K + k0)); the 128x64
-//   tiles keep the cases where they fill the rounds better.  Products with a triangular operand or a triangular C keep
-//   .86 (ZSYRK 8192: 71.4 TFLOP/s with the 128x64 tiles, 69.9 with these; 6144: 70.5 / 70.9).
+//   tiles keep the cases where they fill the rounds better.  Products with a triangular operand or a triangular C are
+//   credited .86 with the 64x64 tiles and .84 (operand) / .86 (C) with the 128x64 ones, from runs with each tile
+//   forced: ZTRMM 3000 60.3 / 64.2 TFLOP/s (128x64 / 64x64), 5000 63.8 / 66.9, 6000 67.7 / 69.0, 8192 69.6 / 70.4;
+//   ZSYRK 3000 50.1 / 65.2, 5000 64.8 / 67.4, 6000 67.9 / 69.6 and only at 8192 70.3 / 69.3, where the equal
+//   credits leave the choice to the count of rounds.
 //   A sliced tail costs these tiles more than the others (3000 x 1500 x 1000, 1128 tiles with 104 in the tail
 //   round: 60.4 TFLOP/s against 64.4 with the 128x64 tiles), so it is priced at 0.35 rounds instead of 0.05.
 static const TileEntry<Cx<double>> *c64_tiles(int *n) {
     static const TileEntry<Cx<double>> tab[] = {
-        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, true, true>(0.93, 0.85, -1.0, 44.0),
+        make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, true, true>(0.93, 0.85, 0.84, 44.0, 0.05, 0.86),
         make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true, 0, true>(0.945, 0.85, 0.86, 35.0, 0.35, 0.86),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));
