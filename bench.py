@@ -263,6 +263,8 @@ def opencl_cpu_probe():
 
 
 TILE_MODEL_SHAPES = (
+    # small products: a few hundred tiles of 64x64 at most (one launch of smaller tiles against a K split)
+    (384, 384, 384), (512, 512, 512), (640, 640, 640), (512, 1024, 512), (800, 600, 400), (896, 896, 896), (512, 512, 2048),
     (768, 768, 768), (1000, 1000, 1000), (1280, 1280, 1280), (1500, 1500, 1500), (1792, 1792, 1792), (2000, 2000, 2000),
     (2304, 2304, 2304), (2560, 2560, 2560), (3000, 3000, 3000), (3328, 3328, 3328), (3584, 3584, 3584), (3700, 3700, 3700),
     (4097, 4095, 1031), (5000, 1000, 1000), (1800, 2200, 2600), (4200, 1700, 900), (6000, 6000, 640), (4480, 4480, 2000),
@@ -285,7 +287,8 @@ def tile_model_block(torch, clblas_amd, gen, keep_forced=False):
     column-major NN, alpha = beta = 1.  Per shape: [default TFLOP/s, default tile, best forced TFLOP/s, best
     tile]; `mispicks` lists the shapes where the default runs more than 3 % behind a different, forced tile."""
     out = {}
-    for name, dt, fn, ntiles in (("sgemm", torch.float32, clblas_amd.sgemm, 5), ("dgemm", torch.float64, clblas_amd.dgemm, 2)):
+    for name, dt, fn in (("sgemm", torch.float32, clblas_amd.sgemm), ("dgemm", torch.float64, clblas_amd.dgemm)):
+        ntiles = len(clblas_amd.tile_model_query(name[0], 1024, 1024, 1024)["tiles"])
         rows, mispicks, worst, forced = {}, [], 1.0, {}
         for (M, N, K) in TILE_MODEL_SHAPES:
             if name == "dgemm" and M * N * K > 6.5e10 and M not in (8192, 9000, 10000, 12000):
@@ -298,7 +301,8 @@ def tile_model_block(torch, clblas_amd, gen, keep_forced=False):
                 st = fn(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 1.0, C, 0, M)
                 if st != 0:
                     raise RuntimeError("clblas %s returned %d" % (name, st))
-            reps = int(min(40, max(2, 2e11 / (2.0 * M * N * K))))   # a few milliseconds per batch
+            # a few milliseconds per batch (the small products, of some 10 us, in batches of 200)
+            reps = int(min(200 if 2.0 * M * N * K < 2e9 else 40, max(2, 2e11 / (2.0 * M * N * K))))
             ms_default = timed_batch(torch, call, reps, 2, batches=3)
             import re
             default_tile = re.search(r"<\w,(\d+x\d+)x", clblas_amd.last_dispatch()[0]).group(1)

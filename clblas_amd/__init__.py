@@ -246,7 +246,7 @@ def workspace_stats():
     return a.value, b.value
 
 
-TILE_PARAMS = ("eff", "alone", "k0", "tail_extra", "deep_gain", "split_gain")
+TILE_PARAMS = ("eff", "alone", "k0", "tail_extra", "deep_gain", "split_gain", "streamed_gain")
 
 
 def tile_model_query(type_letter, M, N, K):

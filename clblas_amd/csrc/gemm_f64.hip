@@ -6,7 +6,15 @@ namespace cba {
 // Ordered from the largest tile to the smallest.
 //   0: 128x128x16, wave 64x64 (2 workgroups of 4 waves per CU), split-K capable for small C with deep K
 //      (1024 x 1024 x 16384: 50 -> 69 TFLOP/s, 1280 x 1280 x 8192 54 -> 66, 256 x 4096 x 8192 46 -> 66)
-//   1:  64x64x16,  wave 32x32, split-K capable.  Credited with .90 for plain and triangular-C
+//   1:  64x32x32,  wave 32x16, and
+//   2:  32x32x32,  wave 16x16: for products of up to a few hundred tiles of 64x64, which they cover with one
+//      workgroup or more per CU in a single launch, where the 64x64 tiles leave CUs idle or cut K and pay a second,
+//      dependent launch (DGEMM 512^3 14.7 -> 8.6 us, the vendor library 11.6; 448^3 13.4 -> 7.8, 704^3 21.1 -> 15.6,
+//      800 x 600 x 400 17.2 -> 11.0, 512 x 1024 x 512 - an update of DTRSM 1024 - 19.2 -> 12.1; from 900^3 on and
+//      for deep K the 64x64 tiles are ahead again).  Plain products only (no K ranges, no triangular forms).  A
+//      workgroup of 32x32 alone on its CU runs at 0.44 of the CU's peak, two at 0.61, three or more at 0.7; one of
+//      64x32 at 0.79 alone, 0.83-0.85 in company, with about 3 us before its first MFMA: eff / alone / k0 below.
+//   3:  64x64x16,  wave 32x32, split-K capable.  Credited with .90 for plain and triangular-C
 //      products (2304^3 64.7 -> 67.9 TFLOP/s, 3328^3 64.5 -> 68.6, 3000 x 1500 x 1000 56.6 -> 61.1 against
 //      .84) and with .84 where an operand is triangular (DTRMM / DSYMM 6144 lose 2-3 % with .90).
 //      With panels of depth 32 where a workgroup's K range is at least 1024 (1024^3 54.9 -> 58.5 TFLOP/s,
@@ -20,6 +28,8 @@ namespace cba {
 static TileEntry<double> *f64_tiles(int *n) {
     static TileEntry<double> tab[] = {
         make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 85.0),
+        with_streamed_gain(make_tile_entry<double, 64, 32, 32, 32, 16, 2, false, false>(0.75, 1.0, -1.0, 100.0), 0.95),
+        with_streamed_gain(make_tile_entry<double, 32, 32, 32, 16, 16, 2, false, false>(0.80, 0.6, -1.0, 200.0), 0.75),
         // (in launches that cut K it is credited 4 % less: DGEMM 100 x 5000 x 20000 ran 5.6 % behind the 128x128
         // tile in twelve ranges with it)
         with_split_gain(make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32, true>(0.90, 0.85, 0.84, 68.0, 0.35), 0.96),

@@ -22,6 +22,8 @@ template <typename T> struct TileEntry {
     // round of workgroups: see where the variant is chosen).
     int bk_deep;
     double deep_gain;  // factor on `eff` where the deep form runs (plain products, K range from 1024)
+    double streamed_gain;  // factor on `eff` where the operands are streamed from HBM (beyond the memory-side cache): the
+                           // tiles of 32 rows or columns read a streamed operand more often than the larger ones
     double split_gain; // factor on `eff` in a launch that cuts K into ranges (the 64x128 FP32 tile: 4-6 % ahead of 128x64 there, behind it everywhere else)
     size_t smem_deep[4];
     void (*plain_deep[4])(const GemmParams<T>);
@@ -62,6 +64,7 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
     TileEntry<T> e;
     e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK;
     e.split_gain = 1.0;
+    e.streamed_gain = 1.0;
     e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri; e.k0 = k0; e.tail_extra = tail_extra;
     e.eff_tri_c = eff_tri_c < 0 ? eff : eff_tri_c;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
@@ -272,7 +275,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
                    split_overhead_cost<T>(M, N, K, s);
         };
         const bool split_model = knobs().split_model != 0 && !need_tri;
-        double best = 0, best_split = 0;
+        double best = 0, best_split = 0, cost_last = 0;
         int pick_of_split = -1;
         bool have = false;
         for (int i = 0; i < ntab; ++i) {
@@ -298,6 +301,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             // tiles 0.77 ms, 128x128 0.60 ms, 64x64 0.67 ms).
             if (tri_operand) rounds = (double)t / (2.0 * kCUs) + 0.4;
             double eff = tri_operand ? tab[i].eff_tri : tri_c ? tab[i].eff_tri_c : tab[i].eff;
+            if (streamed) eff *= tab[i].streamed_gain;
             // (credited up to three rounds of tiles: beyond that the small tile's memory traffic costs more
             // than the deeper panels gain - 2000^3 FP32 128 TFLOP/s with 128x64 tiles, 119 with 64x64)
             if (!need_tri && ts <= 1 && tab[i].bk_deep > 0 && ((K >= 1024 && t <= 3 * kCUs) || (K >= 512 && t <= kCUs))) eff *= tab[i].deep_gain;
@@ -305,6 +309,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             if (t <= kCUs) cost /= tab[i].alone * lone_stream;  // a workgroup alone on its CU cannot keep the MFMA pipes full
             cost *= 1.0 + tab[i].k0 / K;
             if (costs_out) costs_out[i] = cost;
+            if (i == ntab - 1) cost_last = cost;
             if (!have || cost < best) { best = cost; pick = i; have = true; }
             // Small C, deep K: the larger tiles with a K split, ranges of at least 512 and 32 panels.
             if (split_model && tab[i].has_splitk && i != ntab - 1) {
@@ -322,21 +327,26 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
         // is hard on one round of unsplit small tiles over a deep K: DGEMM 1024 x 1024 x 8192 and 2048 x 512 x 8192
         // run 69.1 TFLOP/s on 256 tiles of 64x64 and 66.6 on 128x128 tiles in 8 ranges, which it had 7 % ahead;
         // 896 x 896 x 8192, 60.4 against 53.1 the other way, it has further ahead than that).
+        // Tiles below it in size (listed before it, without K ranges of their own) fill the CUs of a small product
+        // in one launch; against them the last tile is priced with its best number of ranges as well.
         const int last = ntab - 1;
         int last_splits = -1;  // -1: the rule without the model
-        if (split_model && pick == last && tab[last].has_splitk) {
+        const bool below_last = pick != last && tab[pick].bm * tab[pick].bn < tab[last].bm * tab[last].bn;
+        if (split_model && (pick == last || below_last) && tab[last].has_splitk) {
             const int64_t t = active_tiles(M, N, tab[last].bm, tab[last].bn, 0);
             const int s_max = splits_for(t, K, tab[last].bk);
             if (s_max > 1) {
                 static const int kCand[] = {2, 3, 4, 5, 6, 8, 10, 12, 16, 20, 24, 32, 40, 48, 64, 96, 128, 192, 256, 384};
-                last_splits = 1;  // `best` is the cost of one range
+                double c_best = cost_last;  // the cost of one range
+                int s_best = 1;
                 for (int s : kCand) {
                     if (s >= s_max) break;
                     const double c = split_cost(last, t, s);
-                    if (c < best) { best = c; last_splits = s; }
+                    if (c < c_best) { c_best = c; s_best = s; }
                 }
                 const double c = split_cost(last, t, s_max);
-                if (c < best) { best = c; last_splits = s_max; }
+                if (c < c_best) { c_best = c; s_best = s_max; }
+                if (pick == last || c_best < best) { pick = last; best = c_best; last_splits = s_best; }
             }
         }
         if (pick_of_split >= 0) {
@@ -640,7 +650,14 @@ template <typename T> static TileEntry<T> with_split_gain(TileEntry<T> e, double
     return e;
 }
 
-// One parameter of the choice model of tile `i`: 0 eff, 1 alone, 2 k0, 3 tail_extra, 4 deep_gain, 5 split_gain.
+// A table entry with its credit on streamed operands set (see TileEntry::streamed_gain).
+template <typename T> static TileEntry<T> with_streamed_gain(TileEntry<T> e, double g) {
+    e.streamed_gain = g;
+    return e;
+}
+
+// One parameter of the choice model of tile `i`: 0 eff, 1 alone, 2 k0, 3 tail_extra, 4 deep_gain, 5 split_gain,
+// 6 streamed_gain.
 template <typename T> static double *model_param(TileEntry<T> *tab, int ntab, int i, int which) {
     if (i < 0 || i >= ntab) return nullptr;
     switch (which) {
@@ -650,6 +667,7 @@ template <typename T> static double *model_param(TileEntry<T> *tab, int ntab, in
         case 3: return &tab[i].tail_extra;
         case 4: return &tab[i].deep_gain;
         case 5: return &tab[i].split_gain;
+        case 6: return &tab[i].streamed_gain;
         default: return nullptr;
     }
 }

@@ -377,7 +377,8 @@ void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes);
  * clblasAmdTileModelParam reads (set == 0) or sets one parameter of one tile's model - which: 0 the
  * efficiency credited to the tile, 1 the factor for a workgroup alone on its CU, 2 the fixed time per
  * workgroup as a depth, 3 the price of a sliced tail in rounds, 4 the credit of the deep-panel form, 5 the
- * factor on the efficiency in a launch that cuts K into ranges - returning 0, or -1 for no such tile or parameter.  Both exist for clblas_amd/fit_tile_model.py, which
+ * factor on the efficiency in a launch that cuts K into ranges, 6 the factor on the efficiency where the
+ * operands are streamed from HBM - returning 0, or -1 for no such tile or parameter.  Both exist for clblas_amd/fit_tile_model.py, which
  * refits the parameters to measured times; setting parameters while another thread is inside a GEMM call
  * is not supported.  No counterpart in the reference (its selection table is generated at build time,
  * src/library/blas/AutoGemm/KernelSelection.py). */

@@ -17,7 +17,7 @@ from helpers import (COL, ROW, NOTRANS, TRANS, CONJ, LEFT, LOWER, NONUNIT, buf_l
 pytestmark = pytest.mark.gpu
 
 DT = {"f32": np.float32, "f64": np.float64}
-N_TILES = {np.float32: 5, np.float64: 2}
+N_TILES = {np.float32: 5, np.float64: 4}
 
 
 @pytest.fixture(scope="module")
