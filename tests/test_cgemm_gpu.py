@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 CDT = [np.complex64, np.complex128]
 ALL_T = [NOTRANS, TRANS, CONJ]
-N_TILES = 2
+N_TILES = {np.complex64: 2, np.complex128: 4}
 
 
 @pytest.fixture(scope="module")
@@ -60,7 +60,7 @@ def test_gaussian_integer_exact_all_tiles(gpu, dtype, order, tA, tB):
         want = C.copy()
         assert oracle.gemm(order, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, want, offs[2],
                            ldc) == 0
-        for tile in [None] + list(range(N_TILES)):
+        for tile in [None] + list(range(N_TILES[dtype])):
             st, got = gpu.gemm(order, tA, tB, M, N, K, alpha, A, offs[0], lda, B, offs[1], ldb, beta, C, offs[2], ldc,
                                tile=tile)
             assert st == 0
