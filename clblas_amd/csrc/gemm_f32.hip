@@ -38,7 +38,17 @@ namespace cba {
 //   2 % more than its twin in launches that cut K, where it is 4-6 % ahead of it whichever dimension is the short
 //   one (10000 x 100 x 10000, 100 x 10000 x 10000, 200 x 3000 x 6000, 768 x 768 x 16384), while it is behind
 //   it in every launch of whole tiles.
-//   4:  64x64x32,  wave 32x32, split-K capable (small / deep-K problems; 1024^3: 94 against 86 with
+//   4:  64x32x64,  wave 32x16, and
+//   5:  32x32x64,  wave 16x16, both on the 16x16x4 MFMA (workgroups of four wavefronts on tiles below 64x64): for
+//      products of up to a few hundred 64x64 tiles, which they cover with one workgroup or more per CU in a single
+//      launch where the 64x64 tiles leave CUs idle or cut K and pay a second, dependent launch (SGEMM 448^3 11.9 ->
+//      7.1 us, 512^3 10.4 -> 7.1, 704^3 16.0 -> 9.9, 800 x 600 x 400 11.7 -> 7.9, 512 x 1024 x 512 12.6 -> 8.0,
+//      1024^3 21.1-21.9 -> 20.2-20.4 in all four transpose cases, 9000 x 130 x 9000 290 -> 228; from about 1100^3 on
+//      and for deep K the larger tiles are ahead again).  Plain products only (no K ranges, no triangular forms).
+//      Parameters from runs with every tile forced on 23 shapes, fitted through the model query; checked against
+//      the library without them on 63 further shapes (nothing more than 1.1 % slower).  Tiles 32 wide read a
+//      streamed operand more often: credited .88 / .75 there (16384 x 64 x 10000 stays with 128x64 in four ranges).
+//   6:  64x64x32,  wave 32x32, split-K capable (small / deep-K problems; 1024^3: 94 against 86 with
 //      depth 16, 8192 x 64 x 8192: 106-112 against 91-94); with panels of depth 64 where a workgroup's K
 //      range is at least 1024 (1024^3 95.4 -> 99.0 TFLOP/s, 1024 x 1024 x 2048 109 -> 115, 960 x 960 x 2048
 //      96 -> 101, 512 x 512 x 4096 85 -> 90)
@@ -49,6 +59,8 @@ static TileEntry<float> *f32_tiles(int *n) {
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.07),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.9, 0.0, 10.0),
         with_split_gain(make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.9, 0.885, 10.0), 1.02),
+        with_streamed_gain(make_tile_entry<float, 64, 32, 64, 32, 16, 2, false, false>(0.85, 1.0, -1.0, 30.0), 0.88),
+        with_streamed_gain(make_tile_entry<float, 32, 32, 64, 16, 16, 2, false, false>(0.84, 0.6, -1.0, 30.0), 0.75),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64, true>(0.88, 0.85, 0.83, 0.0, 0.02),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

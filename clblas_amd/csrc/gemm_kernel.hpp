@@ -180,6 +180,28 @@ template <> struct Mma<double> {
     }
 };
 
+// FP32 on the 16x16x4 instruction (the operand and result layout of the FP64 one, but for the rows of a
+// result column: four consecutive ones per lane): for wave tiles of 16 rows or columns, i.e. workgroups of
+// four wavefronts on tiles below 64x64.
+struct MmaF32Small {
+    static constexpr int MB = 16;
+    static constexpr int KS = 4;
+    static constexpr int NACC = 4;
+    typedef f32x4 Acc;
+    static __device__ __forceinline__ Acc run(float a, float b, Acc c) {
+        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int row(int v, int lane) {
+        return 4 * (lane >> 4) + v;
+    }
+};
+
+// The instruction for a wave tile of WM x WN elements of real type R.
+template <typename R, int WM, int WN> struct MmaFor { typedef Mma<R> type; };
+template <int WM, int WN> struct MmaFor<float, WM, WN> {
+    typedef typename std::conditional<WM % 32 == 0 && WN % 32 == 0, Mma<float>, MmaF32Small>::type type;
+};
+
 template <typename T> struct GemmParams {
     const T *A;
     const T *B;
@@ -458,7 +480,7 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
 };
 
 template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_KC, bool WIDE = false> struct GemmCfg {
-    typedef Mma<typename Elem<T>::Real> M;
+    typedef typename MmaFor<typename Elem<T>::Real, WM, WN>::type M;
     static constexpr bool CPLX = Elem<T>::CPLX;
     static constexpr int VEC = 16 / (int)sizeof(T);
     static constexpr int MB = M::MB, KS = M::KS, NACC = M::NACC;
@@ -494,7 +516,7 @@ gemm_mfma_kernel(const GemmParams<T> p) {
     static_assert(!(SPLITK && TRI), "triangular variants do not split K");
     typedef GemmCfg<T, BM, BN, BK, WM, WN, A_KC, B_KC, WIDE> Cfg;
     typedef typename Elem<T>::Real R;
-    typedef Mma<R> M;
+    typedef typename Cfg::M M;
     constexpr bool CPLX = Cfg::CPLX;
     constexpr int NP = CPLX ? 2 : 1;  // MFMA accumulator blocks per C block (re, im)
     constexpr int MB = Cfg::MB, KS = Cfg::KS, NACC = Cfg::NACC;

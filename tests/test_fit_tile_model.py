@@ -29,13 +29,13 @@ def synthetic_block(letter):
 @pytest.fixture
 def restore_params():
     saved = {(l, t, p): clblas_amd.tile_model_param(l, t, p)
-             for l, n in (("s", 5), ("d", 4)) for t in range(n) for p in fit_tile_model.GRIDS}
+             for l, n in (("s", 7), ("d", 4)) for t in range(n) for p in fit_tile_model.GRIDS}
     yield
     for (l, t, p), v in saved.items():
         clblas_amd.tile_model_param(l, t, p, v)
 
 
-@pytest.mark.parametrize("letter,ntiles", [("s", 5), ("d", 4)])
+@pytest.mark.parametrize("letter,ntiles", [("s", 7), ("d", 4)])
 def test_model_has_no_regret_on_its_own_costs_and_fit_repairs_a_spoiled_parameter(letter, ntiles, restore_params):
     block = synthetic_block(letter)
     shapes, skipped = fit_tile_model.shapes_of(block)

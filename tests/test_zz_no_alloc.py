@@ -73,7 +73,7 @@ def test_noalloc_rejects_what_does_not_fit_its_scratch():
     A = torch.from_numpy(oracle.uniform(M * K, 1, np.float32)).cuda()
     B = torch.from_numpy(oracle.uniform(K * N, 2, np.float32)).cuda()
     C = torch.full((M * N,), 3.0, device="cuda")
-    with debug_env(CLBLAS_AMD_GEMM_TILE=4, CLBLAS_AMD_GEMM_SPLITS=64):
+    with debug_env(CLBLAS_AMD_GEMM_TILE=6, CLBLAS_AMD_GEMM_SPLITS=64):   # the 64x64 tile, last in the FP32 table
         st = clblas_amd.sgemm_noalloc(COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 0.0, C, 0, M)
         torch.cuda.synchronize()
         assert st == clblas_amd.Status.OutOfResources
