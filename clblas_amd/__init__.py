@@ -252,7 +252,7 @@ TILE_PARAMS = ("eff", "alone", "k0", "tail_extra", "deep_gain", "split_gain", "s
 def tile_model_query(type_letter, M, N, K):
     """The tile choice for a plain product, without launching: dict with the chosen tile's index, its K
     ranges and tail slices, and per tile of the table its dimensions "BMxBNxBK" and the model's cost
-    (None: not offered).  type_letter: "s", "d" or "z"."""
+    (None: not offered).  type_letter: "s", "d", "c" or "z"."""
     n = 16
     tile, splits, tail = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
     costs, dims = (ctypes.c_double * n)(), (ctypes.c_int * (3 * n))()

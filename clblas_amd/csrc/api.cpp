@@ -634,13 +634,14 @@ int clblasAmdTileModelQuery(char type, size_t M, size_t N, size_t K, int *tile, 
     if (M == 0 || N == 0 || K == 0 || M > kMaxDim || N > kMaxDim || K > kMaxDim) return -1;
     if (type == 's') return cba::sgemm_model_query((int)M, (int)N, (int)K, tile, splits, tail_slices, costs, max_tiles, dims);
     if (type == 'd') return cba::dgemm_model_query((int)M, (int)N, (int)K, tile, splits, tail_slices, costs, max_tiles, dims);
+    if (type == 'c') return cba::cgemm_model_query((int)M, (int)N, (int)K, tile, splits, tail_slices, costs, max_tiles, dims);
     if (type == 'z') return cba::zgemm_model_query((int)M, (int)N, (int)K, tile, splits, tail_slices, costs, max_tiles, dims);
     return -1;
 }
 
 int clblasAmdTileModelParam(char type, int tile, int which, double *value, int set) {
     double *p = type == 's' ? cba::sgemm_model_param(tile, which) : type == 'd' ? cba::dgemm_model_param(tile, which)
-                : type == 'z' ? cba::zgemm_model_param(tile, which) : nullptr;
+                : type == 'c' ? cba::cgemm_model_param(tile, which) : type == 'z' ? cba::zgemm_model_param(tile, which) : nullptr;
     if (!p || !value) return -1;
     if (set) *p = *value;
     else *value = *p;

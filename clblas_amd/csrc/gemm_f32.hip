@@ -59,7 +59,7 @@ static TileEntry<float> *f32_tiles(int *n) {
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.07),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.9, 0.0, 10.0),
         with_split_gain(make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.9, 0.885, 10.0), 1.02),
-        with_streamed_gain(make_tile_entry<float, 64, 32, 64, 32, 16, 2, false, false>(0.85, 1.0, -1.0, 30.0), 0.88),
+        with_streamed_gain(make_tile_entry<float, 64, 32, 64, 32, 16, 2, false, false>(0.85, 1.0, -1.0, 10.0), 0.88),
         with_streamed_gain(make_tile_entry<float, 32, 32, 64, 16, 16, 2, false, false>(0.84, 0.6, -1.0, 30.0), 0.75),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64, true>(0.88, 0.85, 0.83, 0.0, 0.02),
     };

@@ -159,6 +159,8 @@ double *sgemm_model_param(int tile, int which);  // nullptr: no such tile / para
 double *dgemm_model_param(int tile, int which);
 int zgemm_model_query(int M, int N, int K, int *tile, int *splits, int *tail_slices, double *costs, int max_costs, int *dims);
 double *zgemm_model_param(int tile, int which);
+int cgemm_model_query(int M, int N, int K, int *tile, int *splits, int *tail_slices, double *costs, int max_costs, int *dims);
+double *cgemm_model_param(int tile, int which);
 
 // Complex variants: conjA / conjB conjugate the elements of op(A) / op(B) (clblasConjTrans).
 hipError_t cgemm_colmajor(bool transA, bool transB, bool conjA, bool conjB, int M, int N, int K, Cx<float> alpha,

@@ -367,7 +367,7 @@ clblasStatus clblasAmdReserveWorkspace(hipStream_t stream, size_t gemm_bytes, si
  * outgrown ones that are parked until the stream is released). */
 void clblasAmdWorkspaceStats(size_t *streams, size_t *bytes);
 
-/* The tile choice of clblasSgemm (type 's') / clblasDgemm ('d') / clblasZgemm ('z') for a plain M x N x K product, as a
+/* The tile choice of clblasSgemm (type 's') / clblasDgemm ('d') / clblasCgemm ('c') / clblasZgemm ('z') for a plain M x N x K product, as a
  * function that launches nothing: the chosen tile (index into the type's tile table), its number of K
  * ranges and tail slices, the cost the choice model puts on every tile in one K range (negative: tile not
  * offered) and the tiles' dimensions (bm, bn, bk per tile, 3 ints each; `costs` and `dims` hold max_tiles

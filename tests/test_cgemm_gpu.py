@@ -18,7 +18,7 @@ pytestmark = pytest.mark.gpu
 
 CDT = [np.complex64, np.complex128]
 ALL_T = [NOTRANS, TRANS, CONJ]
-N_TILES = {np.complex64: 2, np.complex128: 4}
+N_TILES = {np.complex64: 4, np.complex128: 4}
 
 
 @pytest.fixture(scope="module")

@@ -416,7 +416,7 @@ def test_small_c_deep_k_integer_exact(gpu, dtype):
     default tile choice and every tile forced; odd offsets and leading dimensions."""
     cplx = np.dtype(dtype).kind == "c"
     alpha, beta = ((2 - 1j), (-1 + 2j)) if cplx else (3.0, -2.0)
-    n_tiles = {np.float32: 7, np.float64: 4, np.complex64: 2, np.complex128: 4}[dtype]
+    n_tiles = {np.float32: 7, np.float64: 4, np.complex64: 4, np.complex128: 4}[dtype]
     for (M, N, K), (tA, tB) in (((640, 520, 6000), (NOTRANS, NOTRANS)), ((300, 900, 5000), (TRANS, CONJ))):
         lda, ldb, ldc, na, nb, nc = _layout(COL, tA, tB, M, N, K, 1, (3, 5, 7))
         lim = 8 if cplx else exact_int_limits(K, alpha, beta, dtype)[0]

@@ -17,7 +17,7 @@ from l3_util import (ALL, REAL, CPLX, abs1, bound, err, is_cplx, matrix, nan_of,
                      scalars, sym_dense, tri_dense, tri_mask)
 
 pytestmark = pytest.mark.gpu
-N_TILES = {np.dtype(np.float32): 7, np.dtype(np.float64): 4, np.dtype(np.complex64): 2, np.dtype(np.complex128): 4}
+N_TILES = {np.dtype(np.float32): 7, np.dtype(np.float64): 4, np.dtype(np.complex64): 4, np.dtype(np.complex128): 4}
 WIDE = lambda dt: np.complex128 if is_cplx(dt) else np.float64
 
 

@@ -19,7 +19,7 @@ from test_oracle_rank2k_hermitian import (DT, GOLDEN, call_rank2k, hemm_case, ra
                                           rank2k_variants, run_golden)
 
 pytestmark = pytest.mark.gpu
-N_TILES = {np.dtype(np.float32): 7, np.dtype(np.float64): 4, np.dtype(np.complex64): 2, np.dtype(np.complex128): 4}
+N_TILES = {np.dtype(np.float32): 7, np.dtype(np.float64): 4, np.dtype(np.complex64): 4, np.dtype(np.complex128): 4}
 WIDE = lambda dt: np.complex128 if is_cplx(dt) else np.float64
 
 
