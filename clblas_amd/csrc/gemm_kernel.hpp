@@ -329,7 +329,8 @@ struct PanelSrc {
 // offsets inside a row stay below the row's length in the panel (at most 1 KiB).  One load
 // instruction per row instead of one per 64 lanes: slower, and only instantiated for the smallest
 // tile of each type, but there is no leading dimension it cannot serve.
-template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1, bool WIDE = false> struct PanelLoader {
+// GRP: lanes that read one k row together in a fragment read (the block edge of the MFMA: 32, or 16).
+template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1, bool WIDE = false, int GRP = 32> struct PanelLoader {
     static constexpr int VEC = 16 / (int)sizeof(T);
     static constexpr int NVEC = BX * BK / VEC;
     static constexpr int PER = NVEC / NT;  // 16-byte vectors per thread = wave-wide loads per wave
@@ -346,14 +347,33 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
     // all groups start in the same bank (measured: any stagger costs half of the LDS cycles),
     // which the unpadded image gives (rows are multiples of 256 bytes apart).
     static constexpr bool FP64_GROUPS = sizeof(typename Elem<T>::Real) == 8;
+    // FP32 and complex FP32 on the 16x16x4 MFMA: four groups of 16 lanes read four rows VEC apart.  Measured
+    // (SQ_LDS_BANK_CONFLICT over SQ_LDS_IDX_ACTIVE, 19-50 % with the layout of the 32-lane groups, 0 % with this):
+    // with 16 bytes per lane a group fills a pass by itself and, as for FP64, all groups start in the same bank (no
+    // gap); with 8 or 4 bytes per lane two groups are read together and have to lie next to each other, one group's
+    // bytes (16 lanes) apart.  Rows VEC apart in different chunks: the gap after a chunk does it.  Rows VEC apart in
+    // the same chunk (panels 32 wide, a row being two groups long): every other set of VEC rows is stored with its
+    // two halves exchanged - the loads name their source freely.
+    static constexpr bool SMALL_GROUPS = GRP == 16 && !FP64_GROUPS && MODE == LM_DMA_X;
+    static constexpr int LANE_BYTES = IL * (int)sizeof(T);
+    static constexpr int GROUP_ELEMS = 16 * IL;
+    static constexpr bool NEED_STAGGER = SMALL_GROUPS && LANE_BYTES < 16;
+    static constexpr bool FLIP_HALVES = NEED_STAGGER && ROWS_PER_CHUNK > VEC;
+    static_assert(!FLIP_HALVES || (BX == 2 * GROUP_ELEMS && !WIDE), "exchanged halves: a row is two groups long");
     static constexpr int CHUNK_PAD =
-        (MODE == LM_DMA_X && !FP64_GROUPS) ? (64 / (int)sizeof(T)) / CHUNKS_APART : 0;  // elements
+        MODE != LM_DMA_X || FP64_GROUPS ? 0
+        : SMALL_GROUPS ? ((NEED_STAGGER && !FLIP_HALVES) ? GROUP_ELEMS / CHUNKS_APART : 0)
+                       : (64 / (int)sizeof(T)) / CHUNKS_APART;  // elements
     static constexpr int CHUNK_PITCH = CHUNK + CHUNK_PAD;
     static constexpr int LDS_PITCH = MODE == LM_DMA_X ? BX : BK;
     static constexpr int LDS_ELEMS = (NVEC / 64) * CHUNK_PITCH;
+    // LM_DMA_X: column of the image that holds column x of k row k (and the other way round).
+    static __device__ __forceinline__ int image_col(int k, int x) {
+        return FLIP_HALVES ? x ^ (((k / VEC) & 1) * GROUP_ELEMS) : x;
+    }
     // LM_DMA_X: LDS element offset of image element (k, x).
     static __device__ __forceinline__ int lds_at(int k, int x) {
-        const int e = k * BX + x;
+        const int e = k * BX + image_col(k, x);
         return e + (e / CHUNK) * CHUNK_PAD;
     }
     // LM_DMA_K swizzle: S slots per row; rows x and x + 16/S start in the same bank.
@@ -384,7 +404,7 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
         for (int i = 0; i < PER; ++i) {
             if (MODE == LM_DMA_X) {
                 const int e = (wave + i * NW) * CHUNK + lane * VEC;  // element index in the [k][x] image
-                const int k = e / BX, x = e % BX;
+                const int k = e / BX, x = image_col(k, e % BX);
                 if (WIDE) {
                     voff[i] = (uint32_t)(x * (int)sizeof(T));
                     my_row = k - ((wave + i * NW) * CHUNK) / BX;  // the same for every i
@@ -449,7 +469,7 @@ template <typename T, int BX, int BK, int NT, int MODE, int IL = 1, int MBLK = 1
         for (int i = 0; i < PER; ++i) {
             if (MODE == LM_DMA_X) {
                 const int e0 = (wave + i * NW) * CHUNK + lane * VEC;
-                const int k = e0 / BX, x = e0 % BX;
+                const int k = e0 / BX, x = image_col(k, e0 % BX);
                 T *q = lds + (wave + i * NW) * CHUNK_PITCH + lane * VEC;
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) fix(q[e], x0 + x + e, k0 + k);
@@ -498,8 +518,8 @@ template <typename T, int BM, int BN, int BK, int WM, int WN, bool A_KC, bool B_
     static constexpr int VNM = B_KLAY ? 1 : VN;  // n interleave used by the fragment/epilogue mapping
     static constexpr int NG = KS;                // lane groups along k
     static_assert(BK % (VEC * NG) == 0, "panel depth must hold whole k groups");
-    typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_DMA_K : LM_DMA_X, VM, MB, WIDE> LoaderA;
-    typedef PanelLoader<T, BN, BK, NT, B_KC ? LM_DMA_K : LM_DMA_X, 1, 1, WIDE> LoaderB;
+    typedef PanelLoader<T, BM, BK, NT, A_KC ? LM_DMA_K : LM_DMA_X, VM, MB, WIDE, MB> LoaderA;
+    typedef PanelLoader<T, BN, BK, NT, B_KC ? LM_DMA_K : LM_DMA_X, 1, 1, WIDE, MB> LoaderB;
     static constexpr int PITCH_A = LoaderA::LDS_PITCH, PITCH_B = LoaderB::LDS_PITCH;
     static constexpr int A_ELEMS = LoaderA::LDS_ELEMS;
     static constexpr int STAGE = LoaderA::LDS_ELEMS + LoaderB::LDS_ELEMS;  // elements per LDS stage
