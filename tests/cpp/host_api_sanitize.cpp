@@ -40,6 +40,10 @@ int sgemm_model_query(int, int, int, int *, int *, int *, double *, int, int *) 
 int dgemm_model_query(int, int, int, int *, int *, int *, double *, int, int *) { return 0; }
 double *sgemm_model_param(int, int) { return nullptr; }
 double *dgemm_model_param(int, int) { return nullptr; }
+int cgemm_model_query(int, int, int, int *, int *, int *, double *, int, int *) { return 0; }
+int zgemm_model_query(int, int, int, int *, int *, int *, double *, int, int *) { return 0; }
+double *cgemm_model_param(int, int) { return nullptr; }
+double *zgemm_model_param(int, int) { return nullptr; }
 
 #define INST(T)                                                                                                         \
     template hipError_t launch_gemm<T>(bool, bool, bool, bool, int, int, int, T, const T *, int64_t, const T *, int64_t, T, \
