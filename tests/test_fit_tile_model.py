@@ -69,3 +69,26 @@ def test_main_prints_a_report(tmp_path, capsys, restore_params):
     out = capsys.readouterr().out
     assert "== sgemm: %d shapes" % len(SHAPES) in out and "== dgemm" in out
     assert "regret 0.0000 -> 0.0000" in out
+
+
+@pytest.mark.parametrize("letter", ["s", "d", "c", "z"])
+def test_small_products_take_the_small_tiles_and_deep_or_large_ones_do_not(letter):
+    """The choice model is a host function: a product of a few hundred 64x64 tiles goes to a 64x32 / 32x32 tile
+    in one K range, the same C over a deep K to the K-split 64x64 tile, a large product to a large tile; and the
+    last entry of every table is the 64x64 tile that takes the K ranges."""
+    q = clblas_amd.tile_model_query(letter, 512, 512, 512)
+    tiles = q["tiles"]
+    assert tiles[-1].startswith("64x64x") and len(tiles) >= 4
+    small = [i for i, t in enumerate(tiles) if t.startswith("64x32x") or t.startswith("32x32x")]
+    assert len(small) == 2 and max(small) < len(tiles) - 1
+    assert q["tile"] in small and q["splits"] == 1
+    for sh in ((448, 448, 448), (800, 600, 400), (512, 1024, 512)):
+        q = clblas_amd.tile_model_query(letter, *sh)
+        assert q["tile"] in small and q["splits"] == 1, (sh, q)
+    q = clblas_amd.tile_model_query(letter, 256, 256, 8192)       # deep K: ranges of the 64x64 tile (or a larger one)
+    assert q["tile"] not in small and q["splits"] > 1, q
+    q = clblas_amd.tile_model_query(letter, 8192, 8192, 8192)
+    assert q["tile"] not in small and q["splits"] == 1, q
+    # 32-wide tiles are not taken where one operand is streamed from HBM and only a few columns wide
+    q = clblas_amd.tile_model_query(letter, 16384, 64, 10000)
+    assert not tiles[q["tile"]].startswith("32x32x"), q
