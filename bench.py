@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the xGEMM / xTRSM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|trsm|host|tilemodel|vendor|tiles|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only sgemm|dgemm|dtrsm|cgemm|zgemm|level3|configs|deepk|small|big|trsm|host|tilemodel|vendor|tiles|copy]
 
 A "step" is one call of the hot path on the headline workload (BASELINE config 2: SGEMM,
 column-major NN, M=N=K=8192, tight leading dimensions, alpha=1, beta=1, inputs resident in
@@ -402,7 +402,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K (8192 is the BASELINE configuration)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, big, trsm, vendor, tiles or copy "
+    ap.add_argument("--only", default="", help="run only sgemm, dgemm, dtrsm, cgemm, zgemm, level3, configs, deepk, small, big, trsm, vendor, tiles or copy "
                     "(profiling; copy = a plain 1 GiB device copy used to scale the HBM traffic counters; tiles = every tile "
                     "the five configurations use, --steps times each, for the counter profile)")
     args = ap.parse_args()
@@ -735,6 +735,32 @@ def main():
                         "torch_mm_tflops": vendor_tf}
                     del A, B, C
             extra["small_c_deep_k"] = dk
+
+        # ---- Small products: a few hundred 64x64 tiles at most, which the 64x32 / 32x32 tiles cover in one launch
+        #      (column-major NN, alpha = 1, beta = 0; timed through `bind`: a call takes some 10 us); the vendor BLAS
+        #      behind torch.mm on the same product beside it. ----
+        if args.only in ("", "small"):
+            sp = {}
+            for name, sym, dt, flop in (("sgemm", "clblasSgemm", torch.float32, 2.0), ("dgemm", "clblasDgemm", torch.float64, 2.0),
+                                        ("cgemm", "clblasCgemm", torch.complex64, 8.0), ("zgemm", "clblasZgemm", torch.complex128, 8.0)):
+                for (M, N, K) in ((512, 512, 512), (704, 704, 704), (512, 1024, 512), (1024, 1024, 1024)):
+                    real = torch.float32 if dt in (torch.float32, torch.complex64) else torch.float64
+                    mk = lambda r, c: (torch.rand(r, c, device="cuda", dtype=real, generator=gen) * 2 - 1).to(dt)
+                    A, B = mk(K, M), mk(N, K)      # column-major M x K and K x N
+                    C = torch.zeros(N, M, device="cuda", dtype=dt)
+                    bound = clblas_amd.bind(sym, COL, NOTRANS, NOTRANS, M, N, K, 1.0, A, 0, M, B, 0, K, 0.0, C, 0, M)
+
+                    def call():
+                        if bound() != 0:
+                            raise RuntimeError("%s failed" % sym)
+                    ms = timed_batch(torch, call, 100, 5)
+                    kernel = clblas_amd.last_dispatch()[0]
+                    vendor_tf, vendor_ms = vendor_rate(torch, lambda: torch.mm(B, A, out=C), 100, 5, flop * M * N * K)
+                    sp["%s %dx%dx%d" % (name, M, N, K)] = {
+                        "us": round(ms * 1e3, 2), "tflops": round(flop * M * N * K / ms / 1e9, 2),
+                        "torch_mm_us": None if vendor_ms is None else round(vendor_ms * 1e3, 2), "kernel": kernel}
+                    del A, B, C
+            extra["small_products"] = sp
 
         # ---- Beyond 8192: the part has 288 GB, and matrices of 16384 .. 32768 are ordinary there (1 .. 8.6 GB each).
         #      Column-major NN / left-lower-notrans-nonunit, alpha = beta = 1, tight leading dimensions. ----
