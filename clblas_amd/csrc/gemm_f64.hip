@@ -28,8 +28,8 @@ namespace cba {
 static TileEntry<double> *f64_tiles(int *n) {
     static TileEntry<double> tab[] = {
         make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 85.0),
-        with_streamed_gain(make_tile_entry<double, 64, 32, 32, 32, 16, 2, false, false>(0.75, 1.0, -1.0, 100.0), 0.95),
-        with_streamed_gain(make_tile_entry<double, 32, 32, 32, 16, 16, 2, false, false>(0.80, 0.6, -1.0, 200.0), 0.75),
+        with_streamed_gain(make_tile_entry<double, 64, 32, 32, 32, 16, 2, false, false>(0.77, 1.0, -1.0, 100.0), 0.95),
+        with_streamed_gain(make_tile_entry<double, 32, 32, 32, 16, 16, 2, false, false>(0.80, 0.62, -1.0, 200.0), 0.75),
         // (in launches that cut K it is credited 4 % less: DGEMM 100 x 5000 x 20000 ran 5.6 % behind the 128x128
         // tile in twelve ranges with it)
         with_split_gain(make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32, true>(0.90, 0.85, 0.84, 68.0, 0.35), 0.96),
