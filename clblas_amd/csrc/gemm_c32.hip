@@ -11,14 +11,14 @@ namespace cba {
 //   1:  64x32x32, wave 32x16, and
 //   2:  32x32x32, wave 16x16, both on the 16x16x4 MFMA: for small products, which they cover in one launch where
 //      the 64x64 tiles leave CUs idle or cut K and pay a second, dependent launch (CGEMM 512^3 20.4 -> 14.4 us,
-//      1024^3 79 -> 68, 512 x 1024 x 512 30.4 -> 21.7, 896^3 69.5 -> 59.7); plain products only.
+//      1024^3 79 -> 68, 512 x 1024 x 512 30.4 -> 21.7, 896^3 69.5 -> 59.7); no K ranges; triangular forms without sliced tails.
 //   3:  64x64x8,  wave 32x32, split-K capable (credited with .90; .84 where an operand is triangular:
 //      3328^3 127 -> 135 TFLOP/s, 3000 x 1500 x 1000 120 -> 126, CSYRK 6144 130 -> 139 against .84 for all)
 static TileEntry<Cx<float>> *c32_tiles(int *n) {
     static TileEntry<Cx<float>> tab[] = {
         make_tile_entry<Cx<float>, 128, 128, 16, 64, 64, 2, true, true>(0.93),
-        with_streamed_gain(make_tile_entry<Cx<float>, 64, 32, 32, 32, 16, 2, false, false>(0.88, 1.0, -1.0, 10.0), 0.9),
-        with_streamed_gain(make_tile_entry<Cx<float>, 32, 32, 32, 16, 16, 2, false, false>(0.86, 0.7, -1.0, 10.0), 0.75),
+        with_streamed_gain(make_tile_entry<Cx<float>, 64, 32, 32, 32, 16, 2, false, true>(0.88, 1.0, -1.0, 10.0), 0.9),
+        with_streamed_gain(make_tile_entry<Cx<float>, 32, 32, 32, 16, 16, 2, false, true>(0.86, 0.7, -1.0, 10.0), 0.75),
         make_tile_entry<Cx<float>, 64, 64, 8, 32, 32, 2, true, true, 0, true>(0.90, 0.85, 0.84),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

@@ -9,7 +9,7 @@ namespace cba {
 //   1:  64x32x16, wave 32x16, and
 //   2:  32x32x16, wave 16x16: for small products, which they cover in one launch where the 64x64 tiles leave CUs
 //      idle or cut K and pay a second, dependent launch (ZGEMM 512^3 28.2 -> 23.6 us, 800 x 600 x 400 45.6 -> 31.7,
-//      640 x 640 x 128 21.7 -> 12.9, 1024^3 141 -> 131, 9000 x 130 x 9000 2.14 -> 1.63 ms); plain products only.
+//      640 x 640 x 128 21.7 -> 12.9, 1024^3 141 -> 131, 9000 x 130 x 9000 2.14 -> 1.63 ms); no K ranges; triangular forms without sliced tails.
 //   3:  64x64x8, wave 32x32, split-K capable
 //   On large C the 64x64 tiles are the faster ones at every depth (8192^3: 73.2 against 72.0 TFLOP/s, 8192 x 8192 x
 //   2048 72.8 / 71.4, x 512 71.6 / 69.4, x 64 53.3 / 48.8, 4096 x 4096 x 32 38.5 / 32.4), so they are credited with
@@ -24,8 +24,8 @@ namespace cba {
 static TileEntry<Cx<double>> *c64_tiles(int *n) {
     static TileEntry<Cx<double>> tab[] = {
         make_tile_entry<Cx<double>, 128, 64, 8, 64, 32, 2, true, true>(0.93, 0.85, 0.84, 44.0, 0.05, 0.86),
-        with_streamed_gain(make_tile_entry<Cx<double>, 64, 32, 16, 32, 16, 2, false, false>(0.86, 0.8, -1.0, 30.0), 0.95),
-        with_streamed_gain(make_tile_entry<Cx<double>, 32, 32, 16, 16, 16, 2, false, false>(0.82, 0.9, -1.0, 30.0), 0.75),
+        with_streamed_gain(make_tile_entry<Cx<double>, 64, 32, 16, 32, 16, 2, false, true>(0.86, 0.8, -1.0, 30.0), 0.95),
+        with_streamed_gain(make_tile_entry<Cx<double>, 32, 32, 16, 16, 16, 2, false, true>(0.82, 0.9, -1.0, 30.0), 0.75),
         make_tile_entry<Cx<double>, 64, 64, 8, 32, 32, 2, true, true, 0, true>(0.945, 0.85, 0.86, 35.0, 0.35, 0.86),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

@@ -44,7 +44,9 @@ namespace cba {
 //      launch where the 64x64 tiles leave CUs idle or cut K and pay a second, dependent launch (SGEMM 448^3 11.9 ->
 //      7.1 us, 512^3 10.4 -> 7.1, 704^3 16.0 -> 9.9, 800 x 600 x 400 11.7 -> 7.9, 512 x 1024 x 512 12.6 -> 8.0,
 //      1024^3 21.1-21.9 -> 20.2-20.4 in all four transpose cases, 9000 x 130 x 9000 290 -> 228; from about 1100^3 on
-//      and for deep K the larger tiles are ahead again).  Plain products only (no K ranges, no triangular forms).
+//      and for deep K the larger tiles are ahead again).  No K ranges; with the triangular
+//      forms (SSYRK 512 17 -> 10 us, STRMM 1024 33 -> 25), whose last round is never sliced, credited .74 / .72
+//      where an operand is triangular (with the plain credits STRMM / SSYMM 3000 took them and ran 17-20 % slower).
 //      Parameters from runs with every tile forced on 23 shapes, fitted through the model query; checked against
 //      the library without them on 63 further shapes (nothing more than 1.1 % slower).  Tiles 32 wide read a
 //      streamed operand more often: credited .88 / .75 there (16384 x 64 x 10000 stays with 128x64 in four ranges).
@@ -59,8 +61,8 @@ static TileEntry<float> *f32_tiles(int *n) {
         make_tile_entry<float, 128, 128, 16, 64, 64, 2, true, true>(0.920, 0.85, -1.0, 0.0, 0.07),
         make_tile_entry<float, 128, 64, 32, 64, 32, 2, true, true>(0.92, 0.9, 0.0, 10.0),
         with_split_gain(make_tile_entry<float, 64, 128, 32, 32, 64, 2, true, true>(0.92, 0.9, 0.885, 10.0), 1.02),
-        with_streamed_gain(make_tile_entry<float, 64, 32, 64, 32, 16, 2, false, false>(0.85, 1.0, -1.0, 10.0), 0.88),
-        with_streamed_gain(make_tile_entry<float, 32, 32, 64, 16, 16, 2, false, false>(0.84, 0.6, -1.0, 30.0), 0.75),
+        with_streamed_gain(make_tile_entry<float, 64, 32, 64, 32, 16, 2, false, true>(0.85, 1.0, 0.74, 10.0), 0.88),
+        with_streamed_gain(make_tile_entry<float, 32, 32, 64, 16, 16, 2, false, true>(0.84, 0.6, 0.72, 30.0), 0.75),
         make_tile_entry<float, 64, 64, 32, 32, 32, 2, true, true, 64, true>(0.88, 0.85, 0.83, 0.0, 0.02),
     };
     *n = (int)(sizeof(tab) / sizeof(tab[0]));

@@ -11,7 +11,8 @@ namespace cba {
 //      workgroup or more per CU in a single launch, where the 64x64 tiles leave CUs idle or cut K and pay a second,
 //      dependent launch (DGEMM 512^3 14.7 -> 8.6 us, the vendor library 11.6; 448^3 13.4 -> 7.8, 704^3 21.1 -> 15.6,
 //      800 x 600 x 400 17.2 -> 11.0, 512 x 1024 x 512 - an update of DTRSM 1024 - 19.2 -> 12.1; from 900^3 on and
-//      for deep K the 64x64 tiles are ahead again).  Plain products only (no K ranges, no triangular forms).  A
+//      for deep K the 64x64 tiles are ahead again).  No K ranges; with
+//      the triangular forms (DSYRK 512 25 -> 12 us, DTRMM 1024 52 -> 37), whose last round is never sliced.  A
 //      workgroup of 32x32 alone on its CU runs at 0.44 of the CU's peak, two at 0.61, three or more at 0.7; one of
 //      64x32 at 0.79 alone, 0.83-0.85 in company, with about 3 us before its first MFMA: eff / alone / k0 below.
 //   3:  64x64x16,  wave 32x32, split-K capable.  Credited with .90 for plain and triangular-C
@@ -28,8 +29,8 @@ namespace cba {
 static TileEntry<double> *f64_tiles(int *n) {
     static TileEntry<double> tab[] = {
         make_tile_entry<double, 128, 128, 16, 64, 64, 2, true, true>(0.94, 0.85, -1.0, 85.0),
-        with_streamed_gain(make_tile_entry<double, 64, 32, 32, 32, 16, 2, false, false>(0.77, 1.0, -1.0, 100.0), 0.95),
-        with_streamed_gain(make_tile_entry<double, 32, 32, 32, 16, 16, 2, false, false>(0.80, 0.62, -1.0, 200.0), 0.75),
+        with_streamed_gain(make_tile_entry<double, 64, 32, 32, 32, 16, 2, false, true>(0.77, 1.0, -1.0, 100.0), 0.95),
+        with_streamed_gain(make_tile_entry<double, 32, 32, 32, 16, 16, 2, false, true>(0.80, 0.62, -1.0, 200.0), 0.75),
         // (in launches that cut K it is credited 4 % less: DGEMM 100 x 5000 x 20000 ran 5.6 % behind the 128x128
         // tile in twelve ranges with it)
         with_split_gain(make_tile_entry<double, 64, 64, 16, 32, 32, 2, true, true, 32, true>(0.90, 0.85, 0.84, 68.0, 0.35), 0.96),

@@ -24,6 +24,7 @@ template <typename T> struct TileEntry {
     double deep_gain;  // factor on `eff` where the deep form runs (plain products, K range from 1024)
     double streamed_gain;  // factor on `eff` where the operands are streamed from HBM (beyond the memory-side cache): the
                            // tiles of 32 rows or columns read a streamed operand more often than the larger ones
+    bool slices_tail;  // a last, partly filled round of tiles may be cut into K slices (tiles with triangular forms only)
     double split_gain; // factor on `eff` in a launch that cuts K into ranges (the 64x128 FP32 tile: 4-6 % ahead of 128x64 there, behind it everywhere else)
     size_t smem_deep[4];
     void (*plain_deep[4])(const GemmParams<T>);
@@ -65,6 +66,7 @@ TileEntry<T> make_tile_entry(double eff, double alone = 0.85, double eff_tri = -
     e.bm = BM; e.bn = BN; e.bk = BK; e.threads = Cfg::NT; e.has_splitk = WITH_SPLITK;
     e.split_gain = 1.0;
     e.streamed_gain = 1.0;
+    e.slices_tail = WITH_TRI;
     e.eff = eff; e.alone = alone; e.eff_tri = eff_tri < 0 ? eff : eff_tri; e.k0 = k0; e.tail_extra = tail_extra;
     e.eff_tri_c = eff_tri_c < 0 ? eff : eff_tri_c;
     // LDS need depends on the layout of the B panel (transB): index as plain[].
@@ -283,7 +285,7 @@ static void choose_tile(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
             if (tri_operand && tab[i].eff_tri <= 0) continue;
             const int64_t t = active_tiles(M, N, tab[i].bm, tab[i].bn, tri_c);
             double rounds = (double)ceil_div64(t, kCUs);
-            const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0]);
+            const int ts = tail_slices_for(t, K, tab[i].bk, tail_ok && tab[i].tri[0] && tab[i].slices_tail);
             // A sliced tail round lasts 1 / ts of a round plus what does not shrink with the depth of a slice
             // (its first loads, the partial tiles written and added up by a second pass): about 120 deep.
             if (ts > 1) {
@@ -456,7 +458,7 @@ static hipError_t run_gemm_whole(const TileEntry<T> *tab, int ntab, bool tA, boo
         }
     }
     int64_t grid_x = ntiles;
-    if (splits <= 1 && e.tri[idx]) {
+    if (splits <= 1 && e.tri[idx] && e.slices_tail) {
         const int ts = tail_slices_for(ntiles, K, e.bk, tail_ok);
         if (ts > 1) {
             const int64_t kps = ceil_div64(ceil_div64(K, ts), e.bk) * e.bk;
@@ -641,7 +643,7 @@ static void model_query(const TileEntry<T> *tab, int ntab, int M, int N, int K, 
     for (int i = 0; i < max_costs && i < ntab && i < 16; ++i) costs[i] = c[i];
     const TileEntry<T> &e = tab[*tile];
     const int64_t ntiles = ceil_div64(M, e.bm) * ceil_div64(N, e.bn);
-    *tail_slices = (*splits <= 1 && e.tri[0]) ? tail_slices_for(ntiles, K, e.bk, knobs().tail != 0) : 1;
+    *tail_slices = (*splits <= 1 && e.tri[0] && e.slices_tail) ? tail_slices_for(ntiles, K, e.bk, knobs().tail != 0) : 1;
 }
 
 // A table entry with its credit in launches that cut K set (see TileEntry::split_gain).
@@ -650,9 +652,11 @@ template <typename T> static TileEntry<T> with_split_gain(TileEntry<T> e, double
     return e;
 }
 
-// A table entry with its credit on streamed operands set (see TileEntry::streamed_gain).
+// A table entry with its credit on streamed operands set (see TileEntry::streamed_gain), as the tiles below
+// 64x64 are entered: their last round is never cut into K slices (they are for products of few tiles).
 template <typename T> static TileEntry<T> with_streamed_gain(TileEntry<T> e, double g) {
     e.streamed_gain = g;
+    e.slices_tail = false;
     return e;
 }
 
