@@ -5,10 +5,11 @@
     python -m clblas_amd.fit_tile_model tilemodel.json                 (anywhere: needs no GPU)
 
 The launcher (clblas_amd/csrc/gemm_launch.hpp, choose_tile) prices every tile of a type's table for a
-product and takes the cheapest; each tile carries four fitted numbers: `eff` (share of the MFMA peak it
+product and takes the cheapest; each tile carries these fitted numbers: `eff` (share of the MFMA peak it
 is credited with), `alone` (factor when a workgroup has its CU to itself), `k0` (fixed time per
-workgroup, as a depth), `tail_extra` (price of a sliced last round, in rounds) and `split_gain` (factor on
-`eff` in a launch that cuts K into ranges).  This script takes the
+workgroup, as a depth), `tail_extra` (price of a sliced last round, in rounds), `split_gain` (factor on
+`eff` in a launch that cuts K into ranges) and `streamed_gain` (factor on `eff` where the operands are too
+large for the memory-side cache and come from HBM).  This script takes the
 times of every forced tile on every shape from bench.py, evaluates the library's own model through
 clblasAmdTileModelQuery with trial parameters set through clblasAmdTileModelParam - the model is not
 restated here - and searches, one step of one parameter at a time over a grid around its present value
@@ -33,8 +34,10 @@ GRIDS = {"k0": [-40, -20, -10, 10, 20, 40, 80],
          "tail_extra": [-0.1, -0.05, -0.02, 0.02, 0.05, 0.1, 0.2],
          "alone": [-0.1, -0.05, -0.03, 0.03, 0.05, 0.1],
          "eff": [-0.04, -0.03, -0.02, -0.01, 0.01, 0.02, 0.03, 0.04],
-         "split_gain": [-0.06, -0.04, -0.02, 0.02, 0.04, 0.06]}
-LIMITS = {"eff": (0.6, 1.0), "alone": (0.5, 1.0), "k0": (0.0, 300.0), "tail_extra": (0.0, 1.0), "split_gain": (0.8, 1.2)}
+         "split_gain": [-0.06, -0.04, -0.02, 0.02, 0.04, 0.06],
+         "streamed_gain": [-0.1, -0.05, -0.02, 0.02, 0.05, 0.1]}
+LIMITS = {"eff": (0.6, 1.0), "alone": (0.5, 1.0), "k0": (0.0, 300.0), "tail_extra": (0.0, 1.0), "split_gain": (0.8, 1.2),
+          "streamed_gain": (0.5, 1.0)}
 
 
 def shapes_of(block):
